@@ -1,0 +1,186 @@
+/*
+ * megray_vrank.h -- C ABI of the MI355X virtual-rank MegRay library (libmegray_vrank.so).
+ *
+ * The library's C++ face is MegRay's own API (megray.h: get_communicator, Communicator,
+ * HipContext).  This header is the flat, language-neutral face of the same code: plain pointers,
+ * sizes and integers, no C++ or torch types.  It is what a foreign-function binding (ctypes, cgo,
+ * JNI ...) or a single-threaded benchmark driver calls.
+ *
+ * Conventions
+ *   - dtype / op / status integers carry the numeric values of MegRay::DType, MegRay::ReduceOp and
+ *     MegRay::Status (include/megray/common.h:23-37,106-127 of the reference).
+ *   - every buffer pointer is device memory of the current HIP device; `stream` is a hipStream_t
+ *     passed as void* (NULL = the default stream).  Calls enqueue work and return; results are
+ *     ready when the stream reaches that point.
+ *   - "rank" arrays have `nranks` entries, entry r belonging to virtual rank r.  Lengths are
+ *     element counts with the meaning of the reference's Communicator comments
+ *     (include/megray/communicator.h:63-101).
+ *   - where the reference throws MegRay::Exception (unknown dtype / op, wrong context ...) these
+ *     functions return MEGRAY_INVALID_ARGUMENT (6) and keep the message for mrv_last_error().
+ */
+#ifndef MEGRAY_VRANK_H
+#define MEGRAY_VRANK_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MRV_API __attribute__((visibility("default")))
+
+#define MRV_MAX_RANKS 16
+
+/* Which reference loop fixes the order a chunk's contributions are combined in. */
+enum {
+    MRV_ORDER_UCX = 0,   /* src/ucx/all_reduce.cpp:61-82, src/ucx/reduce_scatter.cpp:44-53 */
+    MRV_ORDER_SHM = 1,   /* src/shm/all_reduce.cpp:38-127 + src/shm/communicator.cpp:24-75 */
+    MRV_ORDER_RANK0 = 2  /* ranks 0..N-1 for every element, test/test_opr.cpp:321-330 */
+};
+
+/* How the collective is laid out in kernel launches. */
+enum {
+    MRV_SCHED_FUSED = 0,     /* one launch: N reads, all destinations written */
+    MRV_SCHED_TWO_PHASE = 1, /* reduce-scatter launch + broadcast-copy launch */
+    MRV_SCHED_RING = 2       /* the reference's 2(N-1) two-input ring steps, one launch each */
+};
+
+/* Collective selector of mrv_describe(). */
+enum {
+    MRV_ALL_REDUCE = 0,
+    MRV_REDUCE_SCATTER = 1,
+    MRV_ALL_GATHER = 2,
+    MRV_ALL_TO_ALL = 3,
+    MRV_SCATTER = 4,
+    MRV_GATHER = 5,
+    MRV_BROADCAST = 6,
+    MRV_REDUCE2 = 7
+};
+
+/* ---- library ------------------------------------------------------------------------------ */
+
+/* Bumped when a signature below changes. */
+MRV_API int mrv_abi_version(void);
+
+/* Message of the last call on this thread that returned a non-zero status ("" if none). */
+MRV_API const char* mrv_last_error(void);
+
+/* MegRay::get_dtype_size (src/core/common.cpp:19-38); 0 where the reference throws "unknown dtype". */
+MRV_API size_t mrv_dtype_size(int dtype);
+
+/* ---- the hot path on the current device ---------------------------------------------------- */
+
+/*
+ * o[i] = i0[i] OP i1[i], MAX/MIN keeping i1 on equal / unordered operands.
+ * Replaces MegRay::reduce(i0, i1, o, len, dtype, op, stream) (src/ucx/utils.h:21-22,
+ * src/ucx/kernel.cu:60-98) and MegRay::cpu_reduce (src/shm/utils.h:32).  FLOAT16 is accepted
+ * (fp32 arithmetic, one rounding); CHAR is rejected like the reference ("unknown dtype").
+ */
+MRV_API int mrv_reduce(const void* i0, const void* i1, void* o, size_t len, int dtype, int op,
+                       void* stream);
+
+/*
+ * recvbuffs[r][0..len) = fold over ranks of sendbuffs[*][0..len), for every r.
+ * Replaces UcxCommunicator::all_reduce (src/ucx/all_reduce.cpp:23-109) and
+ * ShmCommunicator::_shm_all_reduce (src/shm/all_reduce.cpp:38-127) run on all N ranks.
+ * recvbuffs[r] may equal sendbuffs[r].
+ */
+MRV_API int mrv_all_reduce(const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks,
+                           size_t len, int dtype, int op, int order, int schedule, void* stream);
+
+/*
+ * recvbuffs[r][0..recvlen) = fold over ranks of sendbuffs[*][r*recvlen .. (r+1)*recvlen).
+ * Replaces UcxCommunicator::reduce_scatter (src/ucx/reduce_scatter.cpp:21-61) and
+ * ShmCommunicator::_shm_reduce_scatter (src/shm/reduce_scatter.cpp:21-97).
+ */
+MRV_API int mrv_reduce_scatter(const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks,
+                               size_t recvlen, int dtype, int op, int order, void* stream);
+
+/*
+ * recvbuffs[k][i*sendlen + j] = sendbuffs[i][j] for every k.
+ * Replaces UcxCommunicator::all_gather (src/ucx/all_gather.cpp:21-63) and _shm_all_gather
+ * (src/shm/all_gather.cpp:28-55).
+ */
+MRV_API int mrv_all_gather(const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks,
+                           size_t sendlen, int dtype, void* stream);
+
+/*
+ * recvbuffs[j][i*len + k] = sendbuffs[i][j*len + k].
+ * Replaces UcxCommunicator::all_to_all (src/ucx/all_to_all.cpp:21-43) and _shm_all_to_all
+ * (src/shm/all_to_all.cpp:18-59).
+ */
+MRV_API int mrv_all_to_all(const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks,
+                           size_t len, int dtype, void* stream);
+
+/*
+ * recvbuffs[i][j] = sendbuff_root[i*recvlen + j].
+ * Replaces UcxCommunicator::scatter (src/ucx/scatter.cpp:21-46), ShmCommunicator::scatter
+ * (src/shm/scatter.cpp:21-42).
+ */
+MRV_API int mrv_scatter(const void* sendbuff_root, void* const* recvbuffs, uint32_t nranks,
+                        size_t recvlen, int dtype, uint32_t root, void* stream);
+
+/*
+ * recvbuff_root[i*sendlen + j] = sendbuffs[i][j].
+ * Replaces UcxCommunicator::gather (src/ucx/gather.cpp:21-46), _shm_gather (src/shm/gather.cpp:19-49).
+ */
+MRV_API int mrv_gather(const void* const* sendbuffs, void* recvbuff_root, uint32_t nranks,
+                       size_t sendlen, int dtype, uint32_t root, void* stream);
+
+/*
+ * recvbuffs[r][j] = sendbuff_root[j] for every r.
+ * Replaces UcxCommunicator::broadcast (src/ucx/broadcast.cpp:21-76), ShmCommunicator::broadcast
+ * (src/shm/broadcast.cpp:19-51).
+ */
+MRV_API int mrv_broadcast(const void* sendbuff_root, void* const* recvbuffs, uint32_t nranks,
+                          size_t len, int dtype, uint32_t root, void* stream);
+
+/* ---- host-side planning, no device access -------------------------------------------------- */
+
+/* len/C split with the remainder on the first chunks (src/ucx/all_reduce.cpp:33-38,48-51). */
+MRV_API int mrv_chunk_partition(size_t len, uint32_t nchunks, size_t* sizes, size_t* offsets);
+
+/*
+ * Fold order of chunk `chunk` for `collective` (MRV_ALL_REDUCE or MRV_REDUCE_SCATTER): ranks[0]
+ * seeds the accumulator.  *new_wins_ties: MAX/MIN keep the newcomer on equal / unordered operands.
+ * *nchunks: number of chunks the order splits the buffer into.  *owner: rank the ring leaves the
+ * finished chunk on.
+ */
+MRV_API int mrv_fold_order(int collective, int order, uint32_t nranks, uint32_t chunk, uint32_t* ranks,
+                           int* new_wins_ties, uint32_t* nchunks, uint32_t* owner);
+
+/* One run of a planned launch, as mrv_describe() reports it. */
+typedef struct mrv_plan_run {
+    uint32_t step;          /* launch index within the collective */
+    uint32_t kind;          /* 0 = fold run, 1 = block copy of a pack launch */
+    uint32_t nfold;         /* fold: inputs combined per element (1 = copy) */
+    uint32_t nout;          /* fold: destinations */
+    uint32_t new_wins_ties; /* fold */
+    uint32_t vector;        /* fold: 1 = walked in 16-byte vectors; pack: bytes per lane access */
+    uint32_t start;         /* fold: seed rank; pack: source rank */
+    int32_t dir;            /* fold: +1 / -1 */
+    uint32_t out_first;     /* fold: first destination rank; pack: destination rank */
+    uint32_t tiles;         /* workgroups this run occupies */
+    uint64_t in_begin;      /* fold: first element in the inputs; pack: source byte offset */
+    uint64_t out_begin;     /* fold: first element in the outputs; pack: destination byte offset */
+    uint64_t count;         /* fold: elements; pack: bytes */
+} mrv_plan_run;
+
+/*
+ * Plans `collective` exactly as the device entry points do, without touching a device, and writes
+ * up to `cap` runs.  Pointers are only inspected for alignment and aliasing.  For MRV_SCATTER /
+ * MRV_BROADCAST only sendbuffs[root] is read from the send array, for MRV_GATHER only
+ * recvbuffs[root]; for MRV_REDUCE2 sendbuffs = {i0, i1}, recvbuffs = {o}.
+ * *nruns receives the number of runs the plan has (which may exceed cap), *bytes_read /
+ * *bytes_written the algorithmic HBM bytes of the whole plan.
+ */
+MRV_API int mrv_describe(int collective, const void* const* sendbuffs, void* const* recvbuffs,
+                         uint32_t nranks, size_t count, int dtype, int order, int schedule, uint32_t root,
+                         mrv_plan_run* runs, size_t cap, size_t* nruns, uint64_t* bytes_read,
+                         uint64_t* bytes_written);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MEGRAY_VRANK_H */

@@ -1,0 +1,205 @@
+"""Host-side mirror of the MegRay interface for the virtual-rank backend.
+
+Names, argument meaning and error behaviour follow the reference's C++ API
+(include/megray/common.h, include/megray/communicator.h): ``DType`` / ``ReduceOp`` / ``Status``
+carry the same numeric values, lengths are element counts, contract violations raise
+``MegRayError`` where the reference throws ``MegRay::Exception``.
+
+The flat functions here take the buffers of all N virtual ranks at once (device pointers as ints,
+or anything with ``data_ptr()``); they are thin wrappers over the C ABI.
+"""
+import ctypes
+import enum
+
+from . import _lib
+
+
+class Status(enum.IntEnum):
+    OK = 0
+    SYS_ERROR = 1
+    CUDA_ERR = 2
+    NCCL_ERR = 3
+    UCX_ERR = 4
+    ENV_ERROR = 5
+    INVALID_ARGUMENT = 6
+    INVALID_USAGE = 7
+    UNEXPECTED_ERR = 8
+    NOT_IMPLEMENTED = 9
+    HIP_ERR = 10
+    RCCL_ERR = 11
+
+
+class Backend(enum.IntEnum):
+    NCCL = 0
+    UCX = 1
+    RCCL = 2
+    SHM = 3
+    VRANK = 4
+
+
+class DType(enum.IntEnum):
+    INT8 = 0
+    UINT8 = 1
+    INT32 = 2
+    UINT32 = 3
+    INT64 = 4
+    UINT64 = 5
+    FLOAT16 = 6
+    FLOAT32 = 7
+    FLOAT64 = 8
+    CHAR = 9
+
+
+class ReduceOp(enum.IntEnum):
+    SUM = 0
+    MAX = 1
+    MIN = 2
+
+
+class FoldOrder(enum.IntEnum):
+    UCX = 0
+    SHM = 1
+    RANK0 = 2
+
+
+class Schedule(enum.IntEnum):
+    FUSED = 0
+    TWO_PHASE = 1
+    RING = 2
+
+
+class Collective(enum.IntEnum):
+    ALL_REDUCE = 0
+    REDUCE_SCATTER = 1
+    ALL_GATHER = 2
+    ALL_TO_ALL = 3
+    SCATTER = 4
+    GATHER = 5
+    BROADCAST = 6
+    REDUCE2 = 7
+
+
+MAX_RANKS = 16
+
+
+class MegRayError(RuntimeError):
+    """Raised where the reference throws MegRay::Exception or returns a non-OK Status."""
+
+    def __init__(self, status, message):
+        super().__init__(f"[{Status(status).name}] {message}")
+        self.status = Status(status)
+        self.message = message
+
+
+def _check(status):
+    if status != 0:
+        raise MegRayError(status, _lib.load().mrv_last_error().decode())
+
+
+def _ptr(buf):
+    if buf is None:
+        return None
+    if hasattr(buf, "data_ptr"):
+        return buf.data_ptr()
+    return int(buf)
+
+
+def _ptr_array(bufs):
+    arr = (ctypes.c_void_p * len(bufs))()
+    for i, b in enumerate(bufs):
+        arr[i] = _ptr(b)
+    return arr
+
+
+def _stream(stream):
+    if stream is None:
+        return None
+    if hasattr(stream, "cuda_stream"):
+        return stream.cuda_stream
+    return int(stream)
+
+
+def get_dtype_size(dtype):
+    """MegRay::get_dtype_size (src/core/common.cpp:19-38); raises 'unknown dtype'."""
+    size = _lib.load().mrv_dtype_size(int(dtype))
+    if size == 0:
+        raise MegRayError(Status.INVALID_ARGUMENT, _lib.load().mrv_last_error().decode())
+    return size
+
+
+def reduce(i0, i1, o, length, dtype, op, stream=None):
+    """o = i0 OP i1 (MegRay::reduce, src/ucx/utils.h:21-22)."""
+    _check(_lib.load().mrv_reduce(_ptr(i0), _ptr(i1), _ptr(o), length, int(dtype), int(op), _stream(stream)))
+
+
+def all_reduce(sendbuffs, recvbuffs, length, dtype, op, order=FoldOrder.UCX, schedule=Schedule.FUSED,
+               stream=None):
+    _check(_lib.load().mrv_all_reduce(_ptr_array(sendbuffs), _ptr_array(recvbuffs), len(sendbuffs), length,
+                                      int(dtype), int(op), int(order), int(schedule), _stream(stream)))
+
+
+def reduce_scatter(sendbuffs, recvbuffs, recvlen, dtype, op, order=FoldOrder.UCX, stream=None):
+    _check(_lib.load().mrv_reduce_scatter(_ptr_array(sendbuffs), _ptr_array(recvbuffs), len(sendbuffs), recvlen,
+                                          int(dtype), int(op), int(order), _stream(stream)))
+
+
+def all_gather(sendbuffs, recvbuffs, sendlen, dtype, stream=None):
+    _check(_lib.load().mrv_all_gather(_ptr_array(sendbuffs), _ptr_array(recvbuffs), len(sendbuffs), sendlen,
+                                      int(dtype), _stream(stream)))
+
+
+def all_to_all(sendbuffs, recvbuffs, length, dtype, stream=None):
+    _check(_lib.load().mrv_all_to_all(_ptr_array(sendbuffs), _ptr_array(recvbuffs), len(sendbuffs), length,
+                                      int(dtype), _stream(stream)))
+
+
+def scatter(sendbuff_root, recvbuffs, recvlen, dtype, root, stream=None):
+    _check(_lib.load().mrv_scatter(_ptr(sendbuff_root), _ptr_array(recvbuffs), len(recvbuffs), recvlen,
+                                   int(dtype), root, _stream(stream)))
+
+
+def gather(sendbuffs, recvbuff_root, sendlen, dtype, root, stream=None):
+    _check(_lib.load().mrv_gather(_ptr_array(sendbuffs), _ptr(recvbuff_root), len(sendbuffs), sendlen,
+                                  int(dtype), root, _stream(stream)))
+
+
+def broadcast(sendbuff_root, recvbuffs, length, dtype, root, stream=None):
+    _check(_lib.load().mrv_broadcast(_ptr(sendbuff_root), _ptr_array(recvbuffs), len(recvbuffs), length,
+                                     int(dtype), root, _stream(stream)))
+
+
+def chunk_partition(length, nchunks):
+    sizes = (ctypes.c_size_t * nchunks)()
+    offs = (ctypes.c_size_t * nchunks)()
+    _check(_lib.load().mrv_chunk_partition(length, nchunks, sizes, offs))
+    return list(sizes), list(offs)
+
+
+def fold_order(collective, order, nranks, chunk):
+    """-> (ranks, new_wins_ties, nchunks, owner)"""
+    ranks = (ctypes.c_uint32 * max(nranks, 1))()
+    new_wins = ctypes.c_int(0)
+    nchunks = ctypes.c_uint32(0)
+    owner = ctypes.c_uint32(0)
+    _check(_lib.load().mrv_fold_order(int(collective), int(order), nranks, chunk, ranks, ctypes.byref(new_wins),
+                                      ctypes.byref(nchunks), ctypes.byref(owner)))
+    return list(ranks)[:nranks], bool(new_wins.value), nchunks.value, owner.value
+
+
+def describe(collective, sendptrs, recvptrs, count, dtype, order=FoldOrder.UCX, schedule=Schedule.FUSED,
+             root=0, nranks=None):
+    """Plan a collective on the host only.  -> (list of run dicts, bytes_read, bytes_written)"""
+    nranks = nranks if nranks is not None else max(len(sendptrs), len(recvptrs))
+    cap = 4096
+    runs = (_lib.PlanRun * cap)()
+    n = ctypes.c_size_t(0)
+    br = ctypes.c_uint64(0)
+    bw = ctypes.c_uint64(0)
+    _check(_lib.load().mrv_describe(int(collective), _ptr_array(sendptrs), _ptr_array(recvptrs), nranks, count,
+                                    int(dtype), int(order), int(schedule), root, runs, cap, ctypes.byref(n),
+                                    ctypes.byref(br), ctypes.byref(bw)))
+    out = []
+    for i in range(min(n.value, cap)):
+        r = runs[i]
+        out.append({name: getattr(r, name) for name, _ in _lib.PlanRun._fields_})
+    return out, br.value, bw.value

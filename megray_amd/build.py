@@ -1,0 +1,67 @@
+"""Builds libmegray_vrank.so (the gfx950 kernels, the planner, the MegRay C++ API and the C ABI)
+with hipcc, in tree.  Run as ``python -m megray_amd.build``."""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+OBJ_DIR = os.path.join(CSRC, "build")
+LIB_PATH = os.path.join(HERE, "libmegray_vrank.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+ARCH = "gfx950"
+
+COMMON_FLAGS = [
+    "-std=c++17", "-O3", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter",
+    "-ffp-contract=off",  # a fold is a chain of single IEEE operations; never fuse
+    f"-I{os.path.join(ROOT, 'include')}", f"-I{CSRC}",
+]
+# device code: gfx950 only; packed fp32 instructions are kept out of the generated code
+DEVICE_FLAGS = [f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def sources():
+    out = []
+    for name in sorted(os.listdir(CSRC)):
+        if name.endswith(".cpp") or name.endswith(".hip"):
+            out.append(os.path.join(CSRC, name))
+    return out
+
+
+def _compile(src):
+    obj = os.path.join(OBJ_DIR, os.path.basename(src) + ".o")
+    cmd = [HIPCC] + COMMON_FLAGS
+    if src.endswith(".hip"):
+        cmd += ["-x", "hip"] + DEVICE_FLAGS
+    cmd += ["-c", src, "-o", obj]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    return src, obj, proc
+
+
+def build_library(verbose=True):
+    """Compile every source and link the shared library.  Always recompiles."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    srcs = sources()
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+        results = list(pool.map(_compile, srcs))
+    objs = []
+    for src, obj, proc in results:
+        noise = "'-packed-fp32-ops' is not a recognized feature"
+        err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)
+        if proc.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {src}:\n{proc.stdout}\n{proc.stderr}")
+        if verbose and err.strip():
+            print(err, file=sys.stderr)
+        objs.append(obj)
+    link = [HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", LIB_PATH] + objs + ["-lpthread"]
+    proc = subprocess.run(link, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"link failed:\n{proc.stdout}\n{proc.stderr}")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build_library())

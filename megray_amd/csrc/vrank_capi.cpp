@@ -1,0 +1,304 @@
+// extern "C" face of the library (include/megray_vrank.h).
+#include "megray_vrank.h"
+
+#include <cstdio>
+#include <cstring>
+#include <exception>
+
+#include "vrank_engine.h"
+#include "vrank_plan.h"
+
+using namespace MegRay;
+using namespace MegRay::vrank;
+
+namespace {
+
+thread_local char g_last_error[256] = "";
+
+void set_error(const char* text) {
+    std::snprintf(g_last_error, sizeof(g_last_error), "%s", text);
+}
+
+// Runs `body` (which returns a Status), translating exceptions the way the header promises.
+template <typename F>
+int guarded(F&& body) {
+    try {
+        Status st = body();
+        if (st == MEGRAY_INVALID_ARGUMENT) {
+            set_error(plan_error());
+        } else if (st == MEGRAY_HIP_ERR) {
+            set_error("hip error (see the log line on stderr)");
+        } else if (st != MEGRAY_OK) {
+            set_error("error");
+        }
+        return int(st);
+    } catch (const MegRay::Exception& e) {
+        set_error(e.what());
+        return int(MEGRAY_INVALID_ARGUMENT);
+    } catch (const std::exception& e) {
+        set_error(e.what());
+        return int(MEGRAY_UNEXPECTED_ERR);
+    }
+}
+
+hipStream_t as_stream(void* stream) {
+    return static_cast<hipStream_t>(stream);
+}
+
+FoldOrder as_order(int order) {
+    if (order < 0 || order >= kOrderCount) MEGRAY_THROW("unknown fold order");
+    return static_cast<FoldOrder>(order);
+}
+
+Schedule as_schedule(int schedule) {
+    if (schedule < 0 || schedule >= kSchedCount) MEGRAY_THROW("unknown schedule");
+    return static_cast<Schedule>(schedule);
+}
+
+void need(const void* p, const char* what) {
+    if (!p) MEGRAY_THROW(what);
+}
+
+}  // namespace
+
+extern "C" {
+
+int mrv_abi_version(void) {
+    return 1;
+}
+
+const char* mrv_last_error(void) {
+    return g_last_error;
+}
+
+size_t mrv_dtype_size(int dtype) {
+    try {
+        return get_dtype_size(static_cast<DType>(dtype));
+    } catch (const MegRay::Exception& e) {
+        set_error(e.what());
+        return 0;
+    }
+}
+
+int mrv_reduce(const void* i0, const void* i1, void* o, size_t len, int dtype, int op, void* stream) {
+    return guarded([&] {
+        return reduce2(i0, i1, o, len, static_cast<DType>(dtype), static_cast<ReduceOp>(op), as_stream(stream));
+    });
+}
+
+int mrv_all_reduce(const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks, size_t len, int dtype,
+                   int op, int order, int schedule, void* stream) {
+    return guarded([&] {
+        need(sendbuffs, "sendbuffs is null");
+        need(recvbuffs, "recvbuffs is null");
+        return all_reduce(sendbuffs, recvbuffs, nranks, len, static_cast<DType>(dtype), static_cast<ReduceOp>(op),
+                          as_order(order), as_schedule(schedule), as_stream(stream));
+    });
+}
+
+int mrv_reduce_scatter(const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks, size_t recvlen,
+                       int dtype, int op, int order, void* stream) {
+    return guarded([&] {
+        need(sendbuffs, "sendbuffs is null");
+        need(recvbuffs, "recvbuffs is null");
+        return reduce_scatter(sendbuffs, recvbuffs, nranks, recvlen, static_cast<DType>(dtype),
+                              static_cast<ReduceOp>(op), as_order(order), as_stream(stream));
+    });
+}
+
+int mrv_all_gather(const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks, size_t sendlen,
+                   int dtype, void* stream) {
+    return guarded([&] {
+        need(sendbuffs, "sendbuffs is null");
+        need(recvbuffs, "recvbuffs is null");
+        return all_gather(sendbuffs, recvbuffs, nranks, sendlen, static_cast<DType>(dtype), as_stream(stream));
+    });
+}
+
+int mrv_all_to_all(const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks, size_t len, int dtype,
+                   void* stream) {
+    return guarded([&] {
+        need(sendbuffs, "sendbuffs is null");
+        need(recvbuffs, "recvbuffs is null");
+        return all_to_all(sendbuffs, recvbuffs, nranks, len, static_cast<DType>(dtype), as_stream(stream));
+    });
+}
+
+int mrv_scatter(const void* sendbuff_root, void* const* recvbuffs, uint32_t nranks, size_t recvlen, int dtype,
+                uint32_t root, void* stream) {
+    return guarded([&] {
+        need(recvbuffs, "recvbuffs is null");
+        return scatter(sendbuff_root, recvbuffs, nranks, recvlen, static_cast<DType>(dtype), root,
+                       as_stream(stream));
+    });
+}
+
+int mrv_gather(const void* const* sendbuffs, void* recvbuff_root, uint32_t nranks, size_t sendlen, int dtype,
+               uint32_t root, void* stream) {
+    return guarded([&] {
+        need(sendbuffs, "sendbuffs is null");
+        return gather(sendbuffs, recvbuff_root, nranks, sendlen, static_cast<DType>(dtype), root,
+                      as_stream(stream));
+    });
+}
+
+int mrv_broadcast(const void* sendbuff_root, void* const* recvbuffs, uint32_t nranks, size_t len, int dtype,
+                  uint32_t root, void* stream) {
+    return guarded([&] {
+        need(recvbuffs, "recvbuffs is null");
+        return broadcast(sendbuff_root, recvbuffs, nranks, len, static_cast<DType>(dtype), root,
+                         as_stream(stream));
+    });
+}
+
+int mrv_chunk_partition(size_t len, uint32_t nchunks, size_t* sizes, size_t* offsets) {
+    return guarded([&] {
+        if (!nchunks || !sizes || !offsets) MEGRAY_THROW("nchunks must be positive and the arrays non-null");
+        uint64_t s[256], o[256];
+        if (nchunks > 256) MEGRAY_THROW("at most 256 chunks");
+        chunk_partition(len, nchunks, s, o);
+        for (uint32_t i = 0; i < nchunks; ++i) {
+            sizes[i] = size_t(s[i]);
+            offsets[i] = size_t(o[i]);
+        }
+        return MEGRAY_OK;
+    });
+}
+
+int mrv_fold_order(int collective, int order, uint32_t nranks, uint32_t chunk, uint32_t* ranks,
+                   int* new_wins_ties, uint32_t* nchunks, uint32_t* owner) {
+    return guarded([&] {
+        if (collective != MRV_ALL_REDUCE && collective != MRV_REDUCE_SCATTER)
+            MEGRAY_THROW("fold orders exist for all_reduce and reduce_scatter");
+        if (nranks < 1 || nranks > kMaxRanks) MEGRAY_THROW("nranks must be in [1, 16]");
+        const FoldOrder fo = as_order(order);
+        const Collective coll = collective == MRV_ALL_REDUCE ? kAllReduce : kReduceScatter;
+        const uint32_t chunks = order_chunks(fo, nranks);
+        if (chunk >= chunks) MEGRAY_THROW("chunk out of range");
+        uint8_t start, own;
+        int8_t dir;
+        chunk_fold_order(coll, fo, nranks, chunk, &start, &dir, &own);
+        if (ranks)
+            for (uint32_t j = 0; j < nranks; ++j)
+                ranks[j] = dir > 0 ? ring_add(start, j, nranks) : ring_sub(start, j, nranks);
+        if (new_wins_ties) *new_wins_ties = order_new_wins_ties(coll, fo) ? 1 : 0;
+        if (nchunks) *nchunks = chunks;
+        if (owner) *owner = own;
+        return MEGRAY_OK;
+    });
+}
+
+int mrv_describe(int collective, const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks,
+                 size_t count, int dtype, int order, int schedule, uint32_t root, mrv_plan_run* runs, size_t cap,
+                 size_t* nruns, uint64_t* bytes_read, uint64_t* bytes_written) {
+    return guarded([&] {
+        need(sendbuffs, "sendbuffs is null");
+        need(recvbuffs, "recvbuffs is null");
+        const DType dt = static_cast<DType>(dtype);
+        Plan plan;
+        Status st = MEGRAY_OK;
+        switch (collective) {
+            case MRV_ALL_REDUCE:
+                st = plan_all_reduce(plan, sendbuffs, recvbuffs, nranks, count, reduce_elem_size(dt), as_order(order),
+                                     as_schedule(schedule));
+                break;
+            case MRV_REDUCE_SCATTER:
+                st = plan_reduce_scatter(plan, sendbuffs, recvbuffs, nranks, count, reduce_elem_size(dt),
+                                         as_order(order), as_schedule(schedule));
+                break;
+            case MRV_ALL_GATHER:
+                st = plan_all_gather(plan, sendbuffs, recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)));
+                break;
+            case MRV_ALL_TO_ALL:
+                st = plan_all_to_all(plan, sendbuffs, recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)));
+                break;
+            case MRV_SCATTER:
+                if (root >= nranks) MEGRAY_THROW("root out of range");
+                st = plan_scatter(plan, sendbuffs[root], recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)), root);
+                break;
+            case MRV_GATHER:
+                if (root >= nranks) MEGRAY_THROW("root out of range");
+                st = plan_gather(plan, sendbuffs, recvbuffs[root], nranks, count, uint32_t(get_dtype_size(dt)), root);
+                break;
+            case MRV_BROADCAST:
+                if (root >= nranks) MEGRAY_THROW("root out of range");
+                st = plan_broadcast(plan, sendbuffs[root], recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)),
+                                    root);
+                break;
+            case MRV_REDUCE2:
+                st = plan_reduce2(plan, sendbuffs[0], sendbuffs[1], recvbuffs[0], count, reduce_elem_size(dt));
+                break;
+            default:
+                MEGRAY_THROW("unknown collective");
+        }
+        if (st != MEGRAY_OK) return st;
+        size_t n = 0;
+        auto emit = [&](const mrv_plan_run& run) {
+            if (runs && n < cap) runs[n] = run;
+            ++n;
+        };
+        for (size_t i = 0; i < plan.steps.size(); ++i) {
+            const Step& step = plan.steps[i];
+            if (step.kind == Step::kFold) {
+                const FoldLaunch& L = step.fold;
+                for (uint32_t s = 0; s < L.nseg; ++s) {
+                    const FoldSegment& sg = L.seg[s];
+                    mrv_plan_run run;
+                    std::memset(&run, 0, sizeof(run));
+                    run.step = uint32_t(i);
+                    run.kind = 0;
+                    run.nfold = L.nfold;
+                    run.nout = L.nout;
+                    run.new_wins_ties = L.new_wins_ties;
+                    run.vector = (sg.flags & kSegVector) ? 1 : 0;
+                    run.start = sg.start;
+                    run.dir = sg.dir;
+                    run.out_first = sg.out_first;
+                    const uint32_t next = s + 1 < L.nseg ? L.seg[s + 1].first_tile : L.total_tiles;
+                    run.tiles = next - sg.first_tile;
+                    run.in_begin = sg.in_begin;
+                    run.out_begin = sg.out_begin;
+                    run.count = sg.count;
+                    emit(run);
+                }
+            } else {
+                const PackLaunch& L = step.pack;
+                for (uint32_t c = 0; c < L.ncopies; ++c) {
+                    mrv_plan_run run;
+                    std::memset(&run, 0, sizeof(run));
+                    run.step = uint32_t(i);
+                    run.kind = 1;
+                    run.nfold = 1;
+                    run.nout = 1;
+                    run.vector = L.width;
+                    run.dir = 1;
+                    run.tiles = L.tiles_per_copy;
+                    run.count = L.block_bytes;
+                    if (L.mode == kPackAllToAll) {
+                        run.start = c / L.nranks;
+                        run.in_begin = uint64_t(c % L.nranks) * L.block_bytes;
+                        run.out_first = c % L.nranks;
+                        run.out_begin = uint64_t(c / L.nranks) * L.block_bytes;
+                    } else if (L.mode == kPackScatter) {
+                        run.start = L.root;
+                        run.in_begin = uint64_t(c) * L.block_bytes;
+                        run.out_first = c;
+                        run.out_begin = 0;
+                    } else {
+                        run.start = c;
+                        run.in_begin = 0;
+                        run.out_first = L.root;
+                        run.out_begin = uint64_t(c) * L.block_bytes;
+                    }
+                    emit(run);
+                }
+            }
+        }
+        if (nruns) *nruns = n;
+        if (bytes_read) *bytes_read = plan.bytes_read;
+        if (bytes_written) *bytes_written = plan.bytes_written;
+        return MEGRAY_OK;
+    });
+}
+
+}  // extern "C"

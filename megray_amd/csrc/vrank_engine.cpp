@@ -1,0 +1,110 @@
+#include "vrank_engine.h"
+
+#include "megray/hip_context.h"
+#include "vrank_kernels.h"
+
+namespace MegRay {
+namespace vrank {
+
+uint32_t reduce_elem_size(DType dtype) {
+    switch (dtype) {
+        case MEGRAY_INT8:
+        case MEGRAY_UINT8:
+            return 1;
+        case MEGRAY_FLOAT16:
+            return 2;
+        case MEGRAY_INT32:
+        case MEGRAY_UINT32:
+        case MEGRAY_FLOAT32:
+            return 4;
+        case MEGRAY_INT64:
+        case MEGRAY_UINT64:
+        case MEGRAY_FLOAT64:
+            return 8;
+        default:
+            MEGRAY_THROW("unknown dtype");
+    }
+}
+
+void check_reduce_op(ReduceOp op) {
+    if (op != MEGRAY_SUM && op != MEGRAY_MAX && op != MEGRAY_MIN) MEGRAY_THROW("unknown reduce op");
+}
+
+Status execute(const Plan& plan, DType dtype, ReduceOp op, hipStream_t stream) {
+    for (const Step& step : plan.steps) {
+        if (step.kind == Step::kFold) {
+            HIP_CHECK(launch_fold(step.fold, dtype, op, stream));
+        } else {
+            HIP_CHECK(launch_pack(step.pack, stream));
+        }
+    }
+    return MEGRAY_OK;
+}
+
+Status reduce2(const void* i0, const void* i1, void* o, size_t len, DType dtype, ReduceOp op,
+               hipStream_t stream) {
+    const uint32_t size = reduce_elem_size(dtype);
+    check_reduce_op(op);
+    Plan plan;
+    Status st = plan_reduce2(plan, i0, i1, o, len, size);
+    return st == MEGRAY_OK ? execute(plan, dtype, op, stream) : st;
+}
+
+Status all_reduce(const void* const* send, void* const* recv, uint32_t nranks, size_t len, DType dtype,
+                  ReduceOp op, FoldOrder order, Schedule sched, hipStream_t stream) {
+    const uint32_t size = reduce_elem_size(dtype);
+    check_reduce_op(op);
+    // a ring hop stores its partial result in the element type: FLOAT16 would round N-1 times
+    if (sched == kSchedRing && dtype == MEGRAY_FLOAT16)
+        MEGRAY_THROW("the ring schedule is not offered for FLOAT16 (it would round at every hop)");
+    Plan plan;
+    Status st = plan_all_reduce(plan, send, recv, nranks, len, size, order, sched);
+    return st == MEGRAY_OK ? execute(plan, dtype, op, stream) : st;
+}
+
+Status reduce_scatter(const void* const* send, void* const* recv, uint32_t nranks, size_t recvlen,
+                      DType dtype, ReduceOp op, FoldOrder order, hipStream_t stream) {
+    const uint32_t size = reduce_elem_size(dtype);
+    check_reduce_op(op);
+    Plan plan;
+    Status st = plan_reduce_scatter(plan, send, recv, nranks, recvlen, size, order, kSchedFused);
+    return st == MEGRAY_OK ? execute(plan, dtype, op, stream) : st;
+}
+
+Status all_gather(const void* const* send, void* const* recv, uint32_t nranks, size_t sendlen, DType dtype,
+                  hipStream_t stream) {
+    Plan plan;
+    Status st = plan_all_gather(plan, send, recv, nranks, sendlen, uint32_t(get_dtype_size(dtype)));
+    return st == MEGRAY_OK ? execute(plan, dtype, MEGRAY_SUM, stream) : st;
+}
+
+Status all_to_all(const void* const* send, void* const* recv, uint32_t nranks, size_t len, DType dtype,
+                  hipStream_t stream) {
+    Plan plan;
+    Status st = plan_all_to_all(plan, send, recv, nranks, len, uint32_t(get_dtype_size(dtype)));
+    return st == MEGRAY_OK ? execute(plan, dtype, MEGRAY_SUM, stream) : st;
+}
+
+Status scatter(const void* send_root, void* const* recv, uint32_t nranks, size_t recvlen, DType dtype,
+               uint32_t root, hipStream_t stream) {
+    Plan plan;
+    Status st = plan_scatter(plan, send_root, recv, nranks, recvlen, uint32_t(get_dtype_size(dtype)), root);
+    return st == MEGRAY_OK ? execute(plan, dtype, MEGRAY_SUM, stream) : st;
+}
+
+Status gather(const void* const* send, void* recv_root, uint32_t nranks, size_t sendlen, DType dtype,
+              uint32_t root, hipStream_t stream) {
+    Plan plan;
+    Status st = plan_gather(plan, send, recv_root, nranks, sendlen, uint32_t(get_dtype_size(dtype)), root);
+    return st == MEGRAY_OK ? execute(plan, dtype, MEGRAY_SUM, stream) : st;
+}
+
+Status broadcast(const void* send_root, void* const* recv, uint32_t nranks, size_t len, DType dtype,
+                 uint32_t root, hipStream_t stream) {
+    Plan plan;
+    Status st = plan_broadcast(plan, send_root, recv, nranks, len, uint32_t(get_dtype_size(dtype)), root);
+    return st == MEGRAY_OK ? execute(plan, dtype, MEGRAY_SUM, stream) : st;
+}
+
+}  // namespace vrank
+}  // namespace MegRay

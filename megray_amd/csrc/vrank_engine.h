@@ -1,0 +1,44 @@
+// The virtual-rank collectives as plain functions over N rank buffers in one GPU's memory.
+// Both faces of the library sit on these: the C ABI (vrank_capi.cpp) calls them directly, the
+// MegRay::Communicator backend (vrank_communicator.cpp) calls them once all ranks have arrived.
+//
+// Contract violations throw MegRay::Exception like the reference does (unknown dtype / op:
+// src/ucx/kernel.cu:55-56,95-96); planner and HIP failures come back as a Status.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+
+#include "megray/common.h"
+#include "vrank_plan.h"
+
+namespace MegRay {
+namespace vrank {
+
+// Element size of a dtype a reduce kernel exists for; throws "unknown dtype" for MEGRAY_CHAR and
+// out-of-range values.  FLOAT16 is accepted (fp32 accumulation, one rounding).
+uint32_t reduce_elem_size(DType dtype);
+// Throws "unknown reduce op" outside SUM / MAX / MIN.
+void check_reduce_op(ReduceOp op);
+
+// Enqueue every launch of `plan` on `stream`.
+Status execute(const Plan& plan, DType dtype, ReduceOp op, hipStream_t stream);
+
+Status reduce2(const void* i0, const void* i1, void* o, size_t len, DType dtype, ReduceOp op,
+               hipStream_t stream);
+Status all_reduce(const void* const* send, void* const* recv, uint32_t nranks, size_t len, DType dtype,
+                  ReduceOp op, FoldOrder order, Schedule sched, hipStream_t stream);
+Status reduce_scatter(const void* const* send, void* const* recv, uint32_t nranks, size_t recvlen,
+                      DType dtype, ReduceOp op, FoldOrder order, hipStream_t stream);
+Status all_gather(const void* const* send, void* const* recv, uint32_t nranks, size_t sendlen, DType dtype,
+                  hipStream_t stream);
+Status all_to_all(const void* const* send, void* const* recv, uint32_t nranks, size_t len, DType dtype,
+                  hipStream_t stream);
+Status scatter(const void* send_root, void* const* recv, uint32_t nranks, size_t recvlen, DType dtype,
+               uint32_t root, hipStream_t stream);
+Status gather(const void* const* send, void* recv_root, uint32_t nranks, size_t sendlen, DType dtype,
+              uint32_t root, hipStream_t stream);
+Status broadcast(const void* send_root, void* const* recv, uint32_t nranks, size_t len, DType dtype,
+                 uint32_t root, hipStream_t stream);
+
+}  // namespace vrank
+}  // namespace MegRay

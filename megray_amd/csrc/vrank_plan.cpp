@@ -1,0 +1,476 @@
+#include "vrank_plan.h"
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+
+namespace MegRay {
+namespace vrank {
+
+// propagate a planner error without logging: the caller reports it
+#define PLAN_TRY(expr)                              \
+    do {                                            \
+        Status plan_status_ = (expr);               \
+        if (plan_status_ != MEGRAY_OK) return plan_status_; \
+    } while (0)
+
+namespace {
+
+thread_local char g_plan_error[256] = "";
+
+Status invalid(const char* what) {
+    std::snprintf(g_plan_error, sizeof(g_plan_error), "%s", what);
+    return MEGRAY_INVALID_ARGUMENT;
+}
+
+bool aligned16(const void* p) {
+    return (reinterpret_cast<uintptr_t>(p) & (kVecBytes - 1)) == 0;
+}
+
+bool overlaps(const void* a, uint64_t a_bytes, const void* b, uint64_t b_bytes) {
+    if (!a || !b || !a_bytes || !b_bytes) return false;
+    const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+    return a0 < b0 + b_bytes && b0 < a0 + a_bytes;
+}
+
+// Collects runs of elements into fold launches, splitting each run into an unaligned head, a body
+// of whole 16-byte vectors and a tail, and opening a new launch when a descriptor is full.
+class FoldBuilder {
+public:
+    FoldBuilder(Plan& plan, const void* const* in, void* const* out, uint32_t nranks, uint32_t nfold,
+                uint32_t nout, uint32_t elem_size, bool new_wins)
+            : m_plan(plan) {
+        std::memset(&m_launch, 0, sizeof(m_launch));
+        m_aligned = true;
+        for (uint32_t r = 0; r < nranks; ++r) {
+            m_launch.in[r] = in[r];
+            m_launch.out[r] = out[r];
+            m_aligned = m_aligned && aligned16(in[r]) && aligned16(out[r]);  // null counts as aligned
+        }
+        m_launch.nranks = nranks;
+        m_launch.nfold = nfold;
+        m_launch.nout = nout;
+        m_launch.new_wins_ties = new_wins ? 1 : 0;
+        m_launch.unroll = fold_unroll(nfold);
+        m_launch.elem_size = elem_size;
+    }
+
+    void add_run(uint64_t in_begin, uint64_t out_begin, uint64_t count, uint8_t start, int8_t dir,
+                 uint8_t out_first) {
+        if (!count) return;
+        m_plan.bytes_read += count * m_launch.elem_size * m_launch.nfold;
+        m_plan.bytes_written += count * m_launch.elem_size * m_launch.nout;
+        const uint64_t epv = kVecBytes / m_launch.elem_size;
+        const bool vector = m_aligned && (in_begin % epv == out_begin % epv);
+        uint64_t head = 0, body = 0;
+        if (vector) {
+            head = std::min<uint64_t>((epv - in_begin % epv) % epv, count);
+            body = (count - head) / epv * epv;
+        }
+        if (!body) {
+            add_segment(in_begin, out_begin, count, start, dir, out_first, 0);
+            return;
+        }
+        const uint64_t tail = count - head - body;
+        if (head) add_segment(in_begin, out_begin, head, start, dir, out_first, 0);
+        add_segment(in_begin + head, out_begin + head, body, start, dir, out_first, kSegVector);
+        if (tail) add_segment(in_begin + head + body, out_begin + head + body, tail, start, dir, out_first, 0);
+    }
+
+    void finish() {
+        if (!m_launch.nseg) return;
+        Step step;
+        std::memset(&step, 0, sizeof(step));
+        step.kind = Step::kFold;
+        step.is_copy = m_launch.nfold == 1;
+        step.fold = m_launch;
+        m_plan.steps.push_back(step);
+        m_launch.nseg = 0;
+        m_launch.total_tiles = 0;
+    }
+
+private:
+    void add_segment(uint64_t in_begin, uint64_t out_begin, uint64_t count, uint8_t start, int8_t dir,
+                     uint8_t out_first, uint8_t flags) {
+        const uint64_t per_tile = tile_elems(m_launch, flags & kSegVector);
+        const uint64_t max_tiles = 0x7fffffffull;
+        while (count) {
+            if (m_launch.nseg == kMaxSegments || m_launch.total_tiles >= max_tiles) finish();
+            // a segment never takes more tiles than one launch's grid has left
+            const uint64_t room = max_tiles - m_launch.total_tiles;
+            const uint64_t take = std::min(count, room * per_tile);
+            FoldSegment& sg = m_launch.seg[m_launch.nseg++];
+            sg.in_begin = in_begin;
+            sg.out_begin = out_begin;
+            sg.count = take;
+            sg.first_tile = m_launch.total_tiles;
+            sg.start = start;
+            sg.dir = dir;
+            sg.out_first = out_first;
+            sg.flags = flags;
+            m_launch.total_tiles += uint32_t((take + per_tile - 1) / per_tile);
+            in_begin += take;
+            out_begin += take;
+            count -= take;
+        }
+    }
+
+    Plan& m_plan;
+    FoldLaunch m_launch;
+    bool m_aligned;
+};
+
+Status check_ranks(uint32_t nranks) {
+    if (nranks < 1 || nranks > kMaxRanks) return invalid("nranks must be in [1, 16]");
+    return MEGRAY_OK;
+}
+
+Status check_elem(uint32_t elem_size) {
+    if (elem_size != 1 && elem_size != 2 && elem_size != 4 && elem_size != 8)
+        return invalid("element size must be 1, 2, 4 or 8");
+    return MEGRAY_OK;
+}
+
+// Buffers of different ranks must not overlap.  A rank's own receive buffer may overlap its send
+// buffer only at the one offset where every element keeps its address (`recv == send + shift`).
+Status check_overlap(const void* const* send, uint64_t send_bytes, void* const* recv, uint64_t recv_bytes,
+                     uint32_t nranks, int64_t own_shift_bytes_per_rank) {
+    for (uint32_t a = 0; a < nranks; ++a) {
+        for (uint32_t b = a + 1; b < nranks; ++b)
+            if (overlaps(recv[a], recv_bytes, recv[b], recv_bytes))
+                return invalid("receive buffers of two ranks overlap");
+        for (uint32_t b = 0; b < nranks; ++b) {
+            if (!overlaps(recv[a], recv_bytes, send[b], send_bytes)) continue;
+            const intptr_t shift = int64_t(a) * own_shift_bytes_per_rank;
+            const bool in_place = a == b && reinterpret_cast<intptr_t>(recv[a]) ==
+                                                    reinterpret_cast<intptr_t>(send[a]) + shift;
+            if (!in_place) return invalid("a receive buffer overlaps a send buffer out of place");
+        }
+    }
+    return MEGRAY_OK;
+}
+
+}  // namespace
+
+const char* plan_error() {
+    return g_plan_error;
+}
+
+void chunk_partition(uint64_t len, uint32_t nchunks, uint64_t* sizes, uint64_t* offsets) {
+    const uint64_t quotient = len / nchunks, remainder = len % nchunks;
+    uint64_t offset = 0;
+    for (uint32_t i = 0; i < nchunks; ++i) {
+        sizes[i] = quotient + (i < remainder ? 1 : 0);
+        offsets[i] = offset;
+        offset += sizes[i];
+    }
+}
+
+uint32_t order_chunks(FoldOrder order, uint32_t nranks) {
+    switch (order) {
+        case kOrderUcx: return nranks;
+        case kOrderShm: return 2 * nranks;  // k = 2 chunks per rank, src/shm/all_reduce.cpp:42-43
+        default: return 1;
+    }
+}
+
+bool order_new_wins_ties(Collective coll, FoldOrder order) {
+    // src/ucx/reduce_scatter.cpp:50-51 calls reduce(incoming, local): the (i0 > i1) ? i0 : i1 of
+    // src/ucx/kernel.cu:24-38 then keeps the local (new) operand.  Every other loop keeps the
+    // accumulator: src/ucx/all_reduce.cpp:74-76 passes (local, incoming); std::max / std::min in
+    // src/shm/utils.cpp:24-32 return their first argument, the accumulator.
+    return order == kOrderUcx && coll == kReduceScatter;
+}
+
+void chunk_fold_order(Collective coll, FoldOrder order, uint32_t nranks, uint32_t chunk, uint8_t* start,
+                      int8_t* dir, uint8_t* owner) {
+    switch (order) {
+        case kOrderUcx:
+            *dir = 1;
+            if (coll == kAllReduce) {
+                // chunk c starts on rank c and is finished on rank c-1 (src/ucx/all_reduce.cpp:57-60)
+                *start = uint8_t(chunk % nranks);
+                *owner = uint8_t(ring_sub(chunk, 1, nranks));
+            } else {
+                // chunk c starts on rank c+1 and is finished on rank c (src/ucx/reduce_scatter.cpp:40-41)
+                *start = uint8_t(ring_add(chunk, 1, nranks));
+                *owner = uint8_t(chunk % nranks);
+            }
+            break;
+        case kOrderShm:
+            // chunk w belongs to rank w/2, whose copy seeds the arena; ranks w/2-1, w/2-2, ... add
+            // theirs (src/shm/all_reduce.cpp:91-109, src/shm/communicator.cpp:56-68)
+            *dir = -1;
+            *start = uint8_t((chunk / 2) % nranks);
+            *owner = *start;
+            break;
+        default:
+            *dir = 1;
+            *start = 0;
+            *owner = 0;
+            break;
+    }
+}
+
+Status plan_all_reduce(Plan& plan, const void* const* send, void* const* recv, uint32_t nranks,
+                       uint64_t len, uint32_t elem_size, FoldOrder order, Schedule sched) {
+    PLAN_TRY(check_ranks(nranks));
+    PLAN_TRY(check_elem(elem_size));
+    if (order < 0 || order >= kOrderCount) return invalid("unknown fold order");
+    if (sched < 0 || sched >= kSchedCount) return invalid("unknown schedule");
+    if (sched == kSchedRing && order != kOrderUcx) return invalid("the ring schedule exists for the ucx order only");
+    PLAN_TRY(check_overlap(send, len * elem_size, recv, len * elem_size, nranks, 0));
+    const uint32_t nchunks = order_chunks(order, nranks);
+    uint64_t sizes[kMaxChunks], offs[kMaxChunks];
+    chunk_partition(len, nchunks, sizes, offs);
+    const bool new_wins = order_new_wins_ties(kAllReduce, order);
+    const void* recv_in[kMaxRanks];
+    for (uint32_t r = 0; r < nranks; ++r) recv_in[r] = recv[r];
+
+    if (sched == kSchedFused) {
+        FoldBuilder fold(plan, send, recv, nranks, nranks, nranks, elem_size, new_wins);
+        for (uint32_t c = 0; c < nchunks; ++c) {
+            uint8_t start, owner;
+            int8_t dir;
+            chunk_fold_order(kAllReduce, order, nranks, c, &start, &dir, &owner);
+            fold.add_run(offs[c], offs[c], sizes[c], start, dir, 0);
+        }
+        fold.finish();
+        return MEGRAY_OK;
+    }
+
+    if (sched == kSchedTwoPhase) {
+        {   // reduce-scatter: the finished chunk lands on the rank the ring would leave it on
+            FoldBuilder fold(plan, send, recv, nranks, nranks, 1, elem_size, new_wins);
+            for (uint32_t c = 0; c < nchunks; ++c) {
+                uint8_t start, owner;
+                int8_t dir;
+                chunk_fold_order(kAllReduce, order, nranks, c, &start, &dir, &owner);
+                fold.add_run(offs[c], offs[c], sizes[c], start, dir, owner);
+            }
+            fold.finish();
+        }
+        if (nranks > 1) {  // all-gather: read the owner's chunk once, write the other N-1 ranks
+            FoldBuilder copy(plan, recv_in, recv, nranks, 1, nranks - 1, elem_size, false);
+            for (uint32_t c = 0; c < nchunks; ++c) {
+                uint8_t start, owner;
+                int8_t dir;
+                chunk_fold_order(kAllReduce, order, nranks, c, &start, &dir, &owner);
+                copy.add_run(offs[c], offs[c], sizes[c], owner, 1, uint8_t(ring_add(owner, 1, nranks)));
+            }
+            copy.finish();
+        }
+        return MEGRAY_OK;
+    }
+
+    // kSchedRing: the reference's steps, one launch each, with "send + receive into the workspace"
+    // replaced by reading the left neighbour's buffer in place.
+    {   // src/ucx/all_reduce.cpp:44-45
+        FoldBuilder copy(plan, send, recv, nranks, 1, 1, elem_size, false);
+        for (uint32_t r = 0; r < nranks; ++r)
+            if (send[r] != recv[r]) copy.add_run(0, 0, len, uint8_t(r), 1, uint8_t(r));
+        copy.finish();
+    }
+    for (uint32_t i = 0; i + 1 < nranks; ++i) {  // :61-82
+        FoldBuilder fold(plan, recv_in, recv, nranks, 2, 1, elem_size, false);
+        for (uint32_t r = 0; r < nranks; ++r) {
+            const uint32_t c = ring_sub(r, i + 1, nranks);
+            // reduce(local, incoming): incoming (the left rank's chunk) is the accumulator
+            fold.add_run(offs[c], offs[c], sizes[c], uint8_t(ring_sub(r, 1, nranks)), 1, uint8_t(r));
+        }
+        fold.finish();
+    }
+    for (uint32_t i = 0; i + 1 < nranks; ++i) {  // :88-101
+        FoldBuilder copy(plan, recv_in, recv, nranks, 1, 1, elem_size, false);
+        for (uint32_t r = 0; r < nranks; ++r) {
+            const uint32_t c = ring_sub(r, i, nranks);
+            copy.add_run(offs[c], offs[c], sizes[c], uint8_t(ring_sub(r, 1, nranks)), 1, uint8_t(r));
+        }
+        copy.finish();
+    }
+    return MEGRAY_OK;
+}
+
+Status plan_reduce_scatter(Plan& plan, const void* const* send, void* const* recv, uint32_t nranks,
+                           uint64_t recvlen, uint32_t elem_size, FoldOrder order, Schedule sched) {
+    PLAN_TRY(check_ranks(nranks));
+    PLAN_TRY(check_elem(elem_size));
+    if (order < 0 || order >= kOrderCount) return invalid("unknown fold order");
+    if (sched != kSchedFused) return invalid("reduce_scatter has the fused schedule only");
+    const uint64_t total = recvlen * nranks;
+    PLAN_TRY(check_overlap(send, total * elem_size, recv, recvlen * elem_size, nranks,
+                               int64_t(recvlen * elem_size)));
+    const uint32_t nchunks = order_chunks(order, nranks);
+    uint64_t sizes[kMaxChunks], offs[kMaxChunks];
+    chunk_partition(total, nchunks, sizes, offs);
+    FoldBuilder fold(plan, send, recv, nranks, nranks, 1, elem_size, order_new_wins_ties(kReduceScatter, order));
+    for (uint32_t c = 0; c < nchunks; ++c) {
+        uint8_t start, owner;
+        int8_t dir;
+        chunk_fold_order(kReduceScatter, order, nranks, c, &start, &dir, &owner);
+        // rank r receives elements [r * recvlen, (r + 1) * recvlen) whatever chunk they were folded in
+        uint64_t begin = offs[c];
+        const uint64_t end = offs[c] + sizes[c];
+        while (begin < end) {
+            const uint64_t r = begin / recvlen;
+            const uint64_t stop = std::min(end, (r + 1) * recvlen);
+            fold.add_run(begin, begin - r * recvlen, stop - begin, start, dir, uint8_t(r));
+            begin = stop;
+        }
+    }
+    fold.finish();
+    return MEGRAY_OK;
+}
+
+Status plan_all_gather(Plan& plan, const void* const* send, void* const* recv, uint32_t nranks,
+                       uint64_t sendlen, uint32_t elem_size) {
+    PLAN_TRY(check_ranks(nranks));
+    PLAN_TRY(check_elem(elem_size));
+    // in place: rank r's contribution already sits in its slot, send[r] == recv[r] + r * sendlen
+    for (uint32_t a = 0; a < nranks; ++a) {
+        for (uint32_t b = a + 1; b < nranks; ++b)
+            if (overlaps(recv[a], sendlen * nranks * elem_size, recv[b], sendlen * nranks * elem_size))
+                return invalid("receive buffers of two ranks overlap");
+        for (uint32_t b = 0; b < nranks; ++b) {
+            if (!overlaps(recv[a], sendlen * nranks * elem_size, send[b], sendlen * elem_size)) continue;
+            const bool in_place = a == b && static_cast<const char*>(send[a]) ==
+                                                    static_cast<const char*>(recv[a]) + a * sendlen * elem_size;
+            if (!in_place) return invalid("a receive buffer overlaps a send buffer out of place");
+        }
+    }
+    FoldBuilder copy(plan, send, recv, nranks, 1, nranks, elem_size, false);
+    for (uint32_t i = 0; i < nranks; ++i) copy.add_run(0, i * sendlen, sendlen, uint8_t(i), 1, 0);
+    copy.finish();
+    return MEGRAY_OK;
+}
+
+namespace {
+
+uint32_t common_width(uint64_t block_bytes, const void* const* a, const void* const* b, uint32_t n) {
+    uintptr_t bits = uintptr_t(block_bytes);
+    for (uint32_t r = 0; r < n; ++r) bits |= reinterpret_cast<uintptr_t>(a[r]) | reinterpret_cast<uintptr_t>(b[r]);
+    uint32_t width = kVecBytes;
+    while (width > 1 && (bits & (width - 1))) width >>= 1;
+    return width;
+}
+
+Status add_pack(Plan& plan, const void* const* in, void* const* out, uint32_t nranks, uint64_t block_bytes,
+                uint32_t mode, uint32_t root, uint32_t ncopies) {
+    if (!block_bytes) return MEGRAY_OK;
+    Step step;
+    std::memset(&step, 0, sizeof(step));
+    step.kind = Step::kPack;
+    PackLaunch& L = step.pack;
+    const void* out_c[kMaxRanks];
+    for (uint32_t r = 0; r < nranks; ++r) {
+        L.in[r] = in[r];
+        L.out[r] = out[r];
+        out_c[r] = out[r];
+    }
+    L.block_bytes = block_bytes;
+    L.nranks = nranks;
+    L.mode = mode;
+    L.root = root;
+    L.ncopies = ncopies;
+    L.width = common_width(block_bytes, in, out_c, nranks);
+    L.unroll = pack_unroll();
+    const uint64_t per_tile = uint64_t(kThreads) * L.unroll * L.width;
+    const uint64_t tiles = (block_bytes + per_tile - 1) / per_tile;
+    if (tiles * ncopies > 0x7fffffffull) return invalid("block too large for one pack launch");
+    L.tiles_per_copy = uint32_t(tiles);
+    plan.steps.push_back(step);
+    plan.bytes_read += block_bytes * ncopies;
+    plan.bytes_written += block_bytes * ncopies;
+    return MEGRAY_OK;
+}
+
+}  // namespace
+
+Status plan_all_to_all(Plan& plan, const void* const* send, void* const* recv, uint32_t nranks,
+                       uint64_t len, uint32_t elem_size) {
+    PLAN_TRY(check_ranks(nranks));
+    PLAN_TRY(check_elem(elem_size));
+    const uint64_t bytes = len * nranks * elem_size;
+    for (uint32_t a = 0; a < nranks; ++a) {
+        for (uint32_t b = 0; b < nranks; ++b) {
+            if (a < b && overlaps(recv[a], bytes, recv[b], bytes)) return invalid("receive buffers of two ranks overlap");
+            if (overlaps(recv[a], bytes, send[b], bytes)) return invalid("all_to_all cannot run in place");
+        }
+    }
+    return add_pack(plan, send, recv, nranks, len * elem_size, kPackAllToAll, 0, nranks * nranks);
+}
+
+Status plan_scatter(Plan& plan, const void* send_root, void* const* recv, uint32_t nranks, uint64_t recvlen,
+                    uint32_t elem_size, uint32_t root) {
+    PLAN_TRY(check_ranks(nranks));
+    PLAN_TRY(check_elem(elem_size));
+    if (root >= nranks) return invalid("root out of range");
+    const uint64_t block = recvlen * elem_size;
+    for (uint32_t a = 0; a < nranks; ++a) {
+        for (uint32_t b = a + 1; b < nranks; ++b)
+            if (overlaps(recv[a], block, recv[b], block)) return invalid("receive buffers of two ranks overlap");
+        if (overlaps(recv[a], block, send_root, block * nranks)) {
+            const bool in_place = a == root && static_cast<const char*>(recv[a]) ==
+                                                       static_cast<const char*>(send_root) + root * block;
+            if (!in_place) return invalid("a receive buffer overlaps the root's send buffer out of place");
+        }
+    }
+    const void* in[kMaxRanks] = {};
+    in[root] = send_root;
+    return add_pack(plan, in, recv, nranks, block, kPackScatter, root, nranks);
+}
+
+Status plan_gather(Plan& plan, const void* const* send, void* recv_root, uint32_t nranks, uint64_t sendlen,
+                   uint32_t elem_size, uint32_t root) {
+    PLAN_TRY(check_ranks(nranks));
+    PLAN_TRY(check_elem(elem_size));
+    if (root >= nranks) return invalid("root out of range");
+    const uint64_t block = sendlen * elem_size;
+    for (uint32_t b = 0; b < nranks; ++b) {
+        if (overlaps(recv_root, block * nranks, send[b], block)) {
+            const bool in_place = b == root && static_cast<const char*>(send[b]) ==
+                                                       static_cast<const char*>(recv_root) + root * block;
+            if (!in_place) return invalid("the root's receive buffer overlaps a send buffer out of place");
+        }
+    }
+    void* out[kMaxRanks] = {};
+    out[root] = recv_root;
+    return add_pack(plan, send, out, nranks, block, kPackGather, root, nranks);
+}
+
+Status plan_broadcast(Plan& plan, const void* send_root, void* const* recv, uint32_t nranks, uint64_t len,
+                      uint32_t elem_size, uint32_t root) {
+    PLAN_TRY(check_ranks(nranks));
+    PLAN_TRY(check_elem(elem_size));
+    if (root >= nranks) return invalid("root out of range");
+    const uint64_t bytes = len * elem_size;
+    for (uint32_t a = 0; a < nranks; ++a) {
+        for (uint32_t b = a + 1; b < nranks; ++b)
+            if (overlaps(recv[a], bytes, recv[b], bytes)) return invalid("receive buffers of two ranks overlap");
+        if (overlaps(recv[a], bytes, send_root, bytes) && !(a == root && recv[a] == send_root))
+            return invalid("a receive buffer overlaps the root's send buffer out of place");
+    }
+    const void* in[kMaxRanks] = {};
+    in[root] = send_root;
+    FoldBuilder copy(plan, in, recv, nranks, 1, nranks, elem_size, false);
+    copy.add_run(0, 0, len, uint8_t(root), 1, 0);
+    copy.finish();
+    return MEGRAY_OK;
+}
+
+Status plan_reduce2(Plan& plan, const void* i0, const void* i1, void* o, uint64_t len, uint32_t elem_size) {
+    PLAN_TRY(check_elem(elem_size));
+    const uint64_t bytes = len * elem_size;
+    if ((overlaps(o, bytes, i0, bytes) && o != i0) || (overlaps(o, bytes, i1, bytes) && o != i1))
+        return invalid("the output overlaps an input out of place");
+    const void* in[kMaxRanks] = {i0, i1};
+    void* out[kMaxRanks] = {o};
+    // (i0 OP i1) with ties / unordered -> i1: i1 seeds the accumulator, i0 is folded in
+    FoldBuilder fold(plan, in, out, 2, 2, 1, elem_size, false);
+    fold.add_run(0, 0, len, 1, 1, 0);
+    fold.finish();
+    return MEGRAY_OK;
+}
+
+}  // namespace vrank
+}  // namespace MegRay

@@ -1,0 +1,85 @@
+// Shared between the host planner and the gfx950 kernels: launch descriptors for the
+// virtual-rank collectives.  Everything here is plain data that travels as a kernel argument.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+
+namespace MegRay {
+namespace vrank {
+
+constexpr uint32_t kMaxRanks = 16;            // virtual ranks per group
+constexpr uint32_t kMaxChunks = 2 * kMaxRanks;  // the shm order splits a buffer into 2N chunks
+constexpr uint32_t kMaxSegments = 3 * kMaxChunks;  // head / aligned body / tail per chunk
+constexpr uint32_t kThreads = 256;            // workgroup size: four 64-wide wavefronts
+constexpr uint32_t kVecBytes = 16;            // one 128-bit global load / store per lane
+
+enum SegmentFlags : uint8_t {
+    kSegVector = 1,  // tile is walked in 16-byte vectors; begin offsets are vector aligned
+};
+
+// A run of elements that all share one fold order and one set of destinations.
+struct FoldSegment {
+    uint64_t in_begin;    // first element, same index in every input buffer
+    uint64_t out_begin;   // first element in every output buffer
+    uint64_t count;       // elements
+    uint32_t first_tile;  // tiles of all earlier segments
+    uint8_t start;        // rank whose buffer seeds the accumulator
+    int8_t dir;           // +1: start, start+1, ...   -1: start, start-1, ...   (mod nranks)
+    uint8_t out_first;    // destinations are ranks out_first .. out_first+nout-1 (mod nranks)
+    uint8_t flags;
+};
+
+// One launch of the fold kernel: every output element is a left fold, in a fixed order, over the
+// same element of `nfold` input buffers, written to `nout` output buffers.
+struct FoldLaunch {
+    const void* in[kMaxRanks];
+    void* out[kMaxRanks];
+    FoldSegment seg[kMaxSegments];
+    uint32_t nranks;         // modulus of the rank rotation
+    uint32_t nfold;          // inputs folded per element (1 = plain copy)
+    uint32_t nout;           // destinations per element
+    uint32_t nseg;
+    uint32_t total_tiles;
+    uint32_t new_wins_ties;  // float MAX/MIN: an equal / unordered compare keeps the newcomer
+    uint32_t unroll;         // vectors (or elements) per lane per tile; fixes the tile size
+    uint32_t elem_size;
+};
+
+enum PackMode : uint32_t {
+    kPackAllToAll = 0,  // copy b = i*N + j : in[i] block j  -> out[j] block i
+    kPackScatter = 1,   // copy b = i       : in[root] block i -> out[i] block 0
+    kPackGather = 2,    // copy b = i       : in[i] block 0    -> out[root] block i
+};
+
+// One launch of the pack kernel: `ncopies` equally sized block copies whose endpoints follow
+// arithmetically from the copy index.
+struct PackLaunch {
+    const void* in[kMaxRanks];
+    void* out[kMaxRanks];
+    uint64_t block_bytes;
+    uint32_t nranks;
+    uint32_t mode;
+    uint32_t root;
+    uint32_t ncopies;
+    uint32_t tiles_per_copy;
+    uint32_t width;   // bytes per lane access: 16, 8, 4, 2 or 1
+    uint32_t unroll;  // accesses per lane per tile
+};
+
+// Vectors (or elements) each lane moves per tile.  The kernels are instantiated with these values;
+// the planner sizes its tiles with the same function.
+constexpr uint32_t fold_unroll(uint32_t nfold) {
+    return nfold == 1 ? 4u : nfold == 2 ? 4u : (nfold == 3 || nfold == 4) ? 2u : 1u;
+}
+constexpr uint32_t pack_unroll() {
+    return 4u;
+}
+
+inline uint64_t tile_elems(const FoldLaunch& L, bool vector) {
+    uint64_t per_lane = vector ? (kVecBytes / L.elem_size) : 1;
+    return uint64_t(kThreads) * L.unroll * per_lane;
+}
+
+}  // namespace vrank
+}  // namespace MegRay

@@ -1,0 +1,284 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle on the same seeded
+inputs.  Bar: bit-exact for every dtype, including fp32/fp64 SUM under the reference's rank order
+and FLOAT16 (fp32 accumulation, one rounding; the stated tolerance is 1 ulp, the check is exact).
+"""
+import numpy as np
+import pytest
+
+import oracle as orc
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+import megray_amd as mr  # noqa: E402
+from gpu_util import (bits_equal, empty_device, first_mismatch, rand_array, to_device,  # noqa: E402
+                      to_host)
+
+REDUCE_TYPES = [orc.INT8, orc.UINT8, orc.INT32, orc.UINT32, orc.INT64, orc.UINT64, orc.FLOAT16,
+                orc.FLOAT32, orc.FLOAT64]
+OPS = [orc.SUM, orc.MAX, orc.MIN]
+ORDERS = [orc.ORDER_UCX, orc.ORDER_SHM, orc.ORDER_RANK0]
+
+
+def assert_same(got, want, what):
+    if not bits_equal(got, want):
+        raise AssertionError(f"{what}: first mismatch (index, got, want, count) = {first_mismatch(got, want)}")
+
+
+def run_all_reduce(ins, dtype, op, order, sched, offsets=None, inplace=False):
+    n = len(ins)
+    size = orc.dtype_size(dtype)
+    offsets = offsets or [0] * n
+    d_in = [to_device(x, offsets[r]) for r, x in enumerate(ins)]
+    d_out = d_in if inplace else [empty_device(ins[0].size * size, offsets[r]) for r in range(n)]
+    mr.all_reduce(d_in, d_out, ins[0].size, dtype, op, order, sched)
+    torch.cuda.synchronize()
+    return [to_host(o, ins[0].dtype) for o in d_out]
+
+
+@pytest.mark.parametrize("dtype", REDUCE_TYPES)
+@pytest.mark.parametrize("nranks", [1, 2, 3, 4, 5, 8, 16])
+def test_all_reduce_fused_all_orders(dtype, nranks):
+    rng = np.random.default_rng(1000 * dtype + nranks)
+    for length in (0, 1, nranks + 1, 1027, 8 * 4096 + 3, 70001):
+        ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+        for op in OPS:
+            for order in ORDERS:
+                want = orc.fold_all_reduce(ins, dtype, op, order)
+                got = run_all_reduce(ins, dtype, op, order, mr.Schedule.FUSED)
+                for r in range(nranks):
+                    assert_same(got[r], want[r], f"all_reduce dtype={dtype} N={nranks} len={length} op={op} "
+                                                 f"order={order} rank={r}")
+
+
+@pytest.mark.parametrize("dtype", [orc.INT8, orc.INT32, orc.FLOAT32, orc.FLOAT64, orc.UINT64])
+def test_all_reduce_equals_literal_ring_replay(dtype):
+    """Against the oracle's literal replay of src/ucx/all_reduce.cpp, not only its fold form."""
+    rng = np.random.default_rng(dtype)
+    for nranks in (2, 3, 4, 8):
+        for length in (nranks * 1000 + 7, 13):
+            ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+            for op in OPS:
+                want = orc.ucx_all_reduce(ins, dtype, op)
+                for sched in (mr.Schedule.FUSED, mr.Schedule.TWO_PHASE, mr.Schedule.RING):
+                    got = run_all_reduce(ins, dtype, op, orc.ORDER_UCX, sched)
+                    for r in range(nranks):
+                        assert_same(got[r], want[r], f"dtype={dtype} N={nranks} len={length} op={op} sched={sched}")
+                if dtype in (orc.INT8, orc.INT32, orc.FLOAT32):
+                    want = orc.shm_all_reduce(ins, dtype, op)
+                    for sched in (mr.Schedule.FUSED, mr.Schedule.TWO_PHASE):
+                        got = run_all_reduce(ins, dtype, op, orc.ORDER_SHM, sched)
+                        for r in range(nranks):
+                            assert_same(got[r], want[r], f"shm dtype={dtype} N={nranks} op={op} sched={sched}")
+
+
+def test_all_reduce_in_place_and_misaligned():
+    rng = np.random.default_rng(77)
+    for dtype in (orc.FLOAT32, orc.INT8, orc.FLOAT16, orc.INT64):
+        size = orc.dtype_size(dtype)
+        for nranks in (3, 8):
+            ins = [rand_array(dtype, 5000 + nranks, rng) for _ in range(nranks)]
+            want = orc.fold_all_reduce(ins, dtype, orc.SUM, orc.ORDER_UCX)
+            scheds = [mr.Schedule.FUSED, mr.Schedule.TWO_PHASE]
+            if dtype == orc.FLOAT16:  # a ring hop would round to fp16 every time
+                with pytest.raises(mr.MegRayError, match="ring schedule"):
+                    run_all_reduce(ins, dtype, orc.SUM, orc.ORDER_UCX, mr.Schedule.RING)
+            else:
+                scheds.append(mr.Schedule.RING)
+            for sched in scheds:
+                got = run_all_reduce(ins, dtype, orc.SUM, orc.ORDER_UCX, sched, inplace=True)
+                for r in range(nranks):
+                    assert_same(got[r], want[r], f"in-place dtype={dtype} sched={sched}")
+                # every rank buffer off 16-byte alignment by a different element count
+                offs = [size * (1 + r % 3) for r in range(nranks)]
+                got = run_all_reduce(ins, dtype, orc.SUM, orc.ORDER_UCX, sched, offsets=offs)
+                for r in range(nranks):
+                    assert_same(got[r], want[r], f"misaligned dtype={dtype} sched={sched}")
+
+
+def test_float_special_values_and_tie_conventions():
+    """+-0, NaN, inf and denormals through MAX/MIN/SUM: compare + select must follow the reference's
+    ?: (src/ucx/kernel.cu:24-38), not the hardware's max/min."""
+    n = 4
+    base = np.array([0.0, -0.0, np.nan, 1.0, -1.0, np.inf, -np.inf, 1e-45, -1e-45, 3e38, -3e38, 2.5],
+                    dtype=np.float64)
+    rng = np.random.default_rng(3)
+    for dtype in (orc.FLOAT32, orc.FLOAT64, orc.FLOAT16):
+        npdt = orc.NP_DTYPE[dtype]
+        with np.errstate(over="ignore", under="ignore"):
+            vals = base.astype(npdt)
+        ins = [rng.choice(vals, size=4096 + 5).astype(npdt) for _ in range(n)]
+        for op in OPS:
+            for order in ORDERS:
+                want = orc.fold_all_reduce(ins, dtype, op, order)[0]
+                got = run_all_reduce(ins, dtype, op, order, mr.Schedule.FUSED)[0]
+                nan = np.isnan(want)
+                assert np.array_equal(np.isnan(got), nan), f"NaN placement dtype={dtype} op={op} order={order}"
+                assert_same(got[~nan], want[~nan], f"specials dtype={dtype} op={op} order={order}")
+            rs_in = [x[:4096] for x in ins]
+            want = orc.fold_reduce_scatter(rs_in, dtype, op, orc.ORDER_UCX)
+            d_in = [to_device(x) for x in rs_in]
+            d_out = [empty_device(1024 * orc.dtype_size(dtype)) for _ in range(n)]
+            mr.reduce_scatter(d_in, d_out, 1024, dtype, op)
+            torch.cuda.synchronize()
+            for r in range(n):
+                got = to_host(d_out[r], npdt)
+                nan = np.isnan(want[r])
+                assert np.array_equal(np.isnan(got), nan)
+                assert_same(got[~nan], want[r][~nan], f"reduce_scatter specials dtype={dtype} op={op}")
+
+
+@pytest.mark.parametrize("dtype", REDUCE_TYPES)
+def test_reduce_scatter(dtype):
+    rng = np.random.default_rng(50 + dtype)
+    size = orc.dtype_size(dtype)
+    for nranks in (1, 2, 3, 8):
+        for recvlen in (0, 1, 5, 1024, 4099):
+            ins = [rand_array(dtype, nranks * recvlen, rng) for _ in range(nranks)]
+            for op in OPS:
+                for order in ORDERS:
+                    want = orc.fold_reduce_scatter(ins, dtype, op, order)
+                    d_in = [to_device(x) for x in ins]
+                    d_out = [empty_device(recvlen * size) for _ in range(nranks)]
+                    mr.reduce_scatter(d_in, d_out, recvlen, dtype, op, order)
+                    torch.cuda.synchronize()
+                    for r in range(nranks):
+                        assert_same(to_host(d_out[r], ins[0].dtype), want[r],
+                                    f"reduce_scatter dtype={dtype} N={nranks} recvlen={recvlen} op={op} order={order}")
+            if dtype in (orc.INT32, orc.FLOAT32, orc.FLOAT64) and recvlen:
+                want = orc.ucx_reduce_scatter(ins, dtype, orc.SUM)  # the literal replay
+                d_in = [to_device(x) for x in ins]
+                d_out = [empty_device(recvlen * size) for _ in range(nranks)]
+                mr.reduce_scatter(d_in, d_out, recvlen, dtype, orc.SUM)
+                torch.cuda.synchronize()
+                for r in range(nranks):
+                    assert_same(to_host(d_out[r], ins[0].dtype), want[r], "reduce_scatter vs literal replay")
+
+
+COPY_TYPES = [orc.UINT8, orc.FLOAT16, orc.FLOAT32, orc.INT64, orc.CHAR]
+
+
+@pytest.mark.parametrize("dtype", COPY_TYPES)
+def test_pack_collectives(dtype):
+    rng = np.random.default_rng(90 + dtype)
+    size = orc.dtype_size(dtype)
+    gen = orc.UINT8 if dtype == orc.CHAR else dtype
+    for nranks in (1, 2, 3, 8, 16):
+        for length in (0, 1, 6, 1000, 4096 + 3):
+            for misalign in (0, size):
+                ins = [rand_array(gen, nranks * length, rng) for _ in range(nranks)]
+                npdt = ins[0].dtype
+                # all_to_all
+                want = orc.ucx_all_to_all(ins, dtype)
+                d_in = [to_device(x, misalign) for x in ins]
+                d_out = [empty_device(nranks * length * size, misalign) for _ in range(nranks)]
+                mr.all_to_all(d_in, d_out, length, dtype)
+                torch.cuda.synchronize()
+                for r in range(nranks):
+                    assert_same(to_host(d_out[r], npdt), want[r], f"all_to_all dtype={dtype} N={nranks} len={length}")
+                # all_gather
+                parts = [x[:length] for x in ins]
+                want = orc.ucx_all_gather(parts, dtype)
+                d_in = [to_device(x, misalign) for x in parts]
+                d_out = [empty_device(nranks * length * size, misalign) for _ in range(nranks)]
+                mr.all_gather(d_in, d_out, length, dtype)
+                torch.cuda.synchronize()
+                for r in range(nranks):
+                    assert_same(to_host(d_out[r], npdt), want[r], f"all_gather dtype={dtype} N={nranks} len={length}")
+                root = nranks // 2
+                # scatter: only the root has a send buffer
+                want = orc.ucx_scatter([ins[root] if r == root else None for r in range(nranks)], dtype, root)
+                d_root = to_device(ins[root], misalign)
+                d_out = [empty_device(length * size, misalign) for _ in range(nranks)]
+                mr.scatter(d_root, d_out, length, dtype, root)
+                torch.cuda.synchronize()
+                for r in range(nranks):
+                    assert_same(to_host(d_out[r], npdt), want[r], f"scatter dtype={dtype} N={nranks} len={length}")
+                # gather: only the root has a receive buffer
+                want = orc.ucx_gather(parts, dtype, root)[root]
+                d_in = [to_device(x, misalign) for x in parts]
+                d_root = empty_device(nranks * length * size, misalign)
+                mr.gather(d_in, d_root, length, dtype, root)
+                torch.cuda.synchronize()
+                assert_same(to_host(d_root, npdt), want, f"gather dtype={dtype} N={nranks} len={length}")
+                # broadcast
+                want = orc.ucx_broadcast(parts, dtype, root)
+                d_root = to_device(parts[root], misalign)
+                d_out = [empty_device(length * size, misalign) for _ in range(nranks)]
+                mr.broadcast(d_root, d_out, length, dtype, root)
+                torch.cuda.synchronize()
+                for r in range(nranks):
+                    assert_same(to_host(d_out[r], npdt), want[r], f"broadcast dtype={dtype} N={nranks} len={length}")
+
+
+@pytest.mark.parametrize("dtype", REDUCE_TYPES)
+def test_two_input_reduce(dtype):
+    """mrv_reduce against the oracle's restatement of MegRay::reduce (src/ucx/kernel.cu:60-98)."""
+    rng = np.random.default_rng(dtype)
+    size = orc.dtype_size(dtype)
+    for length in (0, 1, 255, 4096, 100003):
+        a, b = rand_array(dtype, length, rng), rand_array(dtype, length, rng)
+        for op in OPS:
+            if dtype == orc.FLOAT16:  # the reference has no FLOAT16 reduce: fp32 arithmetic, one rounding
+                with np.errstate(over="ignore"):
+                    a32, b32 = a.astype(np.float32), b.astype(np.float32)
+                    want = {orc.SUM: (a32 + b32), orc.MAX: np.where(a32 > b32, a32, b32),
+                            orc.MIN: np.where(a32 < b32, a32, b32)}[op].astype(np.float16)
+            else:
+                want = orc.reduce_ucx(a, b, dtype, op)
+            d_a, d_b = to_device(a), to_device(b)
+            d_o = empty_device(length * size)
+            mr.reduce(d_a, d_b, d_o, length, dtype, op)
+            torch.cuda.synchronize()
+            assert_same(to_host(d_o, a.dtype), want, f"reduce dtype={dtype} len={length} op={op}")
+            # in place on the first operand, as every reference caller uses it
+            mr.reduce(d_a, d_b, d_a, length, dtype, op)
+            torch.cuda.synchronize()
+            assert_same(to_host(d_a, a.dtype), want, f"reduce in place dtype={dtype} len={length} op={op}")
+
+
+def test_reference_closed_forms_on_gpu():
+    """The reference's own test vectors (test/test_opr.cpp:286-359, 361-438, 198-257)."""
+    n, length = 3, 10
+    ins = [np.array([(i + 1) * (j + 1) for j in range(length)], dtype=np.float32) for i in range(n)]
+    j1 = np.arange(1, length + 1, dtype=np.float32)
+    for op, want in ((orc.SUM, 6 * j1), (orc.MAX, 3 * j1), (orc.MIN, j1)):
+        for order in ORDERS:
+            for r, got in enumerate(run_all_reduce(ins, orc.FLOAT32, op, order, mr.Schedule.FUSED)):
+                assert np.array_equal(got, want)
+    recvlen = 10
+    ins = [np.array([(i + 1) * (m + 1) for m in range(n * recvlen)], dtype=np.float32) for i in range(n)]
+    for op, factor in ((orc.SUM, 6), (orc.MAX, 3), (orc.MIN, 1)):
+        d_in = [to_device(x) for x in ins]
+        d_out = [empty_device(recvlen * 4) for _ in range(n)]
+        mr.reduce_scatter(d_in, d_out, recvlen, orc.FLOAT32, op)
+        torch.cuda.synchronize()
+        for k in range(n):
+            want = np.array([factor * (k * recvlen + j + 1) for j in range(recvlen)], dtype=np.float32)
+            assert np.array_equal(to_host(d_out[k], np.float32), want)
+    length = 6
+    ins = [np.array([(i + 1) * (j + 2) * (k + 3) for j in range(n) for k in range(length)], dtype=np.float32)
+           for i in range(n)]
+    d_in = [to_device(x) for x in ins]
+    d_out = [empty_device(n * length * 4) for _ in range(n)]
+    mr.all_to_all(d_in, d_out, length, orc.FLOAT32)
+    torch.cuda.synchronize()
+    for j in range(n):
+        want = np.array([(i + 1) * (j + 2) * (k + 3) for i in range(n) for k in range(length)], dtype=np.float32)
+        assert np.array_equal(to_host(d_out[j], np.float32), want)
+
+
+def test_errors_follow_the_reference():
+    d = to_device(np.zeros(64, dtype=np.float32))
+    o = empty_device(256)
+    with pytest.raises(mr.MegRayError, match="unknown dtype"):      # src/ucx/kernel.cu:95-96
+        mr.reduce(d, d, o, 64, mr.DType.CHAR, mr.ReduceOp.SUM)
+    with pytest.raises(mr.MegRayError, match="unknown dtype"):
+        mr.all_reduce([d], [o], 64, 17, mr.ReduceOp.SUM)
+    with pytest.raises(mr.MegRayError, match="unknown reduce op"):  # src/ucx/kernel.cu:55-56
+        mr.all_reduce([d], [o], 64, mr.DType.FLOAT32, 3)
+    with pytest.raises(mr.MegRayError, match="overlap"):
+        mr.all_reduce([d, d], [o, o], 64, mr.DType.FLOAT32, mr.ReduceOp.SUM)
+    with pytest.raises(mr.MegRayError, match="nranks"):
+        mr.all_reduce([d] * 17, [o] * 17, 1, mr.DType.FLOAT32, mr.ReduceOp.SUM)
+    torch.cuda.synchronize()
