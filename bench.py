@@ -1,0 +1,250 @@
+#!/usr/bin/env python3
+"""Headline benchmark: 8 virtual ranks x 2^28 fp32 SUM all_reduce on one MI355X.
+
+A "step" is one whole all_reduce (every rank's 1 GiB buffer read, every rank's result written)
+with all buffers already resident in HBM.  Prints ONE JSON line:
+
+  value      achieved HBM GB/s of the collective = B_min / t, B_min = 2 * N * n * 4 bytes (each
+             input read once, each output written once; the fused schedule executes exactly that)
+  roofline   the fold kernel against the 8 TB/s HBM peak, timed with HIP events on the launch stream
+  cpu_baseline  the reference tests' expected-value loop (test/test_opr.cpp:321-330) re-stated in the
+             CPU oracle, timed on this host on a bounded sample of the same workload
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--log2n 28] [--no-cpu] [--no-small]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+BASE_SEED = 0x4D656752  # "MegR"; rank r draws from seed BASE_SEED + r
+
+# HBM bytes per launch of the fold kernel on the headline workload, from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs scaled by the same counters on a plain copy of known size; the
+# summaries those figures come from are kept as text next to the kernel-trace summaries.
+# None until measured.
+MEASURED_TRAFFIC_BYTES = {"all_reduce_f32_n8_2p28_fused": None}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--log2n", type=int, default=28, help="elements per rank = 2^log2n")
+    ap.add_argument("--ranks", type=int, default=8)
+    ap.add_argument("--schedule", default="fused", choices=["fused", "two_phase", "ring"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-small", action="store_true", help="skip the small-message sweep")
+    ap.add_argument("--no-check", action="store_true", help="skip the correctness checks")
+    return ap.parse_args()
+
+
+def make_inputs(torch, nranks, n):
+    ins = []
+    for r in range(nranks):
+        g = torch.Generator(device="cuda:0")
+        g.manual_seed(BASE_SEED + r)
+        t = torch.rand(n, generator=g, device="cuda:0", dtype=torch.float32)
+        t.mul_(2.0).sub_(1.0)  # uniform[-1, 1)
+        ins.append(t)
+    return ins
+
+
+def check_small(torch, mr, orc, np):
+    """Full bit compare against the oracle's literal ring replay at a size the CPU finishes fast."""
+    nranks, n = 8, (1 << 20) + 5
+    ins = make_inputs(torch, nranks, n)
+    outs = [torch.empty_like(t) for t in ins]
+    mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream=torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    host = [t.cpu().numpy() for t in ins]
+    want = orc.ucx_all_reduce(host, orc.FLOAT32, orc.SUM)
+    for r in range(nranks):
+        got = outs[r].cpu().numpy()
+        if not np.array_equal(got.view(np.uint32), want[r].view(np.uint32)):
+            raise SystemExit("bench: all_reduce differs from the oracle at n=2^20+5")
+
+
+def check_full(torch, mr, ins, outs, n):
+    """Size-independent checks at the full size: every rank holds the same bits, and the fused
+    result equals the 2(N-1)-step ring replay of the reference schedule run on the device."""
+    for r in range(1, len(outs)):
+        if not torch.equal(outs[0].view(torch.int32), outs[r].view(torch.int32)):
+            raise SystemExit(f"bench: rank {r} differs from rank 0")
+    ref = outs[0].clone()
+    mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, schedule=mr.Schedule.RING,
+                  stream=torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    if not torch.equal(ref.view(torch.int32), outs[len(outs) // 2].view(torch.int32)):
+        raise SystemExit("bench: fused schedule differs from the ring replay")
+
+
+def small_message_sweep(torch, mr):
+    """all_reduce SUM fp32, 8 ranks, 4 KiB .. 1 MiB per rank: microseconds per collective, issued
+    back to back on one stream (throughput latency) and one at a time with a host sync (round trip)."""
+    out = {}
+    st = torch.cuda.current_stream()
+    for nbytes in (4096, 16384, 65536, 262144, 1048576):
+        n = nbytes // 4
+        ins = make_inputs(torch, 8, n)
+        outs = [torch.empty_like(t) for t in ins]
+        for _ in range(100):
+            mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream=st)
+        torch.cuda.synchronize()
+        iters = 1000
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(st)
+        for _ in range(iters):
+            mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream=st)
+        e1.record(st)
+        torch.cuda.synchronize()
+        stream_us = e0.elapsed_time(e1) * 1000.0 / iters
+        lat = []
+        for _ in range(300):
+            t0 = time.perf_counter()
+            mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream=st)
+            torch.cuda.synchronize()
+            lat.append((time.perf_counter() - t0) * 1e6)
+        lat.sort()
+        out[str(nbytes)] = {"stream_us": round(stream_us, 2), "sync_median_us": round(lat[len(lat) // 2], 2),
+                            "sync_p99_us": round(lat[int(len(lat) * 0.99)], 2)}
+    return out
+
+
+def cpu_baseline(orc, np, nranks):
+    """The reference tests' expected-value loop on the host: single thread (as the reference runs
+    it) on a 2^25-element-per-rank sample of the headline workload, plus the same loop split over
+    all host cores for scale."""
+    n = 1 << 25
+    rng = np.random.default_rng(BASE_SEED)
+    ins = [rng.random(n, dtype=np.float32) * 2 - 1 for _ in range(nranks)]
+    bmin = 2 * nranks * n * 4
+
+    def timed(threads, reps):
+        orc.test_all_reduce_f32(ins, orc.SUM, nthreads=threads)  # warm-up, touches the outputs
+        times = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            orc.test_all_reduce_f32(ins, orc.SUM, nthreads=threads)
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        return times[len(times) // 2]
+
+    t1 = timed(0, 5)
+    cores = min(os.cpu_count() or 1, 16)
+    tn = timed(cores, 5)
+    return {
+        "value": round(bmin / t1 / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": f"all_reduce SUM fp32, {nranks} ranks x 2^25 elements, test/test_opr.cpp:321-330 loop, "
+                  f"median of 5, {t1 * 1e3:.1f} ms per pass",
+        "all_cores": {"value": round(bmin / tn / 1e9, 3), "cores": cores, "ms": round(tn * 1e3, 1)},
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; the N ranks are virtual ranks inside it "
+              "(use --gpus 1, rank count is --ranks)", file=sys.stderr)
+        return 2
+    import numpy as np
+    import torch
+
+    import megray_amd as mr
+    from megray_amd import _lib
+
+    _lib.load()  # fails loudly when the HIP library is not built
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    torch.cuda.set_device(0)
+    nranks, n = args.ranks, 1 << args.log2n
+    sched = {"fused": mr.Schedule.FUSED, "two_phase": mr.Schedule.TWO_PHASE, "ring": mr.Schedule.RING}[args.schedule]
+
+    if not args.no_check:
+        import oracle as orc
+        check_small(torch, mr, orc, np)
+
+    ins = make_inputs(torch, nranks, n)
+    outs = [torch.empty_like(t) for t in ins]
+    st = torch.cuda.current_stream()
+
+    def step():
+        mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, order=mr.FoldOrder.UCX, schedule=sched,
+                      stream=st)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(st)
+    for _ in range(args.steps):
+        step()
+    e1.record(st)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    event_ms = e0.elapsed_time(e1)
+
+    if not args.no_check:
+        check_full(torch, mr, ins, outs, n)
+
+    ms_per_step = wall * 1e3 / args.steps
+    bmin = 2 * nranks * n * 4
+    runs, bytes_read, bytes_written = mr.describe(mr.Collective.ALL_REDUCE, ins, outs, n, mr.DType.FLOAT32,
+                                                  mr.FoldOrder.UCX, sched)
+    launches = len({r["step"] for r in runs})
+    executed = bytes_read + bytes_written
+    value = bmin / (wall / args.steps) / 1e9
+    kernel_ms = event_ms / args.steps / launches  # average launch duration over the timed region
+    achieved = (executed / launches) / (kernel_ms * 1e-3) / 1e9
+    key = f"all_reduce_f32_n{nranks}_2p{args.log2n}_{args.schedule}"
+    result = {
+        "metric": "achieved HBM GB/s (% of peak) for 8-rank fp32 SUM all_reduce; small-msg µs",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic: uniform[-1,1) fp32, torch generator seeded 0x4D656752 + rank",
+        "config": {
+            "workload": f"all_reduce SUM fp32, {nranks} virtual ranks x 2^{args.log2n} elements, ucx ring order, "
+                        f"{args.schedule} schedule, buffers resident in HBM",
+            "ranks": nranks, "elements_per_rank": n, "order": "ucx", "schedule": args.schedule,
+            "launches_per_step": launches,
+        },
+        "pct_of_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "bytes_min": bmin,
+        "bytes_executed": executed,
+        "roofline": {
+            "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(key),
+            "kernel": "fold_kernel<float, SUM, K=8>" if args.schedule == "fused" else "fold_kernel (several)",
+            "kernel_ms": round(kernel_ms, 4), "algorithmic_bytes_per_launch": executed // launches,
+        },
+    }
+    del ins, outs
+    torch.cuda.empty_cache()
+    if not args.no_small:
+        result["small_msg_us"] = small_message_sweep(torch, mr)
+    if not args.no_cpu:
+        import oracle as orc
+        result["cpu_baseline"] = cpu_baseline(orc, np, nranks)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

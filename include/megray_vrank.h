@@ -157,11 +157,14 @@ typedef struct mrv_plan_run {
     uint32_t nfold;         /* fold: inputs combined per element (1 = copy) */
     uint32_t nout;          /* fold: destinations */
     uint32_t new_wins_ties; /* fold */
-    uint32_t vector;        /* fold: 1 = walked in 16-byte vectors; pack: bytes per lane access */
+    uint32_t vector;        /* fold: 0 = element by element, 1 = 16-byte vectors, 2 = run of a flat launch
+                               (vectors on the buffer's own 1 KiB tile grid); pack: bytes per lane access */
     uint32_t start;         /* fold: seed rank; pack: source rank */
     int32_t dir;            /* fold: +1 / -1 */
     uint32_t out_first;     /* fold: first destination rank; pack: destination rank */
-    uint32_t tiles;         /* workgroups this run occupies */
+    uint32_t tiles;         /* workgroups this run occupies (flat: those wholly inside it) */
+    uint32_t reads_recv;    /* 1 = the launch reads the receive buffers (a later step of a multi-launch plan) */
+    uint32_t reserved;
     uint64_t in_begin;      /* fold: first element in the inputs; pack: source byte offset */
     uint64_t out_begin;     /* fold: first element in the outputs; pack: destination byte offset */
     uint64_t count;         /* fold: elements; pack: bytes */

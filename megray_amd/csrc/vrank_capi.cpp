@@ -254,11 +254,40 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.start = sg.start;
                     run.dir = sg.dir;
                     run.out_first = sg.out_first;
-                    const uint32_t next = s + 1 < L.nseg ? L.seg[s + 1].first_tile : L.total_tiles;
-                    run.tiles = next - sg.first_tile;
+                    const uint32_t next = s + 1 < L.nseg ? L.first_tile[s + 1] : L.total_tiles;
+                    run.tiles = next - L.first_tile[s];
+                    run.reads_recv = (collective == MRV_ALL_REDUCE && sg.start < nranks && L.in[sg.start] == recvbuffs[sg.start] &&
+                                      L.in[sg.start] != sendbuffs[sg.start])
+                                             ? 1
+                                             : 0;
                     run.in_begin = sg.in_begin;
                     run.out_begin = sg.out_begin;
                     run.count = sg.count;
+                    emit(run);
+                }
+            } else if (step.kind == Step::kFlat) {
+                const FlatLaunch& L = step.flat;
+                for (uint32_t s = 0; s < L.nruns; ++s) {
+                    const FlatRun& fr = L.run[s];
+                    mrv_plan_run run;
+                    std::memset(&run, 0, sizeof(run));
+                    run.step = uint32_t(i);
+                    run.kind = 0;
+                    run.nfold = L.nranks;
+                    run.nout = L.nout;
+                    run.new_wins_ties = L.new_wins_ties;
+                    run.vector = 2;
+                    run.start = fr.start;
+                    run.dir = fr.dir;
+                    run.out_first = fr.out_first;
+                    run.tiles = L.tile_hi[s] - L.tile_lo[s];
+                    run.reads_recv = (collective == MRV_ALL_REDUCE && fr.start < nranks &&
+                                      L.in[fr.start] == recvbuffs[fr.start] && L.in[fr.start] != sendbuffs[fr.start])
+                                             ? 1
+                                             : 0;
+                    run.in_begin = fr.begin;
+                    run.out_begin = fr.begin - uint64_t(fr.out_shift);
+                    run.count = fr.end - fr.begin;
                     emit(run);
                 }
             } else {

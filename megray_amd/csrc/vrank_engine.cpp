@@ -34,6 +34,8 @@ Status execute(const Plan& plan, DType dtype, ReduceOp op, hipStream_t stream) {
     for (const Step& step : plan.steps) {
         if (step.kind == Step::kFold) {
             HIP_CHECK(launch_fold(step.fold, dtype, op, stream));
+        } else if (step.kind == Step::kFlat) {
+            HIP_CHECK(launch_flat(step.flat, dtype, op, stream));
         } else {
             HIP_CHECK(launch_pack(step.pack, stream));
         }

@@ -1,17 +1,21 @@
 // gfx950 kernels of the virtual-rank backend.
 //
-// fold_kernel  : every output element is a left fold, in a fixed rank order, over the same element
-//                of K input buffers, stored to M output buffers.  It replaces the 2-input
+// fold_kernel / fold_flat_kernel
+//              : every output element is a left fold, in a fixed rank order, over the same element
+//                of K input buffers, stored to M output buffers.  They replace the 2-input
 //                reduce_{sum,max,min}_kernel of the reference (src/ucx/kernel.cu:16-38) and the
 //                cpu_reduce_kernel loop (src/shm/utils.cpp:16-37): a whole ring of N-1 two-input
 //                steps on one chunk is one pass here, the ring order surviving as the fold order.
+//                fold_flat_kernel is the fast form for K == rank count on aligned buffers;
+//                fold_kernel takes everything else (any K, unaligned buffers, shifted copies).
 // pack_kernel  : equally sized block copies between rank buffers (all_to_all / scatter / gather),
 //                replacing the per-peer send/recv pairs of src/ucx/all_to_all.cpp:30-41,
 //                src/ucx/scatter.cpp:30-44 and src/ucx/gather.cpp:30-44.
 //
-// Both are pure streaming kernels: HBM-bound, one 128-bit access per lane per buffer, no LDS, no
-// matrix instructions.  A workgroup is four 64-wide wavefronts; a wavefront's lanes read
-// consecutive 16-byte vectors, so every load and store instruction covers one contiguous KiB.
+// All are pure streaming kernels: HBM-bound, one 128-bit access per lane per buffer, no LDS, no
+// matrix instructions.  A workgroup is ONE 64-wide wavefront whose lanes read consecutive 16-byte
+// vectors, so every load and store instruction covers one contiguous KiB and a tile is 1 KiB per
+// buffer: on MI355X many small tiles sustain more HBM bandwidth than fewer large ones.
 #include "vrank_kernels.h"
 
 #include <hip/hip_runtime.h>
@@ -136,13 +140,18 @@ __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
     using A = typename Wide<T>::type;
     constexpr uint32_t EPV = kVecBytes / sizeof(T);
     const uint32_t tile = blockIdx.x;
+    // segment lookup: first_tile is ascending and padded with 0xffffffff, so the segment is the
+    // number of entries <= tile, minus one; eight entries per scalar load
     uint32_t s = 0;
-    for (uint32_t i = 1; i < L.nseg; ++i)
-        if (L.seg[i].first_tile <= tile) s = i;
+    for (uint32_t base = 0; base < L.nseg; base += 8) {
+#pragma unroll
+        for (uint32_t i = 0; i < 8; ++i) s += L.first_tile[base + i] <= tile ? 1u : 0u;
+    }
+    s -= 1;
     const uint64_t in_begin = L.seg[s].in_begin;
     const uint64_t out_begin = L.seg[s].out_begin;
     const uint64_t count = L.seg[s].count;
-    const uint32_t local_tile = tile - L.seg[s].first_tile;
+    const uint32_t local_tile = tile - L.first_tile[s];
     const uint32_t start = L.seg[s].start;
     const int dir = L.seg[s].dir;
     const uint32_t out_first = L.seg[s].out_first;
@@ -254,6 +263,102 @@ __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Flat fold: tile t covers bytes [1024 t, 1024 t + 1024) of every input, whatever run it is in.
+// The K loads of a lane therefore depend on nothing but blockIdx and the kernel arguments and are
+// issued first; the run lookup (fold order, destinations) happens while they are in flight.
+
+template <typename T, int OP, int K, int START, int DIR>
+__device__ __forceinline__ u32x4 fold_static(const u32x4 (&x)[K], bool new_wins) {
+    AccFor<T, OP> acc;
+    acc.seed(x[START]);
+#pragma unroll
+    for (int j = 1; j < K; ++j) acc.fold(x[((START + DIR * j) % K + K) % K], new_wins);
+    return acc.finish();
+}
+
+// Uniform dispatch on the seed rank: each case is a straight-line fold with fixed registers.
+template <typename T, int OP, int K, int S = 0>
+__device__ __forceinline__ u32x4 fold_from(const u32x4 (&x)[K], uint32_t start, int dir, bool new_wins) {
+    if constexpr (S == K - 1) {
+        return dir > 0 ? fold_static<T, OP, K, S, 1>(x, new_wins) : fold_static<T, OP, K, S, -1>(x, new_wins);
+    } else {
+        if (start == S)
+            return dir > 0 ? fold_static<T, OP, K, S, 1>(x, new_wins) : fold_static<T, OP, K, S, -1>(x, new_wins);
+        return fold_from<T, OP, K, S + 1>(x, start, dir, new_wins);
+    }
+}
+
+template <typename T, int OP, int K>
+__global__ void __launch_bounds__(kThreads) fold_flat_kernel(const FlatLaunch L) {
+    using A = typename Wide<T>::type;
+    constexpr uint32_t EPV = kVecBytes / sizeof(T);
+    constexpr uint32_t TILE = kThreads * EPV;  // elements per tile
+    const uint32_t tile = blockIdx.x;
+    const uint32_t tid = threadIdx.x;
+    const uint64_t byte_off = (uint64_t(tile) * kThreads + tid) * kVecBytes;
+    const bool whole = (uint64_t(tile) + 1) * TILE <= L.count;  // tile lies inside the buffer
+
+    u32x4 x[K];
+    if (whole) {
+#pragma unroll
+        for (int r = 0; r < K; ++r) x[r] = load_vec(static_cast<const char*>(L.in[r]) + byte_off);
+    }
+
+    // run lookup, eight runs per pair of scalar loads
+    int run = -1;
+    for (uint32_t base = 0; base < L.nruns; base += 8) {
+#pragma unroll
+        for (uint32_t i = 0; i < 8; ++i)
+            if (tile >= L.tile_lo[base + i] && tile < L.tile_hi[base + i]) run = int(base + i);
+    }
+    const bool new_wins = L.new_wins_ties != 0;
+    const uint32_t nout = L.nout;
+
+    if (run >= 0) {
+        // the whole tile shares one fold order (and lies inside the buffer)
+        const uint32_t start = L.run[run].start;
+        const int dir = L.run[run].dir;
+        const uint32_t out_first = L.run[run].out_first;
+        const uint64_t out_off = byte_off - uint64_t(L.run[run].out_shift) * sizeof(T);
+        const u32x4 res = fold_from<T, OP, K>(x, start, dir, new_wins);
+        if (nout == uint32_t(K)) {
+#pragma unroll
+            for (int m = 0; m < K; ++m) store_vec(static_cast<char*>(L.out[m]) + out_off, res);
+        } else {
+            for (uint32_t m = 0; m < nout; ++m)
+                store_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, K)]) + out_off, res);
+        }
+        return;
+    }
+
+    // A tile that straddles a run border or the end of the buffer: element by element, one run at a
+    // time so that ranks and destinations stay uniform.
+    const uint64_t e_lo = uint64_t(tile) * TILE;
+    const uint64_t e_hi = e_lo + TILE < L.count ? e_lo + TILE : L.count;
+    for (uint32_t i = 0; i < L.nruns; ++i) {
+        const uint64_t b = L.run[i].begin > e_lo ? L.run[i].begin : e_lo;
+        const uint64_t e = L.run[i].end < e_hi ? L.run[i].end : e_hi;
+        if (b >= e) continue;
+        const uint32_t start = L.run[i].start;
+        const int dir = L.run[i].dir;
+        const uint32_t out_first = L.run[i].out_first;
+        const uint64_t shift = uint64_t(L.run[i].out_shift);
+        for (uint32_t k = 0; k < EPV; ++k) {
+            const uint64_t el = e_lo + uint64_t(tid) * EPV + k;
+            if (el < b || el >= e) continue;
+            A a = static_cast<A>(static_cast<const T*>(L.in[start])[el]);
+            for (uint32_t j = 1; j < uint32_t(K); ++j)
+                a = combine<OP, A>(a, static_cast<A>(static_cast<const T*>(L.in[rotate_rank(start, dir, j, K)])[el]),
+                                   new_wins);
+            const T r = static_cast<T>(a);
+            for (uint32_t m = 0; m < nout; ++m)
+                static_cast<T*>(L.out[rotate_rank(out_first, 1, m, K)])[el - shift] = r;
+        }
+    }
+}
+
 template <typename W>
 __device__ __forceinline__ W load_w(const char* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const W*>(p));
@@ -332,6 +437,25 @@ FoldFn pick_copy(uint32_t elem_size) {
     }
 }
 
+
+using FlatFn = void (*)(const FlatLaunch);
+
+template <typename T, int OP>
+FlatFn pick_flat(uint32_t nranks) {
+    switch (nranks) {
+        case 2: return fold_flat_kernel<T, OP, 2>;
+        case 3: return fold_flat_kernel<T, OP, 3>;
+        case 4: return fold_flat_kernel<T, OP, 4>;
+        case 8: return fold_flat_kernel<T, OP, 8>;
+        default: return nullptr;
+    }
+}
+
+template <typename T>
+FlatFn pick_flat_minmax(int op, uint32_t nranks) {
+    return op == kMax ? pick_flat<T, kMax>(nranks) : pick_flat<T, kMin>(nranks);
+}
+
 }  // namespace
 
 hipError_t launch_fold(const FoldLaunch& L, DType dtype, ReduceOp op, hipStream_t stream) {
@@ -369,6 +493,42 @@ hipError_t launch_fold(const FoldLaunch& L, DType dtype, ReduceOp op, hipStream_
     } else {
         return hipErrorInvalidValue;
     }
+    hipLaunchKernelGGL(fn, dim3(L.total_tiles), dim3(kThreads), 0, stream, L);
+    return hipGetLastError();
+}
+
+
+hipError_t launch_flat(const FlatLaunch& L, DType dtype, ReduceOp op, hipStream_t stream) {
+    if (L.total_tiles == 0) return hipSuccess;
+    FlatFn fn = nullptr;
+    if (op == MEGRAY_SUM) {
+        switch (dtype) {
+            case MEGRAY_INT8:
+            case MEGRAY_UINT8: fn = pick_flat<uint8_t, kSum>(L.nranks); break;
+            case MEGRAY_INT32:
+            case MEGRAY_UINT32: fn = pick_flat<uint32_t, kSum>(L.nranks); break;
+            case MEGRAY_INT64:
+            case MEGRAY_UINT64: fn = pick_flat<uint64_t, kSum>(L.nranks); break;
+            case MEGRAY_FLOAT16: fn = pick_flat<_Float16, kSum>(L.nranks); break;
+            case MEGRAY_FLOAT32: fn = pick_flat<float, kSum>(L.nranks); break;
+            case MEGRAY_FLOAT64: fn = pick_flat<double, kSum>(L.nranks); break;
+            default: return hipErrorInvalidValue;
+        }
+    } else if (op == MEGRAY_MAX || op == MEGRAY_MIN) {
+        switch (dtype) {
+            case MEGRAY_INT8: fn = pick_flat_minmax<int8_t>(op, L.nranks); break;
+            case MEGRAY_UINT8: fn = pick_flat_minmax<uint8_t>(op, L.nranks); break;
+            case MEGRAY_INT32: fn = pick_flat_minmax<int32_t>(op, L.nranks); break;
+            case MEGRAY_UINT32: fn = pick_flat_minmax<uint32_t>(op, L.nranks); break;
+            case MEGRAY_INT64: fn = pick_flat_minmax<int64_t>(op, L.nranks); break;
+            case MEGRAY_UINT64: fn = pick_flat_minmax<uint64_t>(op, L.nranks); break;
+            case MEGRAY_FLOAT16: fn = pick_flat_minmax<_Float16>(op, L.nranks); break;
+            case MEGRAY_FLOAT32: fn = pick_flat_minmax<float>(op, L.nranks); break;
+            case MEGRAY_FLOAT64: fn = pick_flat_minmax<double>(op, L.nranks); break;
+            default: return hipErrorInvalidValue;
+        }
+    }
+    if (!fn) return hipErrorInvalidValue;
     hipLaunchKernelGGL(fn, dim3(L.total_tiles), dim3(kThreads), 0, stream, L);
     return hipGetLastError();
 }

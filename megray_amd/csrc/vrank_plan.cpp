@@ -33,80 +33,159 @@ bool overlaps(const void* a, uint64_t a_bytes, const void* b, uint64_t b_bytes) 
     return a0 < b0 + b_bytes && b0 < a0 + a_bytes;
 }
 
-// Collects runs of elements into fold launches, splitting each run into an unaligned head, a body
-// of whole 16-byte vectors and a tail, and opening a new launch when a descriptor is full.
+// Collects runs of elements (one fold order, one destination set each) and turns them into
+// launches: one flat launch where the runs tile a buffer in order and everything is vector aligned,
+// general launches (runs split into an unaligned head, a body of whole 16-byte vectors and a tail,
+// a new launch whenever a descriptor fills up) otherwise.
 class FoldBuilder {
 public:
     FoldBuilder(Plan& plan, const void* const* in, void* const* out, uint32_t nranks, uint32_t nfold,
                 uint32_t nout, uint32_t elem_size, bool new_wins)
-            : m_plan(plan) {
-        std::memset(&m_launch, 0, sizeof(m_launch));
+            : m_plan(plan), m_nranks(nranks), m_nfold(nfold), m_nout(nout), m_elem(elem_size),
+              m_new_wins(new_wins) {
         m_aligned = true;
-        for (uint32_t r = 0; r < nranks; ++r) {
-            m_launch.in[r] = in[r];
-            m_launch.out[r] = out[r];
-            m_aligned = m_aligned && aligned16(in[r]) && aligned16(out[r]);  // null counts as aligned
+        for (uint32_t r = 0; r < kMaxRanks; ++r) {
+            m_in[r] = r < nranks ? in[r] : nullptr;
+            m_out[r] = r < nranks ? out[r] : nullptr;
+            m_aligned = m_aligned && aligned16(m_in[r]) && aligned16(m_out[r]);  // null counts as aligned
         }
-        m_launch.nranks = nranks;
-        m_launch.nfold = nfold;
-        m_launch.nout = nout;
-        m_launch.new_wins_ties = new_wins ? 1 : 0;
-        m_launch.unroll = fold_unroll(nfold);
-        m_launch.elem_size = elem_size;
     }
 
     void add_run(uint64_t in_begin, uint64_t out_begin, uint64_t count, uint8_t start, int8_t dir,
                  uint8_t out_first) {
         if (!count) return;
-        m_plan.bytes_read += count * m_launch.elem_size * m_launch.nfold;
-        m_plan.bytes_written += count * m_launch.elem_size * m_launch.nout;
-        const uint64_t epv = kVecBytes / m_launch.elem_size;
-        const bool vector = m_aligned && (in_begin % epv == out_begin % epv);
-        uint64_t head = 0, body = 0;
-        if (vector) {
-            head = std::min<uint64_t>((epv - in_begin % epv) % epv, count);
-            body = (count - head) / epv * epv;
-        }
-        if (!body) {
-            add_segment(in_begin, out_begin, count, start, dir, out_first, 0);
-            return;
-        }
-        const uint64_t tail = count - head - body;
-        if (head) add_segment(in_begin, out_begin, head, start, dir, out_first, 0);
-        add_segment(in_begin + head, out_begin + head, body, start, dir, out_first, kSegVector);
-        if (tail) add_segment(in_begin + head + body, out_begin + head + body, tail, start, dir, out_first, 0);
+        m_plan.bytes_read += count * m_elem * m_nfold;
+        m_plan.bytes_written += count * m_elem * m_nout;
+        m_runs.push_back(Run{in_begin, out_begin, count, start, dir, out_first});
     }
 
     void finish() {
+        if (m_runs.empty()) return;
+        if (!emit_flat()) emit_general();
+        m_runs.clear();
+    }
+
+private:
+    struct Run {
+        uint64_t in_begin, out_begin, count;
+        uint8_t start;
+        int8_t dir;
+        uint8_t out_first;
+    };
+
+    // The flat kernel folds exactly nranks inputs with the rank count known at compile time.
+    static bool flat_width(uint32_t n) { return n == 2 || n == 3 || n == 4 || n == 8; }
+
+    bool emit_flat() {
+        if (!m_aligned || m_nfold != m_nranks || !flat_width(m_nranks) || m_runs.size() > kMaxFlatRuns)
+            return false;
+        const uint64_t epv = kVecBytes / m_elem;
+        const uint64_t tile = uint64_t(kThreads) * epv;  // elements per tile
+        uint64_t expect = 0;
+        for (const Run& r : m_runs) {
+            if (r.in_begin != expect) return false;  // runs must tile [0, count) in order
+            if (r.out_begin > r.in_begin || (r.in_begin - r.out_begin) % epv) return false;
+            expect = r.in_begin + r.count;
+        }
+        const uint64_t total = (expect + tile - 1) / tile;
+        if (total > 0x7fffffffull) return false;
+        Step step;
+        std::memset(&step, 0, sizeof(step));
+        step.kind = Step::kFlat;
+        FlatLaunch& L = step.flat;
+        for (uint32_t r = 0; r < kMaxRanks; ++r) {
+            L.in[r] = m_in[r];
+            L.out[r] = m_out[r];
+        }
+        for (size_t i = 0; i < m_runs.size(); ++i) {
+            const Run& r = m_runs[i];
+            FlatRun& fr = L.run[i];
+            fr.begin = r.in_begin;
+            fr.end = r.in_begin + r.count;
+            fr.out_shift = int64_t(r.in_begin - r.out_begin);
+            fr.start = r.start;
+            fr.dir = r.dir;
+            fr.out_first = r.out_first;
+            const uint64_t lo = (fr.begin + tile - 1) / tile, hi = fr.end / tile;
+            L.tile_lo[i] = uint32_t(lo);
+            L.tile_hi[i] = uint32_t(hi > lo ? hi : lo);
+        }
+        L.count = expect;
+        L.nranks = m_nranks;
+        L.nout = m_nout;
+        L.nruns = uint32_t(m_runs.size());
+        L.total_tiles = uint32_t(total);
+        L.new_wins_ties = m_new_wins ? 1 : 0;
+        L.elem_size = m_elem;
+        m_plan.steps.push_back(step);
+        return true;
+    }
+
+    void emit_general() {
+        open_launch();
+        const uint64_t epv = kVecBytes / m_elem;
+        for (const Run& r : m_runs) {
+            const bool vector = m_aligned && (r.in_begin % epv == r.out_begin % epv);
+            uint64_t head = 0, body = 0;
+            if (vector) {
+                head = std::min<uint64_t>((epv - r.in_begin % epv) % epv, r.count);
+                body = (r.count - head) / epv * epv;
+            }
+            if (!body) {
+                add_segment(r.in_begin, r.out_begin, r.count, r, 0);
+                continue;
+            }
+            const uint64_t tail = r.count - head - body;
+            if (head) add_segment(r.in_begin, r.out_begin, head, r, 0);
+            add_segment(r.in_begin + head, r.out_begin + head, body, r, kSegVector);
+            if (tail) add_segment(r.in_begin + head + body, r.out_begin + head + body, tail, r, 0);
+        }
+        close_launch();
+    }
+
+    void open_launch() {
+        std::memset(&m_launch, 0, sizeof(m_launch));
+        for (uint32_t r = 0; r < kMaxRanks; ++r) {
+            m_launch.in[r] = m_in[r];
+            m_launch.out[r] = m_out[r];
+        }
+        for (uint32_t i = 0; i < kMaxSegments; ++i) m_launch.first_tile[i] = 0xffffffffu;
+        m_launch.nranks = m_nranks;
+        m_launch.nfold = m_nfold;
+        m_launch.nout = m_nout;
+        m_launch.new_wins_ties = m_new_wins ? 1 : 0;
+        m_launch.unroll = fold_unroll(m_nfold);
+        m_launch.elem_size = m_elem;
+    }
+
+    void close_launch() {
         if (!m_launch.nseg) return;
         Step step;
         std::memset(&step, 0, sizeof(step));
         step.kind = Step::kFold;
-        step.is_copy = m_launch.nfold == 1;
         step.fold = m_launch;
         m_plan.steps.push_back(step);
-        m_launch.nseg = 0;
-        m_launch.total_tiles = 0;
     }
 
-private:
-    void add_segment(uint64_t in_begin, uint64_t out_begin, uint64_t count, uint8_t start, int8_t dir,
-                     uint8_t out_first, uint8_t flags) {
+    void add_segment(uint64_t in_begin, uint64_t out_begin, uint64_t count, const Run& r, uint8_t flags) {
         const uint64_t per_tile = tile_elems(m_launch, flags & kSegVector);
         const uint64_t max_tiles = 0x7fffffffull;
         while (count) {
-            if (m_launch.nseg == kMaxSegments || m_launch.total_tiles >= max_tiles) finish();
+            if (m_launch.nseg == kMaxSegments || m_launch.total_tiles >= max_tiles) {
+                close_launch();
+                open_launch();
+            }
             // a segment never takes more tiles than one launch's grid has left
             const uint64_t room = max_tiles - m_launch.total_tiles;
             const uint64_t take = std::min(count, room * per_tile);
+            m_launch.first_tile[m_launch.nseg] = m_launch.total_tiles;
             FoldSegment& sg = m_launch.seg[m_launch.nseg++];
             sg.in_begin = in_begin;
             sg.out_begin = out_begin;
             sg.count = take;
-            sg.first_tile = m_launch.total_tiles;
-            sg.start = start;
-            sg.dir = dir;
-            sg.out_first = out_first;
+            sg.start = r.start;
+            sg.dir = r.dir;
+            sg.out_first = r.out_first;
             sg.flags = flags;
             m_launch.total_tiles += uint32_t((take + per_tile - 1) / per_tile);
             in_begin += take;
@@ -116,8 +195,13 @@ private:
     }
 
     Plan& m_plan;
-    FoldLaunch m_launch;
+    const void* m_in[kMaxRanks];
+    void* m_out[kMaxRanks];
+    uint32_t m_nranks, m_nfold, m_nout, m_elem;
+    bool m_new_wins;
     bool m_aligned;
+    std::vector<Run> m_runs;
+    FoldLaunch m_launch;
 };
 
 Status check_ranks(uint32_t nranks) {

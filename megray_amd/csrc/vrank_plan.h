@@ -37,10 +37,10 @@ enum Schedule : int {
 enum Collective : int { kAllReduce = 0, kReduceScatter = 1 };
 
 struct Step {
-    enum Kind : int { kFold = 0, kPack = 1 } kind;
-    bool is_copy;  // a fold step with nfold == 1: dtype / op do not matter
+    enum Kind : int { kFold = 0, kPack = 1, kFlat = 2 } kind;
     FoldLaunch fold;
     PackLaunch pack;
+    FlatLaunch flat;
 };
 
 struct Plan {

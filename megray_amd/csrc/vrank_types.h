@@ -11,7 +11,7 @@ namespace vrank {
 constexpr uint32_t kMaxRanks = 16;            // virtual ranks per group
 constexpr uint32_t kMaxChunks = 2 * kMaxRanks;  // the shm order splits a buffer into 2N chunks
 constexpr uint32_t kMaxSegments = 3 * kMaxChunks;  // head / aligned body / tail per chunk
-constexpr uint32_t kThreads = 256;            // workgroup size: four 64-wide wavefronts
+constexpr uint32_t kThreads = 64;             // workgroup = one 64-wide wavefront (measured best: 1 KiB per buffer per tile)
 constexpr uint32_t kVecBytes = 16;            // one 128-bit global load / store per lane
 
 enum SegmentFlags : uint8_t {
@@ -23,7 +23,7 @@ struct FoldSegment {
     uint64_t in_begin;    // first element, same index in every input buffer
     uint64_t out_begin;   // first element in every output buffer
     uint64_t count;       // elements
-    uint32_t first_tile;  // tiles of all earlier segments
+    uint32_t reserved;
     uint8_t start;        // rank whose buffer seeds the accumulator
     int8_t dir;           // +1: start, start+1, ...   -1: start, start-1, ...   (mod nranks)
     uint8_t out_first;    // destinations are ranks out_first .. out_first+nout-1 (mod nranks)
@@ -36,6 +36,7 @@ struct FoldLaunch {
     const void* in[kMaxRanks];
     void* out[kMaxRanks];
     FoldSegment seg[kMaxSegments];
+    uint32_t first_tile[kMaxSegments];  // tiles of all earlier segments; unused entries 0xffffffff
     uint32_t nranks;         // modulus of the rank rotation
     uint32_t nfold;          // inputs folded per element (1 = plain copy)
     uint32_t nout;           // destinations per element
@@ -43,6 +44,39 @@ struct FoldLaunch {
     uint32_t total_tiles;
     uint32_t new_wins_ties;  // float MAX/MIN: an equal / unordered compare keeps the newcomer
     uint32_t unroll;         // vectors (or elements) per lane per tile; fixes the tile size
+    uint32_t elem_size;
+};
+
+constexpr uint32_t kMaxFlatRuns = 48;  // 2N chunks cut again at N-1 rank borders
+
+// One run of a flat launch: elements [begin, end) of the buffer, one fold order, one destination
+// set, outputs shifted by a whole number of 16-byte vectors.
+struct FlatRun {
+    uint64_t begin;
+    uint64_t end;
+    int64_t out_shift;  // output index = element index - out_shift
+    uint8_t start;
+    int8_t dir;
+    uint8_t out_first;
+    uint8_t pad[5];
+};
+
+// One launch of the flat fold kernel.  Tile t always covers bytes [1024 t, 1024 t + 1024) of every
+// input buffer, so a wavefront can issue its loads before it knows which run it is in; the run (and
+// with it the fold order) is looked up while the loads are in flight.  Needs nfold == nranks, all
+// buffers 16-byte aligned and every out_shift a multiple of a vector.
+struct FlatLaunch {
+    const void* in[kMaxRanks];
+    void* out[kMaxRanks];
+    uint32_t tile_lo[kMaxFlatRuns];  // tiles [tile_lo, tile_hi) lie wholly inside the run;
+    uint32_t tile_hi[kMaxFlatRuns];  // unused entries are 0, 0
+    FlatRun run[kMaxFlatRuns];
+    uint64_t count;          // elements per input buffer
+    uint32_t nranks;         // == fold width
+    uint32_t nout;
+    uint32_t nruns;
+    uint32_t total_tiles;    // ceil(count * elem_size / 1024)
+    uint32_t new_wins_ties;
     uint32_t elem_size;
 };
 
@@ -70,10 +104,10 @@ struct PackLaunch {
 // Vectors (or elements) each lane moves per tile.  The kernels are instantiated with these values;
 // the planner sizes its tiles with the same function.
 constexpr uint32_t fold_unroll(uint32_t nfold) {
-    return nfold == 1 ? 4u : nfold == 2 ? 4u : (nfold == 3 || nfold == 4) ? 2u : 1u;
+    return nfold ? 1u : 1u;  // measured: one vector per lane beats every deeper unroll, for every fold width
 }
 constexpr uint32_t pack_unroll() {
-    return 4u;
+    return 1u;
 }
 
 inline uint64_t tile_elems(const FoldLaunch& L, bool vector) {

@@ -1,0 +1,94 @@
+"""The C ABI library loads and exports every symbol include/megray_vrank.h declares; host-only
+entry points agree with the oracle.  No compute calls, no GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+import oracle as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "megray_vrank.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from megray_amd import _lib
+    return _lib.load()
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    return re.findall(r"MRV_API\s+[\w\s\*]+?\b(mrv_\w+)\s*\(", text)
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_symbols()
+    for must in ("mrv_reduce", "mrv_all_reduce", "mrv_reduce_scatter", "mrv_all_gather", "mrv_all_to_all",
+                 "mrv_scatter", "mrv_gather", "mrv_broadcast", "mrv_describe", "mrv_fold_order",
+                 "mrv_chunk_partition", "mrv_dtype_size", "mrv_last_error", "mrv_abi_version"):
+        assert must in names
+    assert len(names) == len(set(names))
+
+
+def test_library_exports_every_declared_symbol(lib):
+    for name in declared_symbols():
+        assert hasattr(lib, name), f"{name} is declared in megray_vrank.h but not exported"
+
+
+def test_cxx_api_symbols_are_exported(lib):
+    # MegRay::get_dtype_size(MegRay::DType), the mangled C++ symbol a C++ caller links against
+    assert hasattr(lib, "_ZN6MegRay14get_dtype_sizeENS_5DTypeE")
+
+
+def test_abi_version_and_dtype_sizes(lib):
+    assert lib.mrv_abi_version() >= 1
+    for dtype in range(10):
+        assert lib.mrv_dtype_size(dtype) == orc.dtype_size(dtype)
+    for bad in (-1, 10, 99):
+        assert lib.mrv_dtype_size(bad) == 0
+        assert lib.mrv_last_error() == b"unknown dtype"  # src/core/common.cpp:35-36
+
+
+def test_chunk_partition_matches_oracle():
+    import megray_amd as mr
+    for nchunks in range(1, 33):
+        for length in list(range(0, 70)) + [2 ** 28, 2 ** 28 + 5, 2 ** 33 + 7]:
+            assert mr.chunk_partition(length, nchunks) == tuple(orc.chunk_partition(length, nchunks))
+
+
+def test_fold_order_matches_oracle():
+    import megray_amd as mr
+    for nranks in range(1, 17):
+        for coll in (orc.COLL_ALL_REDUCE, orc.COLL_REDUCE_SCATTER):
+            for order in (orc.ORDER_UCX, orc.ORDER_SHM, orc.ORDER_RANK0):
+                nchunks = orc.fold_order(coll, order, nranks, 0)[2]
+                for chunk in range(nchunks):
+                    ranks, new_wins, nch, owner = mr.fold_order(coll, order, nranks, chunk)
+                    assert (ranks, new_wins, nch) == orc.fold_order(coll, order, nranks, chunk)
+                    assert 0 <= owner < nranks
+                with pytest.raises(mr.MegRayError):
+                    mr.fold_order(coll, order, nranks, nchunks)
+    with pytest.raises(mr.MegRayError):
+        mr.fold_order(0, 0, 17, 0)
+    with pytest.raises(mr.MegRayError):
+        mr.fold_order(0, 5, 4, 0)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    from megray_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libmegray_vrank.so")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        _lib.load()
+
+
+def test_product_never_imports_the_oracle():
+    """The shipped package must not reference the CPU oracle in any way."""
+    pkg = os.path.join(ROOT, "megray_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for name in files:
+            if name.endswith((".py", ".cpp", ".h", ".hip")):
+                text = open(os.path.join(dirpath, name)).read()
+                assert "import oracle" not in text and "megray_oracle" not in text, name

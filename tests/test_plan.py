@@ -1,0 +1,232 @@
+"""Host planner (no GPU): the launches mrv_describe() reports are interpreted here with numpy, run
+by run, and must reproduce the oracle's literal replays bit for bit.  This checks chunking, fold
+orders, tie conventions, the head / vector-body / tail split and the multi-launch schedules
+independently of the kernels."""
+import numpy as np
+import pytest
+
+import megray_amd as mr
+import oracle as orc
+
+SEND_BASE = 0x100000000000
+RECV_BASE = 0x200000000000
+STRIDE = 0x001000000000
+
+REDUCE_TYPES = [orc.INT8, orc.UINT8, orc.INT32, orc.UINT32, orc.INT64, orc.UINT64, orc.FLOAT32, orc.FLOAT64]
+
+
+def rand_array(dtype, n, rng):
+    npdt = orc.NP_DTYPE[dtype]
+    if np.issubdtype(npdt, np.integer):
+        raw = rng.integers(0, 2 ** 64, size=n, dtype=np.uint64)
+        return raw.astype(np.dtype(npdt).str.replace("i", "u")).view(npdt)
+    return (rng.standard_normal(n) * np.exp(rng.uniform(-20, 20, n))).astype(npdt)
+
+
+def fake_ptrs(base, n, offsets):
+    return [base + r * STRIDE + offsets[r] for r in range(n)]
+
+
+def combine(acc, x, op, new_wins):
+    with np.errstate(over="ignore"):
+        if op == orc.SUM:
+            return acc + x
+        if op == orc.MAX:
+            return np.where(acc > x, acc, x) if new_wins else np.where(x > acc, x, acc)
+        return np.where(acc < x, acc, x) if new_wins else np.where(x < acc, x, acc)
+
+
+def execute(runs, sends, recvs, nranks, op, elem_size, send_ptrs, recv_ptrs):
+    """Interpret plan runs in launch order.  Within one launch all reads happen on the values the
+    previous launch left, unless a run reads and writes the very same element (in place)."""
+    steps = sorted({r["step"] for r in runs})
+    for step in steps:
+        snapshot = [x.copy() for x in recvs]
+        for run in (r for r in runs if r["step"] == step):
+            if run["kind"] == 0:
+                src = snapshot if run["reads_recv"] else sends
+                ranks = [(run["start"] + run["dir"] * j) % nranks for j in range(run["nfold"])]
+                lo, cnt = run["in_begin"], run["count"]
+                acc = src[ranks[0]][lo:lo + cnt].copy()
+                for r in ranks[1:]:
+                    acc = combine(acc, src[r][lo:lo + cnt], op, run["new_wins_ties"])
+                for m in range(run["nout"]):
+                    dst = (run["out_first"] + m) % nranks
+                    recvs[dst][run["out_begin"]:run["out_begin"] + cnt] = acc
+                if run["vector"]:
+                    epv = 16 // elem_size
+                    base_in = recv_ptrs if run["reads_recv"] else send_ptrs
+                    if run["vector"] == 1:
+                        assert cnt % epv == 0
+                    else:  # flat launch: bases aligned, outputs shifted by whole vectors
+                        assert (lo - run["out_begin"]) % epv == 0
+                        lo = 0
+                        run = dict(run, out_begin=0)
+                    for r in ranks:
+                        assert (base_in[r] + lo * elem_size) % 16 == 0
+                    for m in range(run["nout"]):
+                        dst = (run["out_first"] + m) % nranks
+                        assert (recv_ptrs[dst] + run["out_begin"] * elem_size) % 16 == 0
+            else:
+                s, d = run["start"], run["out_first"]
+                a, b, cnt = run["in_begin"], run["out_begin"], run["count"]
+                recvs[d].view(np.uint8)[b:b + cnt] = sends[s].view(np.uint8)[a:a + cnt]
+                width = run["vector"]
+                assert cnt % width == 0 and (send_ptrs[s] + a) % width == 0 and (recv_ptrs[d] + b) % width == 0
+    return recvs
+
+
+def bits_equal(a, b):
+    return np.array_equal(np.ascontiguousarray(a).view(np.uint8), np.ascontiguousarray(b).view(np.uint8))
+
+
+@pytest.mark.parametrize("dtype", REDUCE_TYPES)
+@pytest.mark.parametrize("nranks", [1, 2, 3, 4, 7, 8, 16])
+def test_all_reduce_plans_reproduce_the_replays(dtype, nranks):
+    rng = np.random.default_rng(dtype * 100 + nranks)
+    size = orc.dtype_size(dtype)
+    for length in (0, 1, nranks - 1, 3 * nranks + 1, 300, 4099):
+        ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+        for misalign in (False, True):
+            offs = [size * (r % 3) for r in range(nranks)] if misalign else [0] * nranks
+            sp, rp = fake_ptrs(SEND_BASE, nranks, offs), fake_ptrs(RECV_BASE, nranks, offs)
+            for op in (orc.SUM, orc.MAX, orc.MIN):
+                cases = [(orc.ORDER_UCX, s) for s in (mr.Schedule.FUSED, mr.Schedule.TWO_PHASE, mr.Schedule.RING)]
+                cases += [(orc.ORDER_SHM, s) for s in (mr.Schedule.FUSED, mr.Schedule.TWO_PHASE)]
+                cases += [(orc.ORDER_RANK0, mr.Schedule.FUSED)]
+                for order, sched in cases:
+                    runs, br, bw = mr.describe(mr.Collective.ALL_REDUCE, sp, rp, length, dtype, order, sched)
+                    recvs = [np.zeros(length, dtype=ins[0].dtype) for _ in range(nranks)]
+                    got = execute(runs, ins, recvs, nranks, op, size, sp, rp)
+                    if order == orc.ORDER_UCX:
+                        want = orc.ucx_all_reduce(ins, dtype, op)
+                    elif order == orc.ORDER_SHM and dtype in (orc.INT8, orc.UINT8, orc.INT32, orc.UINT32,
+                                                              orc.INT64, orc.FLOAT32):
+                        want = orc.shm_all_reduce(ins, dtype, op)
+                    else:
+                        want = orc.fold_all_reduce(ins, dtype, op, order)
+                    for r in range(nranks):
+                        assert bits_equal(got[r], want[r]), (dtype, nranks, length, misalign, op, order, sched)
+                    # algorithmic bytes of the schedule
+                    ns = length * size
+                    if sched == mr.Schedule.FUSED:
+                        assert (br, bw) == (nranks * ns, nranks * ns)
+                    elif sched == mr.Schedule.TWO_PHASE:
+                        assert (br, bw) == (nranks * ns + (ns if nranks > 1 else 0), ns + (nranks - 1) * ns)
+                    else:  # N copies in, (N-1) steps of 2 reads + 1 write, (N-1) steps of 1 read + 1 write per chunk
+                        assert br + bw == 2 * nranks * ns + 5 * (nranks - 1) * ns
+
+
+@pytest.mark.parametrize("dtype", [orc.INT8, orc.INT32, orc.FLOAT32, orc.FLOAT64, orc.UINT64])
+@pytest.mark.parametrize("nranks", [1, 2, 3, 8, 16])
+def test_reduce_scatter_plans(dtype, nranks):
+    rng = np.random.default_rng(dtype * 10 + nranks)
+    size = orc.dtype_size(dtype)
+    for recvlen in (0, 1, 3, 5, 64, 1031):
+        ins = [rand_array(dtype, nranks * recvlen, rng) for _ in range(nranks)]
+        sp, rp = fake_ptrs(SEND_BASE, nranks, [0] * nranks), fake_ptrs(RECV_BASE, nranks, [0] * nranks)
+        for op in (orc.SUM, orc.MAX, orc.MIN):
+            for order in (orc.ORDER_UCX, orc.ORDER_SHM, orc.ORDER_RANK0):
+                runs, br, bw = mr.describe(mr.Collective.REDUCE_SCATTER, sp, rp, recvlen, dtype, order)
+                recvs = [np.zeros(recvlen, dtype=ins[0].dtype) for _ in range(nranks)]
+                got = execute(runs, ins, recvs, nranks, op, size, sp, rp)
+                if order == orc.ORDER_UCX:
+                    want = orc.ucx_reduce_scatter(ins, dtype, op)
+                elif order == orc.ORDER_SHM and dtype in (orc.INT8, orc.INT32, orc.FLOAT32):
+                    want = orc.shm_reduce_scatter(ins, dtype, op)
+                else:
+                    want = orc.fold_reduce_scatter(ins, dtype, op, order)
+                for r in range(nranks):
+                    assert bits_equal(got[r], want[r]), (dtype, nranks, recvlen, op, order)
+                assert (br, bw) == (nranks * nranks * recvlen * size, nranks * recvlen * size)
+
+
+@pytest.mark.parametrize("nranks", [1, 2, 3, 8, 16])
+def test_pack_plans(nranks):
+    rng = np.random.default_rng(nranks)
+    for dtype in (orc.UINT8, orc.FLOAT16, orc.FLOAT32, orc.INT64, orc.CHAR):
+        size = orc.dtype_size(dtype)
+        gen = orc.UINT8 if dtype == orc.CHAR else dtype
+        for length in (0, 1, 6, 100, 1030):
+            for misalign in (0, size):
+                offs = [misalign] * nranks
+                sp, rp = fake_ptrs(SEND_BASE, nranks, offs), fake_ptrs(RECV_BASE, nranks, offs)
+                ins = [rand_array(gen, nranks * length, rng) if gen != orc.FLOAT16
+                       else rng.standard_normal(nranks * length).astype(np.float16) for _ in range(nranks)]
+                npdt = ins[0].dtype
+
+                def run(coll, sends, out_len, count, root=0):
+                    runs, _, _ = mr.describe(coll, sp, rp, count, dtype, root=root, nranks=nranks)
+                    recvs = [np.zeros(out_len, dtype=npdt) for _ in range(nranks)]
+                    return execute(runs, sends, recvs, nranks, orc.SUM, size, sp, rp)
+
+                got = run(mr.Collective.ALL_TO_ALL, ins, nranks * length, length)
+                want = orc.ucx_all_to_all(ins, dtype)
+                assert all(bits_equal(got[r], want[r]) for r in range(nranks))
+                parts = [x[:length].copy() for x in ins]
+                got = run(mr.Collective.ALL_GATHER, parts, nranks * length, length)
+                want = orc.ucx_all_gather(parts, dtype)
+                assert all(bits_equal(got[r], want[r]) for r in range(nranks))
+                root = nranks - 1
+                got = run(mr.Collective.SCATTER, ins, length, length, root)
+                want = orc.ucx_scatter([ins[root] if r == root else None for r in range(nranks)], dtype, root)
+                assert all(bits_equal(got[r], want[r]) for r in range(nranks))
+                got = run(mr.Collective.GATHER, parts, nranks * length, length, root)
+                assert bits_equal(got[root], orc.ucx_gather(parts, dtype, root)[root])
+                got = run(mr.Collective.BROADCAST, parts, length, length, root)
+                assert all(bits_equal(got[r], parts[root]) for r in range(nranks))
+
+
+def test_two_input_reduce_plan_keeps_i1_on_ties():
+    # src/ucx/kernel.cu:24-38: (i0 > i1) ? i0 : i1
+    a = np.array([0.0, -0.0, np.nan, 1.0, 5.0], dtype=np.float32)
+    b = np.array([-0.0, 0.0, 1.0, np.nan, 2.0], dtype=np.float32)
+    sp = [SEND_BASE, SEND_BASE + STRIDE]
+    rp = [RECV_BASE]
+    for op in (orc.MAX, orc.MIN, orc.SUM):
+        runs, br, bw = mr.describe(mr.Collective.REDUCE2, sp, rp, a.size, orc.FLOAT32, nranks=2)
+        got = execute(runs, [a, b], [np.zeros_like(a), np.zeros_like(a)], 2, op, 4, sp, rp + [0])[0]
+        want = orc.reduce_ucx(a, b, orc.FLOAT32, op)
+        nan = np.isnan(want)
+        assert np.array_equal(np.isnan(got), nan) and bits_equal(got[~nan], want[~nan])
+        assert (br, bw) == (2 * a.size * 4, a.size * 4)
+
+
+def test_full_size_plan_shapes():
+    """The headline shape: 8 ranks x 2^28 fp32 is one launch of 8 vector runs, 65536 x 1 KiB-per-wave
+    tiles... and every planned byte is accounted for."""
+    n = 1 << 28
+    sp, rp = fake_ptrs(SEND_BASE, 8, [0] * 8), fake_ptrs(RECV_BASE, 8, [0] * 8)
+    runs, br, bw = mr.describe(mr.Collective.ALL_REDUCE, sp, rp, n, orc.FLOAT32)
+    assert len(runs) == 8 and all(r["vector"] == 2 and r["nfold"] == 8 and r["nout"] == 8 for r in runs)
+    assert sum(r["tiles"] for r in runs) == n * 4 // 1024
+    assert sum(r["count"] for r in runs) == n
+    assert br == bw == 8 * n * 4
+    # a buffer far beyond one launch's grid is split into several launches, nothing lost
+    big = 1 << 41
+    runs, br, bw = mr.describe(mr.Collective.ALL_REDUCE, [SEND_BASE, SEND_BASE + (1 << 42)],
+                               [RECV_BASE, RECV_BASE + (1 << 42)], big, orc.INT8)
+    assert sum(r["count"] for r in runs) == big and len({r["step"] for r in runs}) >= 1
+    assert all(r["tiles"] <= 0x7fffffff for r in runs)
+
+
+def test_planner_rejects_what_it_cannot_honour():
+    sp, rp = fake_ptrs(SEND_BASE, 4, [0] * 4), fake_ptrs(RECV_BASE, 4, [0] * 4)
+    with pytest.raises(mr.MegRayError, match="ring schedule"):
+        mr.describe(mr.Collective.ALL_REDUCE, sp, rp, 100, orc.FLOAT32, orc.ORDER_SHM, mr.Schedule.RING)
+    with pytest.raises(mr.MegRayError, match="overlap"):
+        mr.describe(mr.Collective.ALL_REDUCE, sp, [sp[1], rp[1], rp[2], rp[3]], 100, orc.FLOAT32)
+    with pytest.raises(mr.MegRayError, match="overlap"):
+        mr.describe(mr.Collective.ALL_REDUCE, sp, [rp[0], rp[0] + 8, rp[2], rp[3]], 100, orc.FLOAT32)
+    with pytest.raises(mr.MegRayError, match="in place"):
+        mr.describe(mr.Collective.ALL_TO_ALL, sp, sp, 100, orc.FLOAT32)
+    with pytest.raises(mr.MegRayError, match="unknown dtype"):
+        mr.describe(mr.Collective.ALL_REDUCE, sp, rp, 100, orc.CHAR)
+    with pytest.raises(mr.MegRayError, match="root"):
+        mr.describe(mr.Collective.SCATTER, sp, rp, 100, orc.FLOAT32, root=4)
+    # in place is fine where every element keeps its address
+    mr.describe(mr.Collective.ALL_REDUCE, sp, sp, 100, orc.FLOAT32)
+    mr.describe(mr.Collective.REDUCE_SCATTER, sp, [sp[r] + r * 400 for r in range(4)], 100, orc.FLOAT32)
+    mr.describe(mr.Collective.ALL_GATHER, [rp[r] + r * 400 for r in range(4)], rp, 100, orc.FLOAT32)
+    with pytest.raises(mr.MegRayError, match="out of place"):
+        mr.describe(mr.Collective.REDUCE_SCATTER, sp, sp, 100, orc.FLOAT32)
