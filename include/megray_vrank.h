@@ -55,7 +55,8 @@ enum {
     MRV_SCATTER = 4,
     MRV_GATHER = 5,
     MRV_BROADCAST = 6,
-    MRV_REDUCE2 = 7
+    MRV_REDUCE2 = 7,
+    MRV_REDUCE = 8
 };
 
 /* ---- library ------------------------------------------------------------------------------ */
@@ -160,7 +161,7 @@ typedef struct mrv_plan_run {
     uint32_t vector;        /* fold: 0 = element by element, 1 = 16-byte vectors, 2 = run of a flat launch
                                (vectors on the buffer's own 1 KiB tile grid); pack: bytes per lane access */
     uint32_t start;         /* fold: seed rank; pack: source rank */
-    int32_t dir;            /* fold: +1 / -1 */
+    int32_t dir;            /* fold: +1 / -1; 0 = binomial tree towards rank `start` */
     uint32_t out_first;     /* fold: first destination rank; pack: destination rank */
     uint32_t tiles;         /* workgroups this run occupies (flat: those wholly inside it) */
     uint32_t reads_recv;    /* 1 = the launch reads the receive buffers (a later step of a multi-launch plan) */
@@ -182,6 +183,69 @@ MRV_API int mrv_describe(int collective, const void* const* sendbuffs, void* con
                          uint32_t nranks, size_t count, int dtype, int order, int schedule, uint32_t root,
                          mrv_plan_run* runs, size_t cap, size_t* nruns, uint64_t* bytes_read,
                          uint64_t* bytes_written);
+
+/* ---- the MegRay::Communicator API, one handle per rank ------------------------------------- */
+
+/*
+ * These bind the C++ API one to one for callers that cannot link C++: a handle owns the
+ * std::shared_ptr<MegRay::Communicator> that MegRay::get_communicator returns
+ * (include/megray.h:33-34), every call wraps `stream` in a MegRay::HipContext
+ * (include/megray/hip_context.h:43-54) and forwards to the virtual of the same name
+ * (include/megray/communicator.h:60-109).  As with the C++ API, each rank's calls come from its own
+ * thread and every rank of a group makes the same calls in the same order; a collective returns
+ * once all ranks have arrived and the work is enqueued.
+ */
+typedef struct mrv_comm mrv_comm;
+
+/* MegRay::get_free_port / MegRay::create_server (include/megray/server.h:19-24). */
+MRV_API int mrv_get_free_port(void);
+MRV_API int mrv_create_server(uint32_t nranks, int port);
+
+/* get_communicator(nranks, rank, backend); backend 4 = MEGRAY_VRANK, anything else: "unknown backend". */
+MRV_API int mrv_comm_create(uint32_t nranks, uint32_t rank, int backend, mrv_comm** comm);
+MRV_API void mrv_comm_destroy(mrv_comm* comm);
+/* Communicator::init(master_ip, port) (src/core/communicator.cpp:17-21). */
+MRV_API int mrv_comm_init(mrv_comm* comm, const char* master_ip, int port);
+/* Fold order / schedule of this rank's communicator (MRV_ORDER_*, MRV_SCHED_*); no reference counterpart. */
+MRV_API int mrv_comm_configure(mrv_comm* comm, int order, int schedule);
+
+MRV_API int mrv_comm_send(mrv_comm* comm, const void* sendbuff, size_t len, int dtype, uint32_t rank,
+                          void* stream);
+MRV_API int mrv_comm_recv(mrv_comm* comm, void* recvbuff, size_t len, int dtype, uint32_t rank, void* stream);
+MRV_API int mrv_comm_scatter(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t recvlen, int dtype,
+                             uint32_t root, void* stream);
+MRV_API int mrv_comm_gather(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t sendlen, int dtype,
+                            uint32_t root, void* stream);
+MRV_API int mrv_comm_all_to_all(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t len, int dtype,
+                                void* stream);
+MRV_API int mrv_comm_all_gather(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t sendlen,
+                                int dtype, void* stream);
+MRV_API int mrv_comm_all_reduce(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t len, int dtype,
+                                int op, void* stream);
+MRV_API int mrv_comm_reduce_scatter(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t recvlen,
+                                    int dtype, int op, void* stream);
+MRV_API int mrv_comm_broadcast(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t len, int dtype,
+                               uint32_t root, void* stream);
+MRV_API int mrv_comm_reduce(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t len, int dtype, int op,
+                            uint32_t root, void* stream);
+MRV_API int mrv_comm_group_start(mrv_comm* comm);
+MRV_API int mrv_comm_group_end(mrv_comm* comm);
+
+/* recv_root = combination of sendbuffs[*] for rank `root`, all ranks' buffers at once.
+ * Replaces UcxCommunicator::reduce (src/ucx/reduce.cpp:21-87: binomial tree, MRV_ORDER_UCX) and
+ * ShmCommunicator reduce (src/shm/reduce.cpp:21-100: MRV_ORDER_SHM). */
+MRV_API int mrv_reduce_to_root(const void* const* sendbuffs, void* recvbuff_root, uint32_t nranks, size_t len,
+                               int dtype, int op, int order, uint32_t root, void* stream);
+
+/* The bootstrap client (include/megray/client.h:24-49), host memory only. */
+typedef struct mrv_client mrv_client;
+MRV_API int mrv_client_create(uint32_t nranks, uint32_t rank, mrv_client** client);
+MRV_API void mrv_client_destroy(mrv_client* client);
+MRV_API int mrv_client_connect(mrv_client* client, const char* master_ip, int port);
+MRV_API int mrv_client_barrier(mrv_client* client);
+MRV_API int mrv_client_broadcast(mrv_client* client, const void* sendbuff, void* recvbuff, size_t len,
+                                 uint32_t root);
+MRV_API int mrv_client_allgather(mrv_client* client, const void* sendbuff, void* recvbuff, size_t sendlen);
 
 #ifdef __cplusplus
 }

@@ -56,6 +56,40 @@ def load():
     L.mrv_describe.argtypes = [i32, pp, pp, u32, sz, i32, i32, i32, u32, ctypes.POINTER(PlanRun), sz,
                                ctypes.POINTER(sz), ctypes.POINTER(ctypes.c_uint64),
                                ctypes.POINTER(ctypes.c_uint64)]
+    L.mrv_reduce_to_root.argtypes = [pp, vp, u32, sz, i32, i32, i32, u32, vp]
+    L.mrv_get_free_port.argtypes = []
+    L.mrv_create_server.argtypes = [u32, i32]
+    L.mrv_comm_create.argtypes = [u32, u32, i32, ctypes.POINTER(vp)]
+    L.mrv_comm_destroy.argtypes = [vp]
+    L.mrv_comm_destroy.restype = None
+    L.mrv_comm_init.argtypes = [vp, ctypes.c_char_p, i32]
+    L.mrv_comm_configure.argtypes = [vp, i32, i32]
+    L.mrv_comm_send.argtypes = [vp, vp, sz, i32, u32, vp]
+    L.mrv_comm_recv.argtypes = [vp, vp, sz, i32, u32, vp]
+    L.mrv_comm_scatter.argtypes = [vp, vp, vp, sz, i32, u32, vp]
+    L.mrv_comm_gather.argtypes = [vp, vp, vp, sz, i32, u32, vp]
+    L.mrv_comm_all_to_all.argtypes = [vp, vp, vp, sz, i32, vp]
+    L.mrv_comm_all_gather.argtypes = [vp, vp, vp, sz, i32, vp]
+    L.mrv_comm_all_reduce.argtypes = [vp, vp, vp, sz, i32, i32, vp]
+    L.mrv_comm_reduce_scatter.argtypes = [vp, vp, vp, sz, i32, i32, vp]
+    L.mrv_comm_broadcast.argtypes = [vp, vp, vp, sz, i32, u32, vp]
+    L.mrv_comm_reduce.argtypes = [vp, vp, vp, sz, i32, i32, u32, vp]
+    L.mrv_comm_group_start.argtypes = [vp]
+    L.mrv_comm_group_end.argtypes = [vp]
+    L.mrv_client_create.argtypes = [u32, u32, ctypes.POINTER(vp)]
+    L.mrv_client_destroy.argtypes = [vp]
+    L.mrv_client_destroy.restype = None
+    L.mrv_client_connect.argtypes = [vp, ctypes.c_char_p, i32]
+    L.mrv_client_barrier.argtypes = [vp]
+    L.mrv_client_broadcast.argtypes = [vp, vp, vp, sz, u32]
+    L.mrv_client_allgather.argtypes = [vp, vp, vp, sz]
+    for name in ("mrv_reduce_to_root", "mrv_get_free_port", "mrv_create_server", "mrv_comm_create",
+                 "mrv_comm_init", "mrv_comm_configure", "mrv_comm_send", "mrv_comm_recv", "mrv_comm_scatter",
+                 "mrv_comm_gather", "mrv_comm_all_to_all", "mrv_comm_all_gather", "mrv_comm_all_reduce",
+                 "mrv_comm_reduce_scatter", "mrv_comm_broadcast", "mrv_comm_reduce", "mrv_comm_group_start",
+                 "mrv_comm_group_end", "mrv_client_create", "mrv_client_connect", "mrv_client_barrier",
+                 "mrv_client_broadcast", "mrv_client_allgather"):
+        getattr(L, name).restype = i32
     for name in ("mrv_reduce", "mrv_all_reduce", "mrv_reduce_scatter", "mrv_all_gather",
                  "mrv_all_to_all", "mrv_scatter", "mrv_gather", "mrv_broadcast", "mrv_chunk_partition",
                  "mrv_fold_order", "mrv_describe"):

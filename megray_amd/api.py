@@ -77,6 +77,7 @@ class Collective(enum.IntEnum):
     GATHER = 5
     BROADCAST = 6
     REDUCE2 = 7
+    REDUCE = 8
 
 
 MAX_RANKS = 16
@@ -168,6 +169,11 @@ def broadcast(sendbuff_root, recvbuffs, length, dtype, root, stream=None):
                                      int(dtype), root, _stream(stream)))
 
 
+def reduce_to_root(sendbuffs, recvbuff_root, length, dtype, op, root, order=FoldOrder.UCX, stream=None):
+    _check(_lib.load().mrv_reduce_to_root(_ptr_array(sendbuffs), _ptr(recvbuff_root), len(sendbuffs), length,
+                                          int(dtype), int(op), int(order), root, _stream(stream)))
+
+
 def chunk_partition(length, nchunks):
     sizes = (ctypes.c_size_t * nchunks)()
     offs = (ctypes.c_size_t * nchunks)()
@@ -203,3 +209,132 @@ def describe(collective, sendptrs, recvptrs, count, dtype, order=FoldOrder.UCX, 
         r = runs[i]
         out.append({name: getattr(r, name) for name, _ in _lib.PlanRun._fields_})
     return out, br.value, bw.value
+
+
+# ---------------------------------------------------------------------------------------------
+# the Communicator API, one object per rank (include/megray/communicator.h:32-123)
+
+def get_free_port():
+    """MegRay::get_free_port (include/megray/server.h:21)."""
+    port = _lib.load().mrv_get_free_port()
+    if port <= 0:
+        raise MegRayError(Status.SYS_ERROR, _lib.load().mrv_last_error().decode())
+    return port
+
+
+def create_server(nranks, port):
+    """MegRay::create_server (include/megray/server.h:24)."""
+    _check(_lib.load().mrv_create_server(nranks, port))
+
+
+class Client:
+    """MegRay::Client (include/megray/client.h:24-49): host-side barrier / broadcast / allgather."""
+
+    def __init__(self, nranks, rank):
+        self._h = ctypes.c_void_p()
+        self.nranks = nranks
+        _check(_lib.load().mrv_client_create(nranks, rank, ctypes.byref(self._h)))
+
+    def connect(self, master_ip, port):
+        _check(_lib.load().mrv_client_connect(self._h, master_ip.encode(), port))
+
+    def barrier(self):
+        _check(_lib.load().mrv_client_barrier(self._h))
+
+    def broadcast(self, data, root, is_root):
+        """data: bytes on the root (any bytes-like of the same length elsewhere) -> bytes"""
+        out = ctypes.create_string_buffer(len(data))
+        src = ctypes.create_string_buffer(bytes(data), len(data)) if is_root else None
+        _check(_lib.load().mrv_client_broadcast(self._h, src, out, len(data), root))
+        return out.raw
+
+    def allgather(self, data):
+        out = ctypes.create_string_buffer(len(data) * self.nranks)
+        src = ctypes.create_string_buffer(bytes(data), len(data))
+        _check(_lib.load().mrv_client_allgather(self._h, src, out, len(data)))
+        return out.raw
+
+    def close(self):
+        if self._h:
+            _lib.load().mrv_client_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        self.close()
+
+
+class Communicator:
+    """One rank's communicator, as returned by MegRay::get_communicator (include/megray.h:33-34).
+
+    Every method takes the device pointers of THIS rank and an optional stream, and must be called
+    from this rank's own thread; it returns when all ranks of the group have made the same call
+    and the work is enqueued.
+    """
+
+    def __init__(self, nranks, rank, backend=Backend.VRANK):
+        self._h = ctypes.c_void_p()
+        self.nranks, self.rank = nranks, rank
+        _check(_lib.load().mrv_comm_create(nranks, rank, int(backend), ctypes.byref(self._h)))
+
+    def init(self, master_ip, port):
+        _check(_lib.load().mrv_comm_init(self._h, master_ip.encode(), port))
+
+    def configure(self, order=FoldOrder.UCX, schedule=Schedule.FUSED):
+        _check(_lib.load().mrv_comm_configure(self._h, int(order), int(schedule)))
+
+    def send(self, sendbuff, length, dtype, rank, stream=None):
+        _check(_lib.load().mrv_comm_send(self._h, _ptr(sendbuff), length, int(dtype), rank, _stream(stream)))
+
+    def recv(self, recvbuff, length, dtype, rank, stream=None):
+        _check(_lib.load().mrv_comm_recv(self._h, _ptr(recvbuff), length, int(dtype), rank, _stream(stream)))
+
+    def scatter(self, sendbuff, recvbuff, recvlen, dtype, root, stream=None):
+        _check(_lib.load().mrv_comm_scatter(self._h, _ptr(sendbuff), _ptr(recvbuff), recvlen, int(dtype), root,
+                                            _stream(stream)))
+
+    def gather(self, sendbuff, recvbuff, sendlen, dtype, root, stream=None):
+        _check(_lib.load().mrv_comm_gather(self._h, _ptr(sendbuff), _ptr(recvbuff), sendlen, int(dtype), root,
+                                           _stream(stream)))
+
+    def all_to_all(self, sendbuff, recvbuff, length, dtype, stream=None):
+        _check(_lib.load().mrv_comm_all_to_all(self._h, _ptr(sendbuff), _ptr(recvbuff), length, int(dtype),
+                                               _stream(stream)))
+
+    def all_gather(self, sendbuff, recvbuff, sendlen, dtype, stream=None):
+        _check(_lib.load().mrv_comm_all_gather(self._h, _ptr(sendbuff), _ptr(recvbuff), sendlen, int(dtype),
+                                               _stream(stream)))
+
+    def all_reduce(self, sendbuff, recvbuff, length, dtype, op, stream=None):
+        _check(_lib.load().mrv_comm_all_reduce(self._h, _ptr(sendbuff), _ptr(recvbuff), length, int(dtype),
+                                               int(op), _stream(stream)))
+
+    def reduce_scatter(self, sendbuff, recvbuff, recvlen, dtype, op, stream=None):
+        _check(_lib.load().mrv_comm_reduce_scatter(self._h, _ptr(sendbuff), _ptr(recvbuff), recvlen, int(dtype),
+                                                   int(op), _stream(stream)))
+
+    def broadcast(self, sendbuff, recvbuff, length, dtype, root, stream=None):
+        _check(_lib.load().mrv_comm_broadcast(self._h, _ptr(sendbuff), _ptr(recvbuff), length, int(dtype), root,
+                                              _stream(stream)))
+
+    def reduce(self, sendbuff, recvbuff, length, dtype, op, root, stream=None):
+        _check(_lib.load().mrv_comm_reduce(self._h, _ptr(sendbuff), _ptr(recvbuff), length, int(dtype), int(op),
+                                           root, _stream(stream)))
+
+    def group_start(self):
+        _check(_lib.load().mrv_comm_group_start(self._h))
+
+    def group_end(self):
+        _check(_lib.load().mrv_comm_group_end(self._h))
+
+    def close(self):
+        if self._h:
+            _lib.load().mrv_comm_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        self.close()
+
+
+def get_communicator(nranks, rank, backend=Backend.VRANK):
+    """MegRay::get_communicator (include/megray.h:33-34); raises 'unknown backend' like src/megray.cpp:56-57."""
+    return Communicator(nranks, rank, backend)

@@ -11,7 +11,8 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(HERE, "libmegray_vrank.so")
 
-HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+HIPCC = os.environ.get("HIPCC", os.path.join(ROCM, "bin", "hipcc"))
 ARCH = "gfx950"
 
 COMMON_FLAGS = [
@@ -36,6 +37,8 @@ def _compile(src):
     cmd = [HIPCC] + COMMON_FLAGS
     if src.endswith(".hip"):
         cmd += ["-x", "hip"] + DEVICE_FLAGS
+    else:  # host-only translation units: plain C++ against the HIP runtime API headers
+        cmd += ["-x", "c++", "-D__HIP_PLATFORM_AMD__=1", "-pthread", f"-I{ROCM}/include"]
     cmd += ["-c", src, "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     return src, obj, proc

@@ -5,8 +5,18 @@
 #include <cstring>
 #include <exception>
 
+#include "megray.h"
+#include "vrank_communicator.h"
 #include "vrank_engine.h"
 #include "vrank_plan.h"
+
+struct mrv_comm {
+    std::shared_ptr<MegRay::Communicator> comm;
+};
+
+struct mrv_client {
+    std::unique_ptr<MegRay::Client> client;
+};
 
 using namespace MegRay;
 using namespace MegRay::vrank;
@@ -28,6 +38,8 @@ int guarded(F&& body) {
             set_error(plan_error());
         } else if (st == MEGRAY_HIP_ERR) {
             set_error("hip error (see the log line on stderr)");
+        } else if (st == MEGRAY_INVALID_USAGE) {
+            set_error("invalid usage (see the log line on stderr)");
         } else if (st != MEGRAY_OK) {
             set_error("error");
         }
@@ -225,6 +237,11 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                 st = plan_broadcast(plan, sendbuffs[root], recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)),
                                     root);
                 break;
+            case MRV_REDUCE:
+                if (root >= nranks) MEGRAY_THROW("root out of range");
+                st = plan_reduce(plan, sendbuffs, recvbuffs[root], nranks, count, reduce_elem_size(dt), as_order(order),
+                                 root);
+                break;
             case MRV_REDUCE2:
                 st = plan_reduce2(plan, sendbuffs[0], sendbuffs[1], recvbuffs[0], count, reduce_elem_size(dt));
                 break;
@@ -278,7 +295,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.new_wins_ties = L.new_wins_ties;
                     run.vector = 2;
                     run.start = fr.start;
-                    run.dir = fr.dir;
+                    run.dir = L.tree ? 0 : fr.dir;
                     run.out_first = fr.out_first;
                     run.tiles = L.tile_hi[s] - L.tile_lo[s];
                     run.reads_recv = (collective == MRV_ALL_REDUCE && fr.start < nranks &&
@@ -290,6 +307,19 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.count = fr.end - fr.begin;
                     emit(run);
                 }
+            } else if (step.kind == Step::kTree) {
+                const TreeLaunch& L = step.tree;
+                mrv_plan_run run;
+                std::memset(&run, 0, sizeof(run));
+                run.step = uint32_t(i);
+                run.nfold = L.nranks;
+                run.nout = 1;
+                run.start = L.root;
+                run.dir = 0;
+                run.out_first = L.root;
+                run.tiles = L.total_tiles;
+                run.count = L.count;
+                emit(run);
             } else {
                 const PackLaunch& L = step.pack;
                 for (uint32_t c = 0; c < L.ncopies; ++c) {
@@ -327,6 +357,169 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
         if (bytes_read) *bytes_read = plan.bytes_read;
         if (bytes_written) *bytes_written = plan.bytes_written;
         return MEGRAY_OK;
+    });
+}
+
+int mrv_reduce_to_root(const void* const* sendbuffs, void* recvbuff_root, uint32_t nranks, size_t len, int dtype,
+                       int op, int order, uint32_t root, void* stream) {
+    return guarded([&] {
+        need(sendbuffs, "sendbuffs is null");
+        return reduce_to_root(sendbuffs, recvbuff_root, nranks, len, static_cast<DType>(dtype),
+                              static_cast<ReduceOp>(op), as_order(order), root, as_stream(stream));
+    });
+}
+
+int mrv_get_free_port(void) {
+    try {
+        return get_free_port();
+    } catch (const std::exception& e) {
+        set_error(e.what());
+        return -1;
+    }
+}
+
+int mrv_create_server(uint32_t nranks, int port) {
+    return guarded([&] { return create_server(nranks, port); });
+}
+
+int mrv_comm_create(uint32_t nranks, uint32_t rank, int backend, mrv_comm** comm) {
+    return guarded([&] {
+        need(comm, "comm is null");
+        *comm = nullptr;
+        auto ptr = get_communicator(nranks, rank, static_cast<Backend>(backend));
+        *comm = new mrv_comm{ptr};
+        return MEGRAY_OK;
+    });
+}
+
+void mrv_comm_destroy(mrv_comm* comm) {
+    delete comm;
+}
+
+int mrv_comm_init(mrv_comm* comm, const char* master_ip, int port) {
+    return guarded([&] {
+        need(comm, "comm is null");
+        need(master_ip, "master_ip is null");
+        return comm->comm->init(master_ip, port);
+    });
+}
+
+int mrv_comm_configure(mrv_comm* comm, int order, int schedule) {
+    return guarded([&] {
+        need(comm, "comm is null");
+        auto* vr = dynamic_cast<VRankCommunicator*>(comm->comm.get());
+        if (!vr) MEGRAY_THROW("not a vrank communicator");
+        vr->set_fold_order(as_order(order));
+        vr->set_schedule(as_schedule(schedule));
+        return MEGRAY_OK;
+    });
+}
+
+#define COMM_CALL(expr)                                               \
+    return guarded([&] {                                              \
+        need(comm, "comm is null");                                   \
+        auto ctx = HipContext::make(as_stream(stream));               \
+        return comm->comm->expr;                                      \
+    })
+
+int mrv_comm_send(mrv_comm* comm, const void* sendbuff, size_t len, int dtype, uint32_t rank, void* stream) {
+    COMM_CALL(send(sendbuff, len, static_cast<DType>(dtype), rank, ctx));
+}
+
+int mrv_comm_recv(mrv_comm* comm, void* recvbuff, size_t len, int dtype, uint32_t rank, void* stream) {
+    COMM_CALL(recv(recvbuff, len, static_cast<DType>(dtype), rank, ctx));
+}
+
+int mrv_comm_scatter(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t recvlen, int dtype, uint32_t root,
+                     void* stream) {
+    COMM_CALL(scatter(sendbuff, recvbuff, recvlen, static_cast<DType>(dtype), root, ctx));
+}
+
+int mrv_comm_gather(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t sendlen, int dtype, uint32_t root,
+                    void* stream) {
+    COMM_CALL(gather(sendbuff, recvbuff, sendlen, static_cast<DType>(dtype), root, ctx));
+}
+
+int mrv_comm_all_to_all(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t len, int dtype, void* stream) {
+    COMM_CALL(all_to_all(sendbuff, recvbuff, len, static_cast<DType>(dtype), ctx));
+}
+
+int mrv_comm_all_gather(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t sendlen, int dtype,
+                        void* stream) {
+    COMM_CALL(all_gather(sendbuff, recvbuff, sendlen, static_cast<DType>(dtype), ctx));
+}
+
+int mrv_comm_all_reduce(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t len, int dtype, int op,
+                        void* stream) {
+    COMM_CALL(all_reduce(sendbuff, recvbuff, len, static_cast<DType>(dtype), static_cast<ReduceOp>(op), ctx));
+}
+
+int mrv_comm_reduce_scatter(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t recvlen, int dtype, int op,
+                            void* stream) {
+    COMM_CALL(reduce_scatter(sendbuff, recvbuff, recvlen, static_cast<DType>(dtype), static_cast<ReduceOp>(op), ctx));
+}
+
+int mrv_comm_broadcast(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t len, int dtype, uint32_t root,
+                       void* stream) {
+    COMM_CALL(broadcast(sendbuff, recvbuff, len, static_cast<DType>(dtype), root, ctx));
+}
+
+int mrv_comm_reduce(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t len, int dtype, int op,
+                    uint32_t root, void* stream) {
+    COMM_CALL(reduce(sendbuff, recvbuff, len, static_cast<DType>(dtype), static_cast<ReduceOp>(op), root, ctx));
+}
+
+int mrv_comm_group_start(mrv_comm* comm) {
+    return guarded([&] {
+        need(comm, "comm is null");
+        return comm->comm->group_start();
+    });
+}
+
+int mrv_comm_group_end(mrv_comm* comm) {
+    return guarded([&] {
+        need(comm, "comm is null");
+        return comm->comm->group_end();
+    });
+}
+
+int mrv_client_create(uint32_t nranks, uint32_t rank, mrv_client** client) {
+    return guarded([&] {
+        need(client, "client is null");
+        *client = new mrv_client{std::make_unique<Client>(nranks, rank)};
+        return MEGRAY_OK;
+    });
+}
+
+void mrv_client_destroy(mrv_client* client) {
+    delete client;
+}
+
+int mrv_client_connect(mrv_client* client, const char* master_ip, int port) {
+    return guarded([&] {
+        need(client, "client is null");
+        return client->client->connect(master_ip, port);
+    });
+}
+
+int mrv_client_barrier(mrv_client* client) {
+    return guarded([&] {
+        need(client, "client is null");
+        return client->client->barrier();
+    });
+}
+
+int mrv_client_broadcast(mrv_client* client, const void* sendbuff, void* recvbuff, size_t len, uint32_t root) {
+    return guarded([&] {
+        need(client, "client is null");
+        return client->client->broadcast(sendbuff, recvbuff, len, root);
+    });
+}
+
+int mrv_client_allgather(mrv_client* client, const void* sendbuff, void* recvbuff, size_t sendlen) {
+    return guarded([&] {
+        need(client, "client is null");
+        return client->client->allgather(sendbuff, recvbuff, sendlen);
     });
 }
 

@@ -1,0 +1,75 @@
+// MEGRAY_VRANK: the MegRay::Communicator backend whose N ranks are virtual ranks inside one
+// process, with all their buffers in one GPU's memory.
+//
+// It takes the place the reference's UcxCommunicator (src/ucx/communicator.h:28-88) and
+// ShmCommunicator (src/shm/communicator.h:84-196) have behind the same abstract class: one object
+// per rank, each driven from its own thread, every rank calling the same collective in the same
+// order.  A collective call deposits this rank's buffers and stream with the group and waits for
+// the other ranks; the last rank to arrive plans the whole collective and enqueues it, after which
+// every rank's stream is ordered behind the result.  Calls return once the work is enqueued
+// (stream-asynchronous, like the reference's NCCL backend, src/nccl/communicator.cpp:175-186).
+#pragma once
+
+#include <memory>
+#include <vector>
+
+#include "megray/communicator.h"
+#include "vrank_plan.h"
+
+namespace MegRay {
+
+namespace vrank {
+class Group;
+struct PendingP2P;
+}  // namespace vrank
+
+class VRankCommunicator final : public Communicator {
+public:
+    VRankCommunicator(uint32_t nranks, uint32_t rank);
+    ~VRankCommunicator();
+
+    Status do_init() override;
+    Status do_init(BcastCallback cb) override;
+
+    Status scatter(const void* sendbuff, void* recvbuff, size_t recvlen, DType dtype, uint32_t root,
+                   std::shared_ptr<Context> ctx) override;
+    Status gather(const void* sendbuff, void* recvbuff, size_t sendlen, DType dtype, uint32_t root,
+                  std::shared_ptr<Context> ctx) override;
+    Status all_to_all(const void* sendbuff, void* recvbuff, size_t len, DType dtype,
+                      std::shared_ptr<Context> ctx) override;
+    Status all_gather(const void* sendbuff, void* recvbuff, size_t sendlen, DType dtype,
+                      std::shared_ptr<Context> ctx) override;
+    Status all_reduce(const void* sendbuff, void* recvbuff, size_t len, DType dtype, ReduceOp op,
+                      std::shared_ptr<Context> ctx) override;
+    Status reduce_scatter(const void* sendbuff, void* recvbuff, size_t recvlen, DType dtype, ReduceOp op,
+                          std::shared_ptr<Context> ctx) override;
+    Status broadcast(const void* sendbuff, void* recvbuff, size_t len, DType dtype, uint32_t root,
+                     std::shared_ptr<Context> ctx) override;
+    Status reduce(const void* sendbuff, void* recvbuff, size_t len, DType dtype, ReduceOp op, uint32_t root,
+                  std::shared_ptr<Context> ctx) override;
+    Status group_start() override;
+    Status group_end() override;
+
+    // Not part of the reference API: which reference loop's combination order all_reduce /
+    // reduce_scatter / reduce reproduce (default: the ucx ring), and how all_reduce is laid out in
+    // launches (default: fused).  Every rank of a group must choose the same.
+    void set_fold_order(vrank::FoldOrder order) { m_order = order; }
+    void set_schedule(vrank::Schedule sched) { m_sched = sched; }
+
+protected:
+    Status _send(const void* sendbuff, size_t size, uint32_t rank, std::shared_ptr<Context> ctx) override;
+    Status _recv(void* recvbuf, size_t size, uint32_t rank, std::shared_ptr<Context> ctx) override;
+
+private:
+    Status join(const uint64_t id[2]);
+    Status p2p(bool is_send, const void* sendbuff, void* recvbuff, size_t size, uint32_t peer,
+               std::shared_ptr<Context> ctx);
+
+    std::shared_ptr<vrank::Group> m_group;
+    vrank::FoldOrder m_order = vrank::kOrderUcx;
+    vrank::Schedule m_sched = vrank::kSchedFused;
+    bool m_grouping = false;
+    std::vector<std::shared_ptr<vrank::PendingP2P>> m_pending;
+};
+
+}  // namespace MegRay

@@ -36,6 +36,8 @@ Status execute(const Plan& plan, DType dtype, ReduceOp op, hipStream_t stream) {
             HIP_CHECK(launch_fold(step.fold, dtype, op, stream));
         } else if (step.kind == Step::kFlat) {
             HIP_CHECK(launch_flat(step.flat, dtype, op, stream));
+        } else if (step.kind == Step::kTree) {
+            HIP_CHECK(launch_tree(step.tree, dtype, op, stream));
         } else {
             HIP_CHECK(launch_pack(step.pack, stream));
         }
@@ -70,6 +72,15 @@ Status reduce_scatter(const void* const* send, void* const* recv, uint32_t nrank
     check_reduce_op(op);
     Plan plan;
     Status st = plan_reduce_scatter(plan, send, recv, nranks, recvlen, size, order, kSchedFused);
+    return st == MEGRAY_OK ? execute(plan, dtype, op, stream) : st;
+}
+
+Status reduce_to_root(const void* const* send, void* recv_root, uint32_t nranks, size_t len, DType dtype,
+                      ReduceOp op, FoldOrder order, uint32_t root, hipStream_t stream) {
+    const uint32_t size = reduce_elem_size(dtype);
+    check_reduce_op(op);
+    Plan plan;
+    Status st = plan_reduce(plan, send, recv_root, nranks, len, size, order, root);
     return st == MEGRAY_OK ? execute(plan, dtype, op, stream) : st;
 }
 

@@ -29,6 +29,8 @@ Status all_reduce(const void* const* send, void* const* recv, uint32_t nranks, s
                   ReduceOp op, FoldOrder order, Schedule sched, hipStream_t stream);
 Status reduce_scatter(const void* const* send, void* const* recv, uint32_t nranks, size_t recvlen,
                       DType dtype, ReduceOp op, FoldOrder order, hipStream_t stream);
+Status reduce_to_root(const void* const* send, void* recv_root, uint32_t nranks, size_t len, DType dtype,
+                      ReduceOp op, FoldOrder order, uint32_t root, hipStream_t stream);
 Status all_gather(const void* const* send, void* const* recv, uint32_t nranks, size_t sendlen, DType dtype,
                   hipStream_t stream);
 Status all_to_all(const void* const* send, void* const* recv, uint32_t nranks, size_t len, DType dtype,

@@ -1,0 +1,587 @@
+// Templates of the fold kernels of the virtual-rank backend (gfx950).  Included by one translation
+// unit per element type (vrank_fold_<type>.hip), each of which instantiates the launchers for its
+// type, so that the types compile in parallel.
+//
+// fold_kernel / fold_flat_kernel / fold_tree_kernel
+//              : every output element is a combination, in a fixed rank order, of the same element
+//                of K input buffers, stored to M output buffers.  They replace the 2-input
+//                reduce_{sum,max,min}_kernel of the reference (src/ucx/kernel.cu:16-38) and the
+//                cpu_reduce_kernel loop (src/shm/utils.cpp:16-37): a whole ring of N-1 two-input
+//                steps on one chunk is one pass here, the ring order surviving as the fold order.
+//                fold_flat_kernel is the fast form for K == rank count on aligned buffers;
+//                fold_kernel takes everything else (any K, unaligned buffers, shifted copies);
+//                fold_tree_kernel is the element-wise binomial tree for arbitrary rank counts.
+//
+// All are pure streaming kernels: HBM-bound, one 128-bit access per lane per buffer, no LDS, no
+// matrix instructions.  A workgroup is ONE 64-wide wavefront whose lanes read consecutive 16-byte
+// vectors, so every load and store instruction covers one contiguous KiB and a tile is 1 KiB per
+// buffer: on MI355X many small tiles sustain more HBM bandwidth than fewer large ones.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <type_traits>
+
+#include "vrank_kernels.h"
+
+namespace MegRay {
+namespace vrank {
+namespace detail {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+enum : int { kSum = 0, kMax = 1, kMin = 2, kCopy = 3 };
+
+// Accumulator type: FLOAT16 is widened to fp32, folded there and rounded once at the end.
+template <typename T>
+struct Wide {
+    using type = T;
+};
+template <>
+struct Wide<_Float16> {
+    using type = float;
+};
+
+template <int OP, typename A>
+__device__ __forceinline__ A combine(A acc, A x, bool new_wins) {
+    if constexpr (OP == kSum) {
+        return static_cast<A>(acc + x);  // unsigned element types: wraps
+    } else if constexpr (OP == kMax) {
+        if constexpr (std::is_floating_point<A>::value) {
+            // explicit compare + select: ties, +-0 and NaN follow the reference's ?: exactly
+            return new_wins ? ((acc > x) ? acc : x) : ((x > acc) ? x : acc);
+        } else {
+            return (x > acc) ? x : acc;
+        }
+    } else if constexpr (OP == kMin) {
+        if constexpr (std::is_floating_point<A>::value) {
+            return new_wins ? ((acc < x) ? acc : x) : ((x < acc) ? x : acc);
+        } else {
+            return (x < acc) ? x : acc;
+        }
+    } else {
+        return x;
+    }
+}
+
+template <typename T>
+union VecOf {
+    u32x4 raw;
+    T v[kVecBytes / sizeof(T)];
+};
+
+__device__ __forceinline__ u32x4 load_vec(const char* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
+__device__ __forceinline__ void store_vec(char* p, u32x4 x) {
+    __builtin_nontemporal_store(x, reinterpret_cast<u32x4*>(p));
+}
+
+__device__ __forceinline__ uint32_t rotate_rank(uint32_t start, int dir, uint32_t j, uint32_t n) {
+    // (start + dir*j) mod n for j < n, without a division
+    if (dir > 0) {
+        uint32_t r = start + j;
+        return r >= n ? r - n : r;
+    }
+    return start >= j ? start - j : start + n - j;
+}
+
+template <typename T, int OP>
+__device__ __forceinline__ u32x4 fold_vec(u32x4 acc_raw, u32x4 x_raw, bool new_wins) {
+    using A = typename Wide<T>::type;
+    VecOf<T> a, x;
+    a.raw = acc_raw;
+    x.raw = x_raw;
+#pragma unroll
+    for (uint32_t e = 0; e < kVecBytes / sizeof(T); ++e)
+        a.v[e] = static_cast<T>(combine<OP, A>(static_cast<A>(a.v[e]), static_cast<A>(x.v[e]), new_wins));
+    return a.raw;
+}
+
+// FLOAT16 keeps its accumulators in fp32 across the whole fold.
+template <int OP>
+struct HalfAcc {
+    float v[8];
+    __device__ __forceinline__ void seed(u32x4 raw) {
+        VecOf<_Float16> x;
+        x.raw = raw;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = static_cast<float>(x.v[e]);
+    }
+    __device__ __forceinline__ void fold(u32x4 raw, bool new_wins) {
+        VecOf<_Float16> x;
+        x.raw = raw;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = combine<OP, float>(v[e], static_cast<float>(x.v[e]), new_wins);
+    }
+    __device__ __forceinline__ void merge(const HalfAcc& other) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = combine<OP, float>(v[e], other.v[e], false);
+    }
+    __device__ __forceinline__ u32x4 finish() const {
+        VecOf<_Float16> x;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x.v[e] = static_cast<_Float16>(v[e]);
+        return x.raw;
+    }
+};
+
+template <typename T, int OP>
+struct VecAcc {
+    u32x4 raw;
+    __device__ __forceinline__ void seed(u32x4 r) { raw = r; }
+    __device__ __forceinline__ void fold(u32x4 r, bool new_wins) { raw = fold_vec<T, OP>(raw, r, new_wins); }
+    __device__ __forceinline__ void merge(const VecAcc& other) { raw = fold_vec<T, OP>(raw, other.raw, false); }
+    __device__ __forceinline__ u32x4 finish() const { return raw; }
+};
+
+// int8 / uint8: the sixteen bytes of a vector are kept as 2 x 4 registers of packed 16-bit lanes
+// (even bytes and odd bytes of each 32-bit word, sign- or zero-extended), so that one packed
+// 16-bit add / max / min handles two elements.  SUM wraps mod 256 because only the low byte of
+// each lane is kept at the end.
+typedef int16_t i16x2 __attribute__((ext_vector_type(2)));
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+
+template <typename T, int OP>
+struct ByteAcc {
+    using Lanes = typename std::conditional<std::is_signed<T>::value, i16x2, u16x2>::type;
+    Lanes even[4], odd[4];
+
+    static __device__ __forceinline__ void split(uint32_t w, Lanes& ev, Lanes& od) {
+        if constexpr (std::is_signed<T>::value) {
+            const i16x2 lanes = __builtin_bit_cast(i16x2, w);
+            ev = (lanes << 8) >> 8;  // arithmetic shift: sign-extends the low byte of each lane
+            od = lanes >> 8;
+        } else {
+            ev = __builtin_bit_cast(u16x2, w & 0x00ff00ffu);
+            od = __builtin_bit_cast(u16x2, (w >> 8) & 0x00ff00ffu);
+        }
+    }
+    static __device__ __forceinline__ Lanes op(Lanes a, Lanes b) {
+        if constexpr (OP == kSum) {
+            return a + b;
+        } else if constexpr (OP == kMax) {
+            return __builtin_elementwise_max(a, b);
+        } else {
+            return __builtin_elementwise_min(a, b);
+        }
+    }
+    __device__ __forceinline__ void seed(u32x4 raw) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) split(raw[w], even[w], odd[w]);
+    }
+    __device__ __forceinline__ void fold(u32x4 raw, bool) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            Lanes ev, od;
+            split(raw[w], ev, od);
+            even[w] = op(even[w], ev);
+            odd[w] = op(odd[w], od);
+        }
+    }
+    __device__ __forceinline__ void merge(const ByteAcc& other) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            even[w] = op(even[w], other.even[w]);
+            odd[w] = op(odd[w], other.odd[w]);
+        }
+    }
+    __device__ __forceinline__ u32x4 finish() const {
+        u32x4 raw;
+#pragma unroll
+        for (int w = 0; w < 4; ++w)
+            raw[w] = (__builtin_bit_cast(uint32_t, even[w]) & 0x00ff00ffu) |
+                     ((__builtin_bit_cast(uint32_t, odd[w]) & 0x00ff00ffu) << 8);
+        return raw;
+    }
+};
+
+// Left folds keep one accumulator, and for bytes the plain element-wise form measured faster; the
+// tree keeps K accumulators alive, where the packed byte form is what fits the register file.
+template <typename T, int OP>
+using AccFor = typename std::conditional<std::is_same<T, _Float16>::value, HalfAcc<OP>, VecAcc<T, OP>>::type;
+
+template <typename T, int OP>
+using TreeAccFor = typename std::conditional<sizeof(T) == 1, ByteAcc<T, OP>, AccFor<T, OP>>::type;
+
+// K > 0: fold count known at compile time, all K loads of a lane are issued before the first use.
+// K == 0: fold count read from the launch, loads issued in groups of four.
+template <typename T, int OP, int K, int U>
+__global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
+    using A = typename Wide<T>::type;
+    constexpr uint32_t EPV = kVecBytes / sizeof(T);
+    const uint32_t tile = blockIdx.x;
+    // segment lookup: first_tile is ascending and padded with 0xffffffff, so the segment is the
+    // number of entries <= tile, minus one; eight entries per scalar load
+    uint32_t s = 0;
+    for (uint32_t base = 0; base < L.nseg; base += 8) {
+#pragma unroll
+        for (uint32_t i = 0; i < 8; ++i) s += L.first_tile[base + i] <= tile ? 1u : 0u;
+    }
+    s -= 1;
+    const uint64_t in_begin = L.seg[s].in_begin;
+    const uint64_t out_begin = L.seg[s].out_begin;
+    const uint64_t count = L.seg[s].count;
+    const uint32_t local_tile = tile - L.first_tile[s];
+    const uint32_t start = L.seg[s].start;
+    const int dir = L.seg[s].dir;
+    const uint32_t out_first = L.seg[s].out_first;
+    const bool vector = (L.seg[s].flags & kSegVector) != 0;
+    const uint32_t nr = L.nranks;
+    const uint32_t nfold = K > 0 ? uint32_t(K) : L.nfold;
+    const uint32_t nout = L.nout;
+    const bool new_wins = L.new_wins_ties != 0;
+    const uint32_t tid = threadIdx.x;
+
+    if (vector) {
+        const uint64_t nvec = count / EPV;
+        const uint64_t vbase = uint64_t(local_tile) * (kThreads * U);
+        const uint64_t in_off = in_begin * sizeof(T) + vbase * kVecBytes;
+        const uint64_t out_off = out_begin * sizeof(T) + vbase * kVecBytes;
+        const uint64_t left = nvec - vbase;  // vectors from this tile's start to the segment's end
+        AccFor<T, OP> acc[U];
+        if (left >= uint64_t(kThreads) * U) {
+            // full tile: no predicates
+            if constexpr (K > 0) {
+                u32x4 x[K][U];
+#pragma unroll
+                for (int j = 0; j < K; ++j) {
+                    const char* src = static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off;
+#pragma unroll
+                    for (int u = 0; u < U; ++u) x[j][u] = load_vec(src + (u * kThreads + tid) * kVecBytes);
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    acc[u].seed(x[0][u]);
+#pragma unroll
+                    for (int j = 1; j < K; ++j) acc[u].fold(x[j][u], new_wins);
+                }
+            } else {
+                {
+                    const char* src = static_cast<const char*>(L.in[start]) + in_off;
+#pragma unroll
+                    for (int u = 0; u < U; ++u) acc[u].seed(load_vec(src + (u * kThreads + tid) * kVecBytes));
+                }
+                uint32_t j = 1;
+                for (; j + 4 <= nfold; j += 4) {
+                    u32x4 x[4][U];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const char* src =
+                                static_cast<const char*>(L.in[rotate_rank(start, dir, j + q, nr)]) + in_off;
+#pragma unroll
+                        for (int u = 0; u < U; ++u) x[q][u] = load_vec(src + (u * kThreads + tid) * kVecBytes);
+                    }
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+#pragma unroll
+                        for (int u = 0; u < U; ++u) acc[u].fold(x[q][u], new_wins);
+                }
+                for (; j < nfold; ++j) {
+                    const char* src = static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off;
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+                        acc[u].fold(load_vec(src + (u * kThreads + tid) * kVecBytes), new_wins);
+                }
+            }
+            u32x4 res[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) res[u] = acc[u].finish();
+            for (uint32_t m = 0; m < nout; ++m) {
+                char* dst = static_cast<char*>(L.out[rotate_rank(out_first, 1, m, nr)]) + out_off;
+#pragma unroll
+                for (int u = 0; u < U; ++u) store_vec(dst + (u * kThreads + tid) * kVecBytes, res[u]);
+            }
+        } else {
+            // last tile of the segment: predicate every vector
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const uint32_t v = u * kThreads + tid;
+                if (v < left) {
+                    AccFor<T, OP> a;
+                    a.seed(load_vec(static_cast<const char*>(L.in[start]) + in_off + v * kVecBytes));
+                    for (uint32_t j = 1; j < nfold; ++j)
+                        a.fold(load_vec(static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off +
+                                        v * kVecBytes),
+                               new_wins);
+                    const u32x4 r = a.finish();
+                    for (uint32_t m = 0; m < nout; ++m)
+                        store_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, nr)]) + out_off +
+                                          v * kVecBytes,
+                                  r);
+                }
+            }
+        }
+    } else {
+        // element tiles: chunk heads / tails and buffers that are not 16-byte aligned
+        const uint64_t ebase = uint64_t(local_tile) * (kThreads * U);
+        const uint64_t left = count - ebase;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t e = u * kThreads + tid;
+            if (e < left) {
+                const uint64_t ie = in_begin + ebase + e;
+                const uint64_t oe = out_begin + ebase + e;
+                A a = static_cast<A>(static_cast<const T*>(L.in[start])[ie]);
+                for (uint32_t j = 1; j < nfold; ++j)
+                    a = combine<OP, A>(
+                            a, static_cast<A>(static_cast<const T*>(L.in[rotate_rank(start, dir, j, nr)])[ie]),
+                            new_wins);
+                const T r = static_cast<T>(a);
+                for (uint32_t m = 0; m < nout; ++m) static_cast<T*>(L.out[rotate_rank(out_first, 1, m, nr)])[oe] = r;
+            }
+        }
+    }
+}
+
+
+// ---------------------------------------------------------------------------------------------
+// Flat fold: tile t covers bytes [1024 t, 1024 t + 1024) of every input, whatever run it is in.
+// The K loads of a lane therefore depend on nothing but blockIdx and the kernel arguments and are
+// issued first; the run lookup (fold order, destinations) happens while they are in flight.
+
+template <typename T, int OP, int K, int START, int DIR>
+__device__ __forceinline__ u32x4 fold_static(const u32x4 (&x)[K], bool new_wins) {
+    AccFor<T, OP> acc;
+    acc.seed(x[START]);
+#pragma unroll
+    for (int j = 1; j < K; ++j) acc.fold(x[((START + DIR * j) % K + K) % K], new_wins);
+    return acc.finish();
+}
+
+// Uniform dispatch on the seed rank: each case is a straight-line fold with fixed registers.
+template <typename T, int OP, int K, int S = 0>
+__device__ __forceinline__ u32x4 fold_from(const u32x4 (&x)[K], uint32_t start, int dir, bool new_wins) {
+    if constexpr (S == K - 1) {
+        return dir > 0 ? fold_static<T, OP, K, S, 1>(x, new_wins) : fold_static<T, OP, K, S, -1>(x, new_wins);
+    } else {
+        if (start == S)
+            return dir > 0 ? fold_static<T, OP, K, S, 1>(x, new_wins) : fold_static<T, OP, K, S, -1>(x, new_wins);
+        return fold_from<T, OP, K, S + 1>(x, start, dir, new_wins);
+    }
+}
+
+// Binomial tree towards virtual rank 0 = actual rank ROOT (src/ucx/reduce.cpp:56-80): in round
+// `bit`, virtual rank v (a multiple of 2*bit) takes in v + bit as reduce(incoming, own), which
+// keeps its own value on a MAX/MIN tie.
+template <typename T, int OP, int K, int ROOT>
+__device__ __forceinline__ u32x4 tree_static(const u32x4 (&x)[K]) {
+    TreeAccFor<T, OP> a[K];
+#pragma unroll
+    for (int v = 0; v < K; ++v) a[v].seed(x[(v + ROOT) % K]);
+#pragma unroll
+    for (int bit = 1; bit < K; bit <<= 1) {
+#pragma unroll
+        for (int v = 0; v + bit < K; v += 2 * bit) a[v].merge(a[v + bit]);
+    }
+    return a[0].finish();
+}
+
+template <typename T, int OP, int K, int S = 0>
+__device__ __forceinline__ u32x4 tree_from(const u32x4 (&x)[K], uint32_t root) {
+    if constexpr (S == K - 1) {
+        return tree_static<T, OP, K, S>(x);
+    } else {
+        if (root == S) return tree_static<T, OP, K, S>(x);
+        return tree_from<T, OP, K, S + 1>(x, root);
+    }
+}
+
+// The same tree on one element.  N > 0: rank count known at compile time (registers only);
+// N == 0: read from `n` (the element-wise kernel for arbitrary rank counts).
+template <typename T, int OP, int N, typename Launch>
+__device__ __forceinline__ T tree_element(const Launch& L, uint32_t n, uint32_t root, uint64_t el) {
+    using A = typename Wide<T>::type;
+    constexpr uint32_t CAP = N > 0 ? uint32_t(N) : kMaxRanks;
+    const uint32_t count = N > 0 ? uint32_t(N) : n;
+    A a[CAP];
+#pragma unroll
+    for (uint32_t v = 0; v < CAP; ++v)
+        if (v < count) a[v] = static_cast<A>(static_cast<const T*>(L.in[rotate_rank(root, 1, v, count)])[el]);
+#pragma unroll
+    for (uint32_t bit = 1; bit < CAP; bit <<= 1) {
+#pragma unroll
+        for (uint32_t v = 0; v + bit < CAP; v += 2 * bit)
+            if (v + bit < count) a[v] = combine<OP, A>(a[v], a[v + bit], false);
+    }
+    return static_cast<T>(a[0]);
+}
+
+template <typename T, int OP>
+__global__ void __launch_bounds__(kThreads) fold_tree_kernel(const TreeLaunch L) {
+    const uint64_t el = uint64_t(blockIdx.x) * kThreads + threadIdx.x;
+    if (el < L.count) static_cast<T*>(L.out)[el] = tree_element<T, OP, 0>(L, L.nranks, L.root, el);
+}
+
+// TREE selects the binomial-tree combination; it is a template parameter, not a run-time branch,
+// so that the tree's K live accumulators do not cost the left fold any registers.
+template <typename T, int OP, int K, bool TREE>
+__global__ void __launch_bounds__(kThreads) fold_flat_kernel(const FlatLaunch L) {
+    using A = typename Wide<T>::type;
+    constexpr uint32_t EPV = kVecBytes / sizeof(T);
+    constexpr uint32_t TILE = kThreads * EPV;  // elements per tile
+    const uint32_t tile = blockIdx.x;
+    const uint32_t tid = threadIdx.x;
+    const uint64_t byte_off = (uint64_t(tile) * kThreads + tid) * kVecBytes;
+    const bool whole = (uint64_t(tile) + 1) * TILE <= L.count;  // tile lies inside the buffer
+
+    u32x4 x[K];
+    if (whole) {
+#pragma unroll
+        for (int r = 0; r < K; ++r) x[r] = load_vec(static_cast<const char*>(L.in[r]) + byte_off);
+    }
+
+    // run lookup, eight runs per pair of scalar loads
+    int run = -1;
+    for (uint32_t base = 0; base < L.nruns; base += 8) {
+#pragma unroll
+        for (uint32_t i = 0; i < 8; ++i)
+            if (tile >= L.tile_lo[base + i] && tile < L.tile_hi[base + i]) run = int(base + i);
+    }
+    const bool new_wins = L.new_wins_ties != 0;
+    const uint32_t nout = L.nout;
+
+    if (run >= 0) {
+        // the whole tile shares one fold order (and lies inside the buffer)
+        const uint32_t start = L.run[run].start;
+        const int dir = L.run[run].dir;
+        const uint32_t out_first = L.run[run].out_first;
+        const uint64_t out_off = byte_off - uint64_t(L.run[run].out_shift) * sizeof(T);
+        u32x4 res;
+        if constexpr (TREE) {
+            res = tree_from<T, OP, K>(x, start);
+        } else {
+            res = fold_from<T, OP, K>(x, start, dir, new_wins);
+        }
+        if (nout == uint32_t(K)) {
+#pragma unroll
+            for (int m = 0; m < K; ++m) store_vec(static_cast<char*>(L.out[m]) + out_off, res);
+        } else {
+            for (uint32_t m = 0; m < nout; ++m)
+                store_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, K)]) + out_off, res);
+        }
+        return;
+    }
+
+    // A tile that straddles a run border or the end of the buffer: element by element, one run at a
+    // time so that ranks and destinations stay uniform.
+    const uint64_t e_lo = uint64_t(tile) * TILE;
+    const uint64_t e_hi = e_lo + TILE < L.count ? e_lo + TILE : L.count;
+    for (uint32_t i = 0; i < L.nruns; ++i) {
+        const uint64_t b = L.run[i].begin > e_lo ? L.run[i].begin : e_lo;
+        const uint64_t e = L.run[i].end < e_hi ? L.run[i].end : e_hi;
+        if (b >= e) continue;
+        const uint32_t start = L.run[i].start;
+        const int dir = L.run[i].dir;
+        const uint32_t out_first = L.run[i].out_first;
+        const uint64_t shift = uint64_t(L.run[i].out_shift);
+        for (uint32_t k = 0; k < EPV; ++k) {
+            const uint64_t el = e_lo + uint64_t(tid) * EPV + k;
+            if (el < b || el >= e) continue;
+            T r;
+            if constexpr (TREE) {
+                r = tree_element<T, OP, K>(L, K, start, el);
+            } else {
+                A a = static_cast<A>(static_cast<const T*>(L.in[start])[el]);
+                for (uint32_t j = 1; j < uint32_t(K); ++j)
+                    a = combine<OP, A>(
+                            a, static_cast<A>(static_cast<const T*>(L.in[rotate_rank(start, dir, j, K)])[el]),
+                            new_wins);
+                r = static_cast<T>(a);
+            }
+            for (uint32_t m = 0; m < nout; ++m)
+                static_cast<T*>(L.out[rotate_rank(out_first, 1, m, K)])[el - shift] = r;
+        }
+    }
+}
+
+
+// ---------------------------------------------------------------------------------------------
+// Launchers for one element type.  `op` is kSum / kMax / kMin; SUM exists for the unsigned and the
+// floating types only (a signed integer SUM runs on its unsigned twin: two's-complement wrap).
+
+using FoldFn = void (*)(const FoldLaunch);
+using FlatFn = void (*)(const FlatLaunch);
+using TreeFn = void (*)(const TreeLaunch);
+
+template <typename T>
+constexpr bool has_sum() {
+    return !(std::is_integral<T>::value && std::is_signed<T>::value);
+}
+
+template <typename T, int OP>
+FoldFn pick_fold(uint32_t nfold) {
+    switch (nfold) {
+        case 2: return fold_kernel<T, OP, 2, fold_unroll(2)>;
+        case 3: return fold_kernel<T, OP, 3, fold_unroll(3)>;
+        case 4: return fold_kernel<T, OP, 4, fold_unroll(4)>;
+        case 8: return fold_kernel<T, OP, 8, fold_unroll(8)>;
+        default: return fold_kernel<T, OP, 0, fold_unroll(0)>;
+    }
+}
+
+template <typename T, int OP, bool TREE>
+FlatFn pick_flat_k(uint32_t nranks) {
+    switch (nranks) {
+        case 2: return fold_flat_kernel<T, OP, 2, TREE>;
+        case 3: return fold_flat_kernel<T, OP, 3, TREE>;
+        case 4: return fold_flat_kernel<T, OP, 4, TREE>;
+        case 8: return fold_flat_kernel<T, OP, 8, TREE>;
+        default: return nullptr;
+    }
+}
+
+template <typename T, int OP>
+FlatFn pick_flat(const FlatLaunch& L) {
+    return L.tree ? pick_flat_k<T, OP, true>(L.nranks) : pick_flat_k<T, OP, false>(L.nranks);
+}
+
+template <typename T>
+hipError_t launch_fold_t(const FoldLaunch& L, int op, hipStream_t stream) {
+    FoldFn fn = nullptr;
+    if (op == kMax) fn = pick_fold<T, kMax>(L.nfold);
+    if (op == kMin) fn = pick_fold<T, kMin>(L.nfold);
+    if constexpr (has_sum<T>()) {
+        if (op == kSum) fn = pick_fold<T, kSum>(L.nfold);
+    }
+    if (!fn) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(fn, dim3(L.total_tiles), dim3(kThreads), 0, stream, L);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_flat_t(const FlatLaunch& L, int op, hipStream_t stream) {
+    FlatFn fn = nullptr;
+    if (op == kMax) fn = pick_flat<T, kMax>(L);
+    if (op == kMin) fn = pick_flat<T, kMin>(L);
+    if constexpr (has_sum<T>()) {
+        if (op == kSum) fn = pick_flat<T, kSum>(L);
+    }
+    if (!fn) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(fn, dim3(L.total_tiles), dim3(kThreads), 0, stream, L);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_tree_t(const TreeLaunch& L, int op, hipStream_t stream) {
+    TreeFn fn = nullptr;
+    if (op == kMax) fn = fold_tree_kernel<T, kMax>;
+    if (op == kMin) fn = fold_tree_kernel<T, kMin>;
+    if constexpr (has_sum<T>()) {
+        if (op == kSum) fn = fold_tree_kernel<T, kSum>;
+    }
+    if (!fn) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(fn, dim3(L.total_tiles), dim3(kThreads), 0, stream, L);
+    return hipGetLastError();
+}
+
+// Defines the three launchers of element type T in the including translation unit.
+#define MEGRAY_VRANK_INSTANTIATE(T)                                                             \
+    template hipError_t launch_fold_t<T>(const FoldLaunch&, int, hipStream_t);                  \
+    template hipError_t launch_flat_t<T>(const FlatLaunch&, int, hipStream_t);                  \
+    template hipError_t launch_tree_t<T>(const TreeLaunch&, int, hipStream_t);
+
+}  // namespace detail
+}  // namespace vrank
+}  // namespace MegRay

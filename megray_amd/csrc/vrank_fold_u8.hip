@@ -1,0 +1,10 @@
+// Fold kernels for element type uint8_t (see vrank_fold_impl.hpp).
+#include "vrank_fold_impl.hpp"
+
+namespace MegRay {
+namespace vrank {
+namespace detail {
+MEGRAY_VRANK_INSTANTIATE(uint8_t)
+}  // namespace detail
+}  // namespace vrank
+}  // namespace MegRay

@@ -65,6 +65,15 @@ public:
         m_runs.clear();
     }
 
+    // Tree combination towards rank `root` of one whole buffer: a flat launch if the shape allows.
+    bool finish_tree(uint64_t count, uint8_t root) {
+        add_run(0, 0, count, root, 1, root);
+        m_tree = true;
+        const bool ok = emit_flat();
+        m_runs.clear();
+        return ok;
+    }
+
 private:
     struct Run {
         uint64_t in_begin, out_begin, count;
@@ -117,6 +126,7 @@ private:
         L.total_tiles = uint32_t(total);
         L.new_wins_ties = m_new_wins ? 1 : 0;
         L.elem_size = m_elem;
+        L.tree = m_tree ? 1 : 0;
         m_plan.steps.push_back(step);
         return true;
     }
@@ -200,6 +210,7 @@ private:
     uint32_t m_nranks, m_nfold, m_nout, m_elem;
     bool m_new_wins;
     bool m_aligned;
+    bool m_tree = false;
     std::vector<Run> m_runs;
     FoldLaunch m_launch;
 };
@@ -539,6 +550,55 @@ Status plan_broadcast(Plan& plan, const void* send_root, void* const* recv, uint
     FoldBuilder copy(plan, in, recv, nranks, 1, nranks, elem_size, false);
     copy.add_run(0, 0, len, uint8_t(root), 1, 0);
     copy.finish();
+    return MEGRAY_OK;
+}
+
+Status plan_reduce(Plan& plan, const void* const* send, void* recv_root, uint32_t nranks, uint64_t len,
+                   uint32_t elem_size, FoldOrder order, uint32_t root) {
+    PLAN_TRY(check_ranks(nranks));
+    PLAN_TRY(check_elem(elem_size));
+    if (order < 0 || order >= kOrderCount) return invalid("unknown fold order");
+    if (root >= nranks) return invalid("root out of range");
+    const uint64_t bytes = len * elem_size;
+    for (uint32_t b = 0; b < nranks; ++b)
+        if (overlaps(recv_root, bytes, send[b], bytes) && !(b == root && recv_root == send[b]))
+            return invalid("the root's receive buffer overlaps a send buffer out of place");
+    void* out[kMaxRanks] = {};
+    out[root] = recv_root;
+    if (order == kOrderUcx) {
+        if (!len) return MEGRAY_OK;
+        const uint64_t before_r = plan.bytes_read, before_w = plan.bytes_written;
+        FoldBuilder fold(plan, send, out, nranks, nranks, 1, elem_size, false);
+        if (fold.finish_tree(len, uint8_t(root))) return MEGRAY_OK;
+        plan.bytes_read = before_r + bytes * nranks;
+        plan.bytes_written = before_w + bytes;
+        Step step;
+        std::memset(&step, 0, sizeof(step));
+        step.kind = Step::kTree;
+        TreeLaunch& L = step.tree;
+        for (uint32_t r = 0; r < nranks; ++r) L.in[r] = send[r];
+        L.out = recv_root;
+        L.count = len;
+        L.nranks = nranks;
+        L.root = root;
+        L.elem_size = elem_size;
+        const uint64_t tiles = (len + kThreads - 1) / kThreads;
+        if (tiles > 0x7fffffffull) return invalid("buffer too large for one tree launch");
+        L.total_tiles = uint32_t(tiles);
+        plan.steps.push_back(step);
+        return MEGRAY_OK;
+    }
+    const uint32_t nchunks = order_chunks(order, nranks);
+    uint64_t sizes[kMaxChunks], offs[kMaxChunks];
+    chunk_partition(len, nchunks, sizes, offs);
+    FoldBuilder fold(plan, send, out, nranks, nranks, 1, elem_size, false);
+    for (uint32_t c = 0; c < nchunks; ++c) {
+        uint8_t start, owner;
+        int8_t dir;
+        chunk_fold_order(kAllReduce, order, nranks, c, &start, &dir, &owner);
+        fold.add_run(offs[c], offs[c], sizes[c], start, dir, uint8_t(root));
+    }
+    fold.finish();
     return MEGRAY_OK;
 }
 

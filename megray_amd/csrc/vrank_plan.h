@@ -37,10 +37,11 @@ enum Schedule : int {
 enum Collective : int { kAllReduce = 0, kReduceScatter = 1 };
 
 struct Step {
-    enum Kind : int { kFold = 0, kPack = 1, kFlat = 2 } kind;
+    enum Kind : int { kFold = 0, kPack = 1, kFlat = 2, kTree = 3 } kind;
     FoldLaunch fold;
     PackLaunch pack;
     FlatLaunch flat;
+    TreeLaunch tree;
 };
 
 struct Plan {
@@ -80,6 +81,10 @@ Status plan_gather(Plan& plan, const void* const* send, void* recv_root, uint32_
                    uint32_t elem_size, uint32_t root);
 Status plan_broadcast(Plan& plan, const void* send_root, void* const* recv, uint32_t nranks, uint64_t len,
                       uint32_t elem_size, uint32_t root);
+// recv_root = combination of send[*] on rank `root`.  kOrderUcx: the binomial tree of
+// src/ucx/reduce.cpp:56-80; kOrderShm: the 2N-chunk fold of src/shm/reduce.cpp:21-100; kOrderRank0.
+Status plan_reduce(Plan& plan, const void* const* send, void* recv_root, uint32_t nranks, uint64_t len,
+                   uint32_t elem_size, FoldOrder order, uint32_t root);
 // o = reduce(i0, i1) with the tie convention of src/ucx/kernel.cu:24-38 (equal / unordered -> i1)
 Status plan_reduce2(Plan& plan, const void* i0, const void* i1, void* o, uint64_t len, uint32_t elem_size);
 

@@ -78,6 +78,19 @@ struct FlatLaunch {
     uint32_t total_tiles;    // ceil(count * elem_size / 1024)
     uint32_t new_wins_ties;
     uint32_t elem_size;
+    uint32_t tree;  // 1: combine in binomial-tree order towards rank run.start instead of a left fold
+};
+
+// One launch of the element-wise tree kernel: out[e] = binomial-tree combination of in[*][e]
+// towards `root`, any rank count, any alignment.
+struct TreeLaunch {
+    const void* in[kMaxRanks];
+    void* out;
+    uint64_t count;
+    uint32_t nranks;
+    uint32_t root;
+    uint32_t elem_size;
+    uint32_t total_tiles;  // kThreads elements per tile
 };
 
 enum PackMode : uint32_t {

@@ -1,0 +1,274 @@
+"""The MegRay::Communicator API on the GPU, driven the way the reference drives it
+(test/test_base.h:26-62): create_server on a free port, N communicators in one process, one thread
+per rank doing init -> alloc -> copy in -> collective -> sync -> copy out, then compare.  Inputs and
+expectations are the closed forms of test/test_opr.cpp (cited per test), plus seeded random data
+against the oracle."""
+import threading
+
+import numpy as np
+import pytest
+
+import oracle as orc
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+import megray_amd as mr  # noqa: E402
+from gpu_util import bits_equal, empty_device, rand_array, to_device, to_host  # noqa: E402
+
+
+def run_test(nranks, inputs, expected, main_func, own_streams=True, configure=None):
+    """Mirror of run_test<T> (test/test_base.h:26-62)."""
+    port = mr.get_free_port()
+    mr.create_server(nranks, port)
+    comms = [mr.get_communicator(nranks, r, mr.Backend.VRANK) for r in range(nranks)]
+    outputs = [None] * nranks
+    errors = []
+
+    def rank_main(rank):
+        try:
+            torch.cuda.set_device(0)  # every virtual rank lives on the one GPU
+            comm = comms[rank]
+            comm.init("localhost", port)
+            if configure:
+                comm.configure(*configure)
+            stream = torch.cuda.Stream() if own_streams else torch.cuda.current_stream()
+            outputs[rank] = main_func(comm, rank, inputs[rank], stream)
+        except BaseException as exc:  # noqa: BLE001
+            errors.append((rank, repr(exc)))
+
+    threads = [threading.Thread(target=rank_main, args=(r,)) for r in range(nranks)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(120)
+        assert not t.is_alive(), "a rank hung"
+    assert not errors, errors
+    for r in range(nranks):
+        if expected[r] is not None:
+            assert bits_equal(outputs[r], expected[r]), f"rank {r}: {outputs[r]} != {expected[r]}"
+    for c in comms:
+        c.close()
+
+
+def f32(values):
+    return np.array(values, dtype=np.float32)
+
+
+def test_send_recv():
+    # test/test_opr.cpp:63-99: rank 0 sends "test_message" as CHAR to rank 1
+    msg = np.frombuffer(b"test_message", dtype=np.uint8).copy()
+
+    def main(comm, rank, inp, stream):
+        with torch.cuda.stream(stream):
+            if rank == 0:
+                buf = to_device(inp)
+                comm.send(buf, msg.size, mr.DType.CHAR, 1, stream)
+                stream.synchronize()
+                return None
+            buf = empty_device(msg.size)
+            comm.recv(buf, msg.size, mr.DType.CHAR, 0, stream)
+            stream.synchronize()
+            return to_host(buf, np.uint8)
+
+    run_test(2, [msg, None], [None, msg], main)
+
+
+def test_grouped_exchange_does_not_deadlock():
+    # both ranks send first, then receive: only works inside group_start / group_end
+    n = 1000
+    data = [np.arange(n, dtype=np.int32) * (r + 1) for r in range(2)]
+
+    def main(comm, rank, inp, stream):
+        with torch.cuda.stream(stream):
+            src, dst = to_device(inp), empty_device(n * 4)
+            comm.group_start()
+            comm.send(src, n, mr.DType.INT32, 1 - rank, stream)
+            comm.recv(dst, n, mr.DType.INT32, 1 - rank, stream)
+            comm.group_end()
+            stream.synchronize()
+            return to_host(dst, np.int32)
+
+    run_test(2, data, [data[1], data[0]], main)
+
+
+def test_scatter_gather():
+    nranks, length, root = 3, 10, 1
+    # test/test_opr.cpp:101-146
+    root_in = f32([(i + 1) * (j + 2) for i in range(nranks) for j in range(length)])
+    parts = [f32([(i + 1) * (j + 2) for j in range(length)]) for i in range(nranks)]
+
+    def scatter_main(comm, rank, inp, stream):
+        with torch.cuda.stream(stream):
+            out = empty_device(length * 4)
+            src = to_device(inp) if rank == root else None  # non-root passes nullptr (:133-135)
+            comm.scatter(src, out, length, mr.DType.FLOAT32, root, stream)
+            stream.synchronize()
+            return to_host(out, np.float32)
+
+    run_test(nranks, [root_in if r == root else None for r in range(nranks)], parts, scatter_main)
+
+    # test/test_opr.cpp:148-196
+    def gather_main(comm, rank, inp, stream):
+        with torch.cuda.stream(stream):
+            src = to_device(inp)
+            out = empty_device(nranks * length * 4) if rank == root else None
+            comm.gather(src, out, length, mr.DType.FLOAT32, root, stream)
+            stream.synchronize()
+            return to_host(out, np.float32) if rank == root else None
+
+    run_test(nranks, parts, [root_in if r == root else None for r in range(nranks)], gather_main)
+
+
+def test_all_to_all_and_all_gather():
+    nranks, length = 3, 6
+    # test/test_opr.cpp:198-241
+    ins = [f32([(i + 1) * (j + 2) * (k + 3) for j in range(nranks) for k in range(length)]) for i in range(nranks)]
+    outs = [f32([(i + 1) * (j + 2) * (k + 3) for i in range(nranks) for k in range(length)]) for j in range(nranks)]
+
+    def a2a_main(comm, rank, inp, stream):
+        with torch.cuda.stream(stream):
+            src, dst = to_device(inp), empty_device(nranks * length * 4)
+            comm.all_to_all(src, dst, length, mr.DType.FLOAT32, stream)
+            stream.synchronize()
+            return to_host(dst, np.float32)
+
+    run_test(nranks, ins, outs, a2a_main)
+
+    # test/test_opr.cpp:243-284
+    sendlen = 10
+    ins = [f32([(i + 1) * (j + 1) for j in range(sendlen)]) for i in range(nranks)]
+    want = np.concatenate(ins)
+
+    def ag_main(comm, rank, inp, stream):
+        with torch.cuda.stream(stream):
+            src, dst = to_device(inp), empty_device(nranks * sendlen * 4)
+            comm.all_gather(src, dst, sendlen, mr.DType.FLOAT32, stream)
+            stream.synchronize()
+            return to_host(dst, np.float32)
+
+    run_test(nranks, ins, [want] * nranks, ag_main)
+
+
+@pytest.mark.parametrize("own_streams", [True, False])
+def test_all_reduce_closed_forms(own_streams):
+    # test/test_opr.cpp:286-359
+    nranks, length = 3, 10
+    ins = [f32([(i + 1) * (j + 1) for j in range(length)]) for i in range(nranks)]
+    j1 = np.arange(1, length + 1, dtype=np.float32)
+    for op, want in ((mr.ReduceOp.SUM, 6 * j1), (mr.ReduceOp.MAX, 3 * j1), (mr.ReduceOp.MIN, j1)):
+        def main(comm, rank, inp, stream, op=op):
+            with torch.cuda.stream(stream):
+                src, dst = to_device(inp), empty_device(length * 4)
+                comm.all_reduce(src, dst, length, mr.DType.FLOAT32, op, stream)
+                stream.synchronize()
+                return to_host(dst, np.float32)
+
+        run_test(nranks, ins, [want] * nranks, main, own_streams=own_streams)
+
+
+def test_reduce_scatter_closed_forms():
+    # test/test_opr.cpp:361-438
+    nranks, recvlen = 3, 10
+    ins = [f32([(i + 1) * (m + 1) for m in range(nranks * recvlen)]) for i in range(nranks)]
+    for op, factor in ((mr.ReduceOp.SUM, 6), (mr.ReduceOp.MAX, 3), (mr.ReduceOp.MIN, 1)):
+        want = [f32([factor * (k * recvlen + j + 1) for j in range(recvlen)]) for k in range(nranks)]
+
+        def main(comm, rank, inp, stream, op=op):
+            with torch.cuda.stream(stream):
+                src, dst = to_device(inp), empty_device(recvlen * 4)
+                comm.reduce_scatter(src, dst, recvlen, mr.DType.FLOAT32, op, stream)
+                stream.synchronize()
+                return to_host(dst, np.float32)
+
+        run_test(nranks, ins, want, main)
+
+
+def test_broadcast_and_reduce_closed_forms():
+    nranks, root, length = 3, 1, 10
+    ins = [f32([(i + 1) * (j + 1) for j in range(length)]) for i in range(nranks)]
+
+    # test/test_opr.cpp:440-485
+    def bcast_main(comm, rank, inp, stream):
+        with torch.cuda.stream(stream):
+            src, dst = to_device(inp), empty_device(length * 4)
+            comm.broadcast(src, dst, length, mr.DType.FLOAT32, root, stream)
+            stream.synchronize()
+            return to_host(dst, np.float32)
+
+    run_test(nranks, ins, [ins[root]] * nranks, bcast_main)
+
+    # test/test_opr.cpp:487-551: only the root allocates a receive buffer
+    j1 = np.arange(1, length + 1, dtype=np.float32)
+    for op, want in ((mr.ReduceOp.SUM, 6 * j1), (mr.ReduceOp.MAX, 3 * j1), (mr.ReduceOp.MIN, j1)):
+        def reduce_main(comm, rank, inp, stream, op=op):
+            with torch.cuda.stream(stream):
+                src = to_device(inp)
+                dst = empty_device(length * 4) if rank == root else None
+                comm.reduce(src, 0xDEAD0000 if dst is None else dst, length, mr.DType.FLOAT32, op, root, stream)
+                stream.synchronize()
+                return to_host(dst, np.float32) if rank == root else None
+
+        run_test(nranks, ins, [want if r == root else None for r in range(nranks)], reduce_main)
+
+
+@pytest.mark.parametrize("nranks", [2, 4, 8])
+def test_random_data_orders_and_work_queued_on_rank_streams(nranks):
+    """Seeded random fp32 through the thread-per-rank API equals the oracle's literal ucx ring replay;
+    with SHM order it equals the shm replay.  Each rank fills its input ON ITS OWN STREAM right before
+    the collective and reads the result on it right after, so a missing cross-stream dependency
+    would show as stale data."""
+    rng = np.random.default_rng(nranks)
+    length = 1 << 18
+    ins = [rand_array(orc.FLOAT32, length, rng) for _ in range(nranks)]
+    for order, want in ((mr.FoldOrder.UCX, orc.ucx_all_reduce(ins, orc.FLOAT32, orc.SUM)),
+                        (mr.FoldOrder.SHM, orc.shm_all_reduce(ins, orc.FLOAT32, orc.SUM))):
+        def main(comm, rank, inp, stream):
+            with torch.cuda.stream(stream):
+                staged = torch.from_numpy(inp.view(np.uint8).copy()).pin_memory()
+                src = torch.empty(length * 4, dtype=torch.uint8, device="cuda:0")
+                dst = torch.full((length * 4,), 0x5A, dtype=torch.uint8, device="cuda:0")
+                host_out = torch.empty(length * 4, dtype=torch.uint8).pin_memory()
+                for _ in range(3):  # several rounds back to back, no host sync in between
+                    src.copy_(staged, non_blocking=True)
+                    comm.all_reduce(src, dst, length, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream)
+                    host_out.copy_(dst, non_blocking=True)
+                stream.synchronize()
+                return host_out.numpy().view(np.float32).copy()
+
+        run_test(nranks, ins, want, main, configure=(order, mr.Schedule.FUSED))
+
+    want = orc.ucx_reduce(ins, orc.FLOAT32, orc.SUM, nranks - 1)
+
+    def reduce_main(comm, rank, inp, stream):
+        with torch.cuda.stream(stream):
+            src, dst = to_device(inp), empty_device(length * 4)
+            comm.reduce(src, dst, length, mr.DType.FLOAT32, mr.ReduceOp.SUM, nranks - 1, stream)
+            stream.synchronize()
+            return to_host(dst, np.float32)
+
+    run_test(nranks, ins, [want[r] if r == nranks - 1 else None for r in range(nranks)], reduce_main)
+
+
+def test_contract_violations_throw_on_the_calling_rank():
+    nranks = 2
+    port = mr.get_free_port()
+    mr.create_server(nranks, port)
+    comms = [mr.get_communicator(nranks, r) for r in range(nranks)]
+    threads = [threading.Thread(target=comms[r].init, args=("localhost", port)) for r in range(nranks)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(60)
+    buf = empty_device(64)
+    with pytest.raises(mr.MegRayError, match="unknown dtype"):      # src/ucx/kernel.cu:95-96
+        comms[0].all_reduce(buf, buf, 16, mr.DType.CHAR, mr.ReduceOp.SUM)
+    with pytest.raises(mr.MegRayError, match="unknown reduce op"):  # src/ucx/kernel.cu:55-56
+        comms[0].all_reduce(buf, buf, 16, mr.DType.FLOAT32, 7)
+    with pytest.raises(mr.MegRayError, match="unknown dtype"):      # src/core/common.cpp:35-36
+        comms[0].all_gather(buf, buf, 1, 42)
+    with pytest.raises(mr.MegRayError):
+        comms[0].broadcast(buf, buf, 1, mr.DType.FLOAT32, 5)
+    fresh = mr.get_communicator(2, 0)
+    with pytest.raises(mr.MegRayError):
+        fresh.all_reduce(buf, buf, 16, mr.DType.FLOAT32, mr.ReduceOp.SUM)  # before init()

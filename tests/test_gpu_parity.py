@@ -282,3 +282,44 @@ def test_errors_follow_the_reference():
     with pytest.raises(mr.MegRayError, match="nranks"):
         mr.all_reduce([d] * 17, [o] * 17, 1, mr.DType.FLOAT32, mr.ReduceOp.SUM)
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("dtype", REDUCE_TYPES)
+def test_reduce_to_root(dtype):
+    """ucx order = the binomial tree of src/ucx/reduce.cpp:56-80, against the oracle's literal replay
+    (FLOAT16: the same tree in fp32 with one rounding)."""
+    rng = np.random.default_rng(300 + dtype)
+    size = orc.dtype_size(dtype)
+    for nranks in (1, 2, 3, 4, 5, 8, 11):
+        for length in (0, 1, 777, 4096 * 4 + 5):
+            ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+            for root in sorted({0, nranks - 1}):
+                for op in OPS:
+                    for misalign in (0, size):
+                        d_in = [to_device(x, misalign) for x in ins]
+                        d_out = empty_device(length * size, misalign)
+                        mr.reduce_to_root(d_in, d_out, length, dtype, op, root)
+                        torch.cuda.synchronize()
+                        got = to_host(d_out, ins[0].dtype)
+                        if dtype == orc.FLOAT16:
+                            a = [ins[(root + v) % nranks].astype(np.float32) for v in range(nranks)]
+                            bit = 1
+                            while bit < nranks:
+                                for v in range(0, nranks - bit, 2 * bit):
+                                    x, y = a[v], a[v + bit]
+                                    with np.errstate(over="ignore"):
+                                        a[v] = {orc.SUM: x + y, orc.MAX: np.where(y > x, y, x),
+                                                orc.MIN: np.where(y < x, y, x)}[op]
+                                bit *= 2
+                            with np.errstate(over="ignore"):
+                                want = a[0].astype(np.float16)
+                        else:
+                            want = orc.ucx_reduce(ins, dtype, op, root)[root]
+                        assert_same(got, want, f"reduce dtype={dtype} N={nranks} len={length} root={root} op={op}")
+                    for order in (orc.ORDER_SHM, orc.ORDER_RANK0):
+                        d_in = [to_device(x) for x in ins]
+                        d_out = empty_device(length * size)
+                        mr.reduce_to_root(d_in, d_out, length, dtype, op, root, order)
+                        torch.cuda.synchronize()
+                        assert_same(to_host(d_out, ins[0].dtype), orc.fold_all_reduce(ins, dtype, op, order)[0],
+                                    f"reduce order={order}")

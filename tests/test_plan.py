@@ -45,11 +45,23 @@ def execute(runs, sends, recvs, nranks, op, elem_size, send_ptrs, recv_ptrs):
         for run in (r for r in runs if r["step"] == step):
             if run["kind"] == 0:
                 src = snapshot if run["reads_recv"] else sends
-                ranks = [(run["start"] + run["dir"] * j) % nranks for j in range(run["nfold"])]
                 lo, cnt = run["in_begin"], run["count"]
-                acc = src[ranks[0]][lo:lo + cnt].copy()
-                for r in ranks[1:]:
-                    acc = combine(acc, src[r][lo:lo + cnt], op, run["new_wins_ties"])
+                if run["dir"] == 0:
+                    # binomial tree towards rank `start` (src/ucx/reduce.cpp:56-80): virtual rank v takes in
+                    # v + bit as reduce(incoming, own), own surviving a tie
+                    ranks = [(run["start"] + v) % nranks for v in range(nranks)]
+                    a = [src[r][lo:lo + cnt].copy() for r in ranks]
+                    bit = 1
+                    while bit < nranks:
+                        for v in range(0, nranks - bit, 2 * bit):
+                            a[v] = combine(a[v], a[v + bit], op, False)
+                        bit *= 2
+                    acc = a[0]
+                else:
+                    ranks = [(run["start"] + run["dir"] * j) % nranks for j in range(run["nfold"])]
+                    acc = src[ranks[0]][lo:lo + cnt].copy()
+                    for r in ranks[1:]:
+                        acc = combine(acc, src[r][lo:lo + cnt], op, run["new_wins_ties"])
                 for m in range(run["nout"]):
                     dst = (run["out_first"] + m) % nranks
                     recvs[dst][run["out_begin"]:run["out_begin"] + cnt] = acc
@@ -175,6 +187,33 @@ def test_pack_plans(nranks):
                 assert bits_equal(got[root], orc.ucx_gather(parts, dtype, root)[root])
                 got = run(mr.Collective.BROADCAST, parts, length, length, root)
                 assert all(bits_equal(got[r], parts[root]) for r in range(nranks))
+
+
+@pytest.mark.parametrize("dtype", [orc.INT8, orc.INT32, orc.FLOAT32, orc.FLOAT64, orc.UINT64])
+@pytest.mark.parametrize("nranks", [1, 2, 3, 4, 5, 8, 13, 16])
+def test_reduce_plans(dtype, nranks):
+    """reduce to a root: the ucx order is the binomial tree of src/ucx/reduce.cpp, checked against the
+    oracle's literal replay of it."""
+    rng = np.random.default_rng(dtype * 31 + nranks)
+    size = orc.dtype_size(dtype)
+    for length in (0, 1, 5, 300, 1031):
+        ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+        for misalign in (False, True):
+            offs = [size * (r % 3) for r in range(nranks)] if misalign else [0] * nranks
+            sp, rp = fake_ptrs(SEND_BASE, nranks, offs), fake_ptrs(RECV_BASE, nranks, offs)
+            for root in sorted({0, nranks // 2, nranks - 1}):
+                for op in (orc.SUM, orc.MAX, orc.MIN):
+                    runs, br, bw = mr.describe(mr.Collective.REDUCE, sp, rp, length, dtype, orc.ORDER_UCX, root=root)
+                    recvs = [np.zeros(length, dtype=ins[0].dtype) for _ in range(nranks)]
+                    got = execute(runs, ins, recvs, nranks, op, size, sp, rp)
+                    want = orc.ucx_reduce(ins, dtype, op, root)
+                    assert bits_equal(got[root], want[root]), (dtype, nranks, length, root, op)
+                    assert (br, bw) == ((nranks * length * size, length * size) if length else (0, 0))
+                    for order in (orc.ORDER_SHM, orc.ORDER_RANK0):
+                        runs, _, _ = mr.describe(mr.Collective.REDUCE, sp, rp, length, dtype, order, root=root)
+                        recvs = [np.zeros(length, dtype=ins[0].dtype) for _ in range(nranks)]
+                        got = execute(runs, ins, recvs, nranks, op, size, sp, rp)
+                        assert bits_equal(got[root], orc.fold_all_reduce(ins, dtype, op, order)[root])
 
 
 def test_two_input_reduce_plan_keeps_i1_on_ties():
