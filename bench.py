@@ -28,8 +28,8 @@ BASE_SEED = 0x4D656752  # "MegR"; rank r draws from seed BASE_SEED + r
 # HBM bytes per launch of the fold kernel on the headline workload, from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE runs scaled by the same counters on a plain copy of known size; the
 # summaries those figures come from are kept as text next to the kernel-trace summaries.
-# None until measured.
-MEASURED_TRAFFIC_BYTES = {"all_reduce_f32_n8_2p28_fused": None}
+# FETCH_SIZE counts 2 KiB per unit on this part (scale 1.99992), WRITE_SIZE 1 KiB (scale 0.99997).
+MEASURED_TRAFFIC_BYTES = {"all_reduce_f32_n8_2p28_fused": 17180153376}
 
 
 def parse_args():
@@ -40,6 +40,11 @@ def parse_args():
     ap.add_argument("--log2n", type=int, default=28, help="elements per rank = 2^log2n")
     ap.add_argument("--ranks", type=int, default=8)
     ap.add_argument("--schedule", default="fused", choices=["fused", "two_phase", "ring"])
+    ap.add_argument("--workload", default="all_reduce",
+                    choices=["all_reduce", "copy", "c2_reduce_scatter", "c2_all_gather", "c3_max_int32",
+                             "c3_min_int64", "c5_all_to_all", "c5_sum_int8"],
+                    help="all_reduce = the headline; copy = 1 GiB plain copy (counter calibration); "
+                         "c2/c3/c5 = the other BASELINE configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-small", action="store_true", help="skip the small-message sweep")
     ap.add_argument("--no-check", action="store_true", help="skip the correctness checks")
@@ -148,6 +153,95 @@ def cpu_baseline(orc, np, nranks):
     }
 
 
+def run_other_workload(args, torch, mr):
+    """The non-headline workloads: same timing, one JSON line, no CPU / small-message legs."""
+    dev = "cuda:0"
+    st = torch.cuda.current_stream()
+    n8 = 8
+    w = args.workload
+
+    def rnd(n, dtype, seed):
+        g = torch.Generator(device=dev)
+        g.manual_seed(BASE_SEED + seed)
+        if dtype.is_floating_point:
+            return (torch.randn(n, generator=g, device=dev, dtype=torch.float32) * 0.01).to(dtype)
+        info = torch.iinfo(dtype)
+        return torch.randint(info.min, info.max, (n,), generator=g, device=dev, dtype=dtype)
+
+    if w == "copy":
+        n = 1 << 30
+        src, dst = [rnd(n, torch.uint8, 0)], [torch.empty(n, dtype=torch.uint8, device=dev)]
+        step = lambda: mr.broadcast(src[0], dst, n, mr.DType.UINT8, 0, stream=st)  # noqa: E731
+        desc = (mr.Collective.BROADCAST, src, dst, n, mr.DType.UINT8)
+        text, dt = "plain copy of 2^30 bytes (one rank, broadcast to itself)", "u8"
+    elif w == "c2_reduce_scatter":
+        recvlen = 1 << 23
+        src = [rnd(n8 * recvlen, torch.float16, r) for r in range(n8)]
+        dst = [torch.empty(recvlen, dtype=torch.float16, device=dev) for _ in range(n8)]
+        step = lambda: mr.reduce_scatter(src, dst, recvlen, mr.DType.FLOAT16, mr.ReduceOp.SUM, stream=st)  # noqa: E731
+        desc = (mr.Collective.REDUCE_SCATTER, src, dst, recvlen, mr.DType.FLOAT16)
+        text, dt = "reduce_scatter SUM fp16 (fp32 accumulate), 8 ranks x 2^26 elements in, 2^23 out", "f16"
+    elif w == "c2_all_gather":
+        sendlen = 1 << 23
+        src = [rnd(sendlen, torch.float16, r) for r in range(n8)]
+        dst = [torch.empty(n8 * sendlen, dtype=torch.float16, device=dev) for _ in range(n8)]
+        step = lambda: mr.all_gather(src, dst, sendlen, mr.DType.FLOAT16, stream=st)  # noqa: E731
+        desc = (mr.Collective.ALL_GATHER, src, dst, sendlen, mr.DType.FLOAT16)
+        text, dt = "all_gather fp16, 8 ranks x 2^23 elements in, 2^26 out", "f16"
+    elif w in ("c3_max_int32", "c3_min_int64"):
+        tdt, mdt, op = ((torch.int32, mr.DType.INT32, mr.ReduceOp.MAX) if w == "c3_max_int32"
+                        else (torch.int64, mr.DType.INT64, mr.ReduceOp.MIN))
+        n = 1 << 28
+        src = [rnd(n, tdt, r) for r in range(n8)]
+        dst = [torch.empty(n, dtype=tdt, device=dev) for _ in range(n8)]
+        step = lambda: mr.all_reduce(src, dst, n, mdt, op, stream=st)  # noqa: E731
+        desc = (mr.Collective.ALL_REDUCE, src, dst, n, mdt)
+        text, dt = f"all_reduce {op.name} {mdt.name.lower()}, 8 ranks x 2^28 elements", mdt.name.lower()
+    elif w == "c5_all_to_all":
+        blk = 1 << 24
+        src = [rnd(n8 * blk, torch.uint8, r) for r in range(n8)]
+        dst = [torch.empty(n8 * blk, dtype=torch.uint8, device=dev) for _ in range(n8)]
+        step = lambda: mr.all_to_all(src, dst, blk, mr.DType.UINT8, stream=st)  # noqa: E731
+        desc = (mr.Collective.ALL_TO_ALL, src, dst, blk, mr.DType.UINT8)
+        text, dt = "all_to_all uint8, 8 ranks x 8 blocks of 16 MiB", "u8"
+    else:
+        n = 1 << 27
+        src = [rnd(n, torch.int8, r) for r in range(n8)]
+        dst = [torch.empty(n, dtype=torch.int8, device=dev) for _ in range(n8)]
+        step = lambda: mr.all_reduce(src, dst, n, mr.DType.INT8, mr.ReduceOp.SUM, stream=st)  # noqa: E731
+        desc = (mr.Collective.ALL_REDUCE, src, dst, n, mr.DType.INT8)
+        text, dt = "all_reduce SUM int8 (wrap-around), 8 ranks x 2^27 elements", "i8"
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(st)
+    for _ in range(args.steps):
+        step()
+    e1.record(st)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    runs, bytes_read, bytes_written = mr.describe(desc[0], desc[1], desc[2], desc[3], desc[4])
+    launches = max(1, len({r["step"] for r in runs}))
+    executed = bytes_read + bytes_written
+    kernel_ms = e0.elapsed_time(e1) / args.steps / launches
+    achieved = executed / launches / (kernel_ms * 1e-3) / 1e9
+    value = executed / (wall / args.steps) / 1e9
+    print(json.dumps({
+        "metric": "achieved HBM GB/s (% of peak)", "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt, "data": "synthetic",
+        "config": {"workload": text, "launches_per_step": launches},
+        "pct_of_peak": round(100.0 * value / HBM_PEAK_GBPS, 2), "bytes_executed": executed,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel_ms": round(kernel_ms, 4), "algorithmic_bytes_per_launch": executed // launches},
+    }))
+    return 0
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -165,6 +259,8 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
     torch.cuda.set_device(0)
+    if args.workload != "all_reduce":
+        return run_other_workload(args, torch, mr)
     nranks, n = args.ranks, 1 << args.log2n
     sched = {"fused": mr.Schedule.FUSED, "two_phase": mr.Schedule.TWO_PHASE, "ring": mr.Schedule.RING}[args.schedule]
 
