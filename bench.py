@@ -44,7 +44,7 @@ def parse_args():
                     choices=["all_reduce", "copy", "c2_reduce_scatter", "c2_all_gather", "c3_max_int32",
                              "c3_min_int64", "c5_all_to_all", "c5_sum_int8"],
                     help="all_reduce = the headline; copy = 1 GiB plain copy (counter calibration); "
-                         "c2/c3/c5 = the other BASELINE configurations")
+                         "c2/c3/c5 = the other benchmark configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-small", action="store_true", help="skip the small-message sweep")
     ap.add_argument("--no-check", action="store_true", help="skip the correctness checks")
