@@ -1,0 +1,182 @@
+"""The benchmark configurations at their full sizes, checked through properties that do not need a
+CPU pass over gigabytes: an independent on-device recomputation with torch's element-wise ops (exact
+for integers and for fp32 in a fixed order), cross-schedule equality, permutation identities, and
+windows cut out of every chunk and compared with the CPU oracle."""
+import numpy as np
+import pytest
+
+import oracle as orc
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+import megray_amd as mr  # noqa: E402
+
+DEV = "cuda:0"
+SEED = 0x4D656752
+
+
+def gen(n, dtype, rank, kind="full"):
+    g = torch.Generator(device=DEV)
+    g.manual_seed(SEED + rank)
+    if dtype.is_floating_point:
+        if kind == "normal":  # normal(0, 0.01)
+            return (torch.randn(n, generator=g, device=DEV, dtype=torch.float32) * 0.01).to(dtype)
+        return (torch.rand(n, generator=g, device=DEV, dtype=torch.float32) * 2 - 1).to(dtype)
+    info = torch.iinfo(dtype)
+    if dtype == torch.int64:  # randint cannot span the whole int64 range in one call
+        hi = torch.randint(-2 ** 31, 2 ** 31, (n,), generator=g, device=DEV, dtype=torch.int64)
+        lo = torch.randint(0, 2 ** 32, (n,), generator=g, device=DEV, dtype=torch.int64)
+        return (hi << 32) | lo
+    return torch.randint(info.min, info.max + 1, (n,), generator=g, device=DEV, dtype=dtype)
+
+
+def bits(t):
+    return t.view(torch.uint8) if t.element_size() == 1 else t.view({2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()])
+
+
+def window_problem(ins, nranks, chunk_len, offset, width):
+    """Host copies of [chunk*chunk_len + offset, +width) of every input for every chunk, laid out as a
+    small collective of length nranks*width whose chunk c is the window of chunk c."""
+    mini = []
+    for t in ins:
+        parts = [t[c * chunk_len + offset: c * chunk_len + offset + width] for c in range(nranks)]
+        mini.append(torch.cat(parts).cpu().numpy())
+    return mini
+
+
+def test_headline_all_reduce_fp32_8x2p28():
+    n, nranks = 1 << 28, 8
+    ins = [gen(n, torch.float32, r) for r in range(nranks)]
+    outs = [torch.empty_like(t) for t in ins]
+    mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM)
+    torch.cuda.synchronize()
+    for r in range(1, nranks):
+        assert torch.equal(bits(outs[0]), bits(outs[r])), f"rank {r} differs"
+    # independent recomputation on the device: chunk c is ((x_c + x_{c+1}) + ...) + x_{c-1}
+    chunk = n // nranks
+    for c in range(nranks):
+        sl = slice(c * chunk, (c + 1) * chunk)
+        acc = ins[c][sl].clone()
+        for j in range(1, nranks):
+            acc += ins[(c + j) % nranks][sl]
+        assert torch.equal(bits(acc), bits(outs[0][sl])), f"chunk {c} is not the ucx ring order"
+    # windows against the CPU oracle's literal ring replay
+    width = 1 << 14
+    for offset in (0, chunk // 2 + 3, chunk - width):
+        mini = window_problem(ins, nranks, chunk, offset, width)
+        want = orc.ucx_all_reduce(mini, orc.FLOAT32, orc.SUM)[0]
+        got = torch.cat([outs[3][c * chunk + offset: c * chunk + offset + width] for c in range(nranks)]).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # the other schedules give the same bits
+    ref = outs[0].clone()
+    for sched in (mr.Schedule.TWO_PHASE, mr.Schedule.RING):
+        for o in outs:
+            o.zero_()
+        mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, schedule=sched)
+        torch.cuda.synchronize()
+        for r in (0, nranks - 1):
+            assert torch.equal(bits(ref), bits(outs[r])), f"schedule {sched} differs on rank {r}"
+
+
+@pytest.mark.parametrize("tdtype,mdtype", [(torch.int32, mr.DType.INT32), (torch.int64, mr.DType.INT64)])
+def test_c3_max_min_integers_8x2p28(tdtype, mdtype):
+    n, nranks = 1 << 28, 8
+    ins = [gen(n, tdtype, r) for r in range(nranks)]
+    outs = [torch.empty_like(t) for t in ins]
+    for op, fn in ((mr.ReduceOp.MAX, torch.maximum), (mr.ReduceOp.MIN, torch.minimum)):
+        mr.all_reduce(ins, outs, n, mdtype, op)
+        torch.cuda.synchronize()
+        want = ins[0].clone()
+        for r in range(1, nranks):
+            fn(want, ins[r], out=want)
+        for r in range(nranks):
+            assert torch.equal(want, outs[r]), f"{op.name} rank {r}"
+        del want
+    # the value range really is the full dtype range
+    info = torch.iinfo(tdtype)
+    assert int(ins[0].max()) > info.max // 2 and int(ins[0].min()) < info.min // 2
+
+
+def test_c2_reduce_scatter_then_all_gather_fp16():
+    nranks, recvlen = 8, 1 << 23
+    total = nranks * recvlen
+    ins = [gen(total, torch.float16, r, "normal") for r in range(nranks)]
+    parts = [torch.empty(recvlen, dtype=torch.float16, device=DEV) for _ in range(nranks)]
+    mr.reduce_scatter(ins, parts, recvlen, mr.DType.FLOAT16, mr.ReduceOp.SUM)
+    gathered = [torch.empty(total, dtype=torch.float16, device=DEV) for _ in range(nranks)]
+    mr.all_gather(parts, gathered, recvlen, mr.DType.FLOAT16)
+    torch.cuda.synchronize()
+    for r in range(1, nranks):
+        assert torch.equal(bits(gathered[0]), bits(gathered[r]))
+    for r in range(nranks):
+        assert torch.equal(bits(gathered[0][r * recvlen:(r + 1) * recvlen]), bits(parts[r]))
+    # on-device recomputation: fp32 accumulate in the ring order of chunk c (c+1, ..., c), one rounding
+    for c in range(nranks):
+        sl = slice(c * recvlen, (c + 1) * recvlen)
+        acc = ins[(c + 1) % nranks][sl].float()
+        for j in range(2, nranks + 1):
+            acc += ins[(c + j) % nranks][sl].float()
+        assert torch.equal(bits(acc.half()), bits(parts[c])), f"chunk {c}"
+    # windows against the oracle (tolerance stated by the task: 1 ulp; asserted: 0)
+    width = 1 << 13
+    for offset in (0, recvlen // 3, recvlen - width):
+        mini = window_problem(ins, nranks, recvlen, offset, width)
+        want = orc.fold_reduce_scatter(mini, orc.FLOAT16, orc.SUM, orc.ORDER_UCX)
+        for r in range(nranks):
+            got = parts[r][offset:offset + width].cpu().numpy()
+            assert np.array_equal(got.view(np.uint16), want[r].view(np.uint16))
+    # reduce_scatter + all_gather == all_reduce when both use one order (RANK0)
+    mr.reduce_scatter(ins, parts, recvlen, mr.DType.FLOAT16, mr.ReduceOp.SUM, mr.FoldOrder.RANK0)
+    mr.all_gather(parts, gathered, recvlen, mr.DType.FLOAT16)
+    ar = [torch.empty(total, dtype=torch.float16, device=DEV) for _ in range(nranks)]
+    mr.all_reduce(ins, ar, total, mr.DType.FLOAT16, mr.ReduceOp.SUM, mr.FoldOrder.RANK0)
+    torch.cuda.synchronize()
+    assert torch.equal(bits(ar[0]), bits(gathered[5]))
+
+
+def test_c5_all_to_all_uint8_and_int8_wraparound():
+    nranks, blk = 8, 1 << 24
+    ins = [gen(nranks * blk, torch.uint8, r) for r in range(nranks)]
+    outs = [torch.empty_like(t) for t in ins]
+    mr.all_to_all(ins, outs, blk, mr.DType.UINT8)
+    torch.cuda.synchronize()
+    for i in range(nranks):
+        for j in range(nranks):
+            assert torch.equal(outs[j][i * blk:(i + 1) * blk], ins[i][j * blk:(j + 1) * blk])
+    back = [torch.empty_like(t) for t in ins]
+    mr.all_to_all(outs, back, blk, mr.DType.UINT8)  # the transposition is an involution
+    torch.cuda.synchronize()
+    for r in range(nranks):
+        assert torch.equal(back[r], ins[r])
+    # int8 SUM on the same shape: must wrap mod 256
+    n = nranks * blk
+    sins = [t.view(torch.int8) for t in ins]
+    souts = [torch.empty_like(t) for t in sins]
+    mr.all_reduce(sins, souts, n, mr.DType.INT8, mr.ReduceOp.SUM)
+    torch.cuda.synchronize()
+    want = sins[0].clone()
+    for r in range(1, nranks):
+        want += sins[r]  # torch wraps int8
+    for r in range(nranks):
+        assert torch.equal(want, souts[r])
+    wide = torch.zeros(1 << 20, dtype=torch.int32, device=DEV)
+    for r in range(nranks):
+        wide += sins[r][:1 << 20].int()
+    assert bool(((wide > 127) | (wide < -128)).any()), "the data never overflows int8: the test would pin nothing"
+    assert torch.equal(((wide + 128) % 256 - 128).to(torch.int8), souts[0][:1 << 20])
+
+
+def test_small_message_sizes_are_exact():
+    # the latency sweep's shapes: 8 ranks, 4 KiB .. 1 MiB per rank
+    rng = np.random.default_rng(4)
+    for nbytes in (4096, 16384, 65536, 262144, 1048576):
+        n = nbytes // 4
+        host = [rng.uniform(-1, 1, n).astype(np.float32) for _ in range(8)]
+        ins = [torch.from_numpy(h).to(DEV) for h in host]
+        outs = [torch.empty_like(t) for t in ins]
+        mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM)
+        torch.cuda.synchronize()
+        want = orc.ucx_all_reduce(host, orc.FLOAT32, orc.SUM)
+        for r in range(8):
+            assert np.array_equal(outs[r].cpu().numpy().view(np.uint32), want[r].view(np.uint32))
