@@ -92,35 +92,73 @@ def check_full(torch, mr, ins, outs, n):
 
 
 def small_message_sweep(torch, mr):
-    """all_reduce SUM fp32, 8 ranks, 4 KiB .. 1 MiB per rank: microseconds per collective, issued
-    back to back on one stream (throughput latency) and one at a time with a host sync (round trip)."""
+    """all_reduce SUM fp32, 8 ranks, 4 KiB .. 1 MiB per rank: microseconds per collective.
+
+    stream_us        planned once (mrv_plan_create), launched back to back on one stream: the rate at
+                     which collectives retire (one kernel launch each)
+    unplanned_us     the same through mrv_all_reduce, which plans on every call
+    sync_median/p99  one planned collective at a time, launch to host-visible completion
+    """
     out = {}
     st = torch.cuda.current_stream()
     for nbytes in (4096, 16384, 65536, 262144, 1048576):
         n = nbytes // 4
         ins = make_inputs(torch, 8, n)
         outs = [torch.empty_like(t) for t in ins]
-        for _ in range(100):
-            mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream=st)
-        torch.cuda.synchronize()
-        iters = 1000
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(st)
-        for _ in range(iters):
-            mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream=st)
-        e1.record(st)
-        torch.cuda.synchronize()
-        stream_us = e0.elapsed_time(e1) * 1000.0 / iters
+        plan = mr.CollectivePlan(mr.Collective.ALL_REDUCE, ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM)
+        raw = st.cuda_stream
+
+        def timed(fn, iters):
+            for _ in range(100):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(st)
+            for _ in range(iters):
+                fn()
+            e1.record(st)
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1000.0 / iters
+
+        stream_us = timed(lambda: plan.launch(raw), 2000)
+        unplanned_us = timed(lambda: mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream=raw), 1000)
         lat = []
-        for _ in range(300):
+        for _ in range(500):
             t0 = time.perf_counter()
-            mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream=st)
+            plan.launch(raw)
             torch.cuda.synchronize()
             lat.append((time.perf_counter() - t0) * 1e6)
         lat.sort()
-        out[str(nbytes)] = {"stream_us": round(stream_us, 2), "sync_median_us": round(lat[len(lat) // 2], 2),
+        out[str(nbytes)] = {"stream_us": round(stream_us, 2), "unplanned_us": round(unplanned_us, 2),
+                            "sync_median_us": round(lat[len(lat) // 2], 2),
                             "sync_p99_us": round(lat[int(len(lat) * 0.99)], 2)}
+        plan.close()
     return out
+
+
+def copy_yardstick(torch, mr):
+    """What this particular GPU sustains on the simplest streaming job, for context: a 1 GiB device copy
+    through this library's copy kernel and through torch (GB/s, read + write)."""
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda:0").zero_()
+    dst = torch.empty_like(src)
+    st = torch.cuda.current_stream()
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(st)
+        for _ in range(20):
+            fn()
+        e1.record(st)
+        torch.cuda.synchronize()
+        return 2 * n / (e0.elapsed_time(e1) / 20 * 1e-3) / 1e9
+
+    lib = timed(lambda: mr.broadcast(src, [dst], n, mr.DType.UINT8, 0, stream=st))
+    tch = timed(lambda: dst.copy_(src))
+    return {"library_copy_gbps": round(lib, 1), "torch_copy_gbps": round(tch, 1)}
 
 
 def cpu_baseline(orc, np, nranks):
@@ -327,12 +365,13 @@ def main():
         "roofline": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(key),
-            "kernel": "fold_kernel<float, SUM, K=8>" if args.schedule == "fused" else "fold_kernel (several)",
+            "kernel": "fold_flat_kernel<float, SUM, K=8>" if args.schedule == "fused" else "fold kernels (several)",
             "kernel_ms": round(kernel_ms, 4), "algorithmic_bytes_per_launch": executed // launches,
         },
     }
     del ins, outs
     torch.cuda.empty_cache()
+    result["copy_yardstick"] = copy_yardstick(torch, mr)
     if not args.no_small:
         result["small_msg_us"] = small_message_sweep(torch, mr)
     if not args.no_cpu:

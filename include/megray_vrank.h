@@ -184,6 +184,28 @@ MRV_API int mrv_describe(int collective, const void* const* sendbuffs, void* con
                          mrv_plan_run* runs, size_t cap, size_t* nruns, uint64_t* bytes_read,
                          uint64_t* bytes_written);
 
+/* ---- planned collectives: plan once, launch many times ------------------------------------- */
+
+/*
+ * A training loop repeats the same collective on the same buffers.  mrv_plan_create does the
+ * host-side planning once (no reference counterpart: the reference re-derives chunk sizes and
+ * re-allocates its workspace on every call, src/ucx/all_reduce.cpp:33-51); mrv_plan_launch then
+ * only enqueues the prepared launches.  With MRV_PLAN_GRAPH the launches of a multi-launch plan
+ * (two-phase, ring) are additionally instantiated as one HIP graph of kernel nodes and replayed
+ * with a single hipGraphLaunch.
+ * `collective` is one of the MRV_* selectors, arguments as for mrv_describe; `op` is ignored by the
+ * copy collectives.  The buffers must stay valid and unchanged in address until mrv_plan_destroy.
+ */
+typedef struct mrv_plan mrv_plan;
+#define MRV_PLAN_GRAPH 1u
+MRV_API int mrv_plan_create(int collective, const void* const* sendbuffs, void* const* recvbuffs,
+                            uint32_t nranks, size_t count, int dtype, int op, int order, int schedule,
+                            uint32_t root, uint32_t flags, mrv_plan** plan);
+MRV_API int mrv_plan_launch(const mrv_plan* plan, void* stream);
+/* number of kernel launches one mrv_plan_launch stands for */
+MRV_API size_t mrv_plan_launch_count(const mrv_plan* plan);
+MRV_API void mrv_plan_destroy(mrv_plan* plan);
+
 /* ---- the MegRay::Communicator API, one handle per rank ------------------------------------- */
 
 /*

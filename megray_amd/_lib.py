@@ -56,6 +56,14 @@ def load():
     L.mrv_describe.argtypes = [i32, pp, pp, u32, sz, i32, i32, i32, u32, ctypes.POINTER(PlanRun), sz,
                                ctypes.POINTER(sz), ctypes.POINTER(ctypes.c_uint64),
                                ctypes.POINTER(ctypes.c_uint64)]
+    L.mrv_plan_create.argtypes = [i32, pp, pp, u32, sz, i32, i32, i32, i32, u32, u32, ctypes.POINTER(vp)]
+    L.mrv_plan_create.restype = i32
+    L.mrv_plan_launch.argtypes = [vp, vp]
+    L.mrv_plan_launch.restype = i32
+    L.mrv_plan_launch_count.argtypes = [vp]
+    L.mrv_plan_launch_count.restype = sz
+    L.mrv_plan_destroy.argtypes = [vp]
+    L.mrv_plan_destroy.restype = None
     L.mrv_reduce_to_root.argtypes = [pp, vp, u32, sz, i32, i32, i32, u32, vp]
     L.mrv_get_free_port.argtypes = []
     L.mrv_create_server.argtypes = [u32, i32]

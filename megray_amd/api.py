@@ -211,6 +211,38 @@ def describe(collective, sendptrs, recvptrs, count, dtype, order=FoldOrder.UCX, 
     return out, br.value, bw.value
 
 
+class CollectivePlan:
+    """A collective planned once and launched many times (mrv_plan_*).  `graph=True` instantiates
+    the launches of a multi-launch plan as one HIP graph.  The buffers must outlive the plan."""
+
+    def __init__(self, collective, sendbuffs, recvbuffs, count, dtype, op=ReduceOp.SUM, order=FoldOrder.UCX,
+                 schedule=Schedule.FUSED, root=0, graph=False, nranks=None):
+        self._h = ctypes.c_void_p()
+        self._keep = (sendbuffs, recvbuffs)
+        nranks = nranks if nranks is not None else max(len(sendbuffs), len(recvbuffs))
+        _check(_lib.load().mrv_plan_create(int(collective), _ptr_array(sendbuffs), _ptr_array(recvbuffs), nranks,
+                                           count, int(dtype), int(op), int(order), int(schedule), root,
+                                           1 if graph else 0, ctypes.byref(self._h)))
+        self._launch = _lib.load().mrv_plan_launch
+
+    @property
+    def launch_count(self):
+        return _lib.load().mrv_plan_launch_count(self._h)
+
+    def launch(self, stream=None):
+        status = self._launch(self._h, _stream(stream))
+        if status:
+            _check(status)
+
+    def close(self):
+        if self._h:
+            _lib.load().mrv_plan_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        self.close()
+
+
 # ---------------------------------------------------------------------------------------------
 # the Communicator API, one object per rank (include/megray/communicator.h:32-123)
 

@@ -4,10 +4,16 @@
 #include <cstdio>
 #include <cstring>
 #include <exception>
+#include <memory>
+#include <vector>
+
+#include <hip/hip_runtime_api.h>
 
 #include "megray.h"
 #include "vrank_communicator.h"
+#include "megray/hip_context.h"
 #include "vrank_engine.h"
+#include "vrank_kernels.h"
 #include "vrank_plan.h"
 
 struct mrv_comm {
@@ -200,54 +206,138 @@ int mrv_fold_order(int collective, int order, uint32_t nranks, uint32_t chunk, u
     });
 }
 
+}  // extern "C"
+
+namespace {
+
+// Plans `collective` the way the device entry points do.  Throws for contract violations.
+Status build_plan(Plan& plan, int collective, const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks,
+                  size_t count, DType dt, int order, int schedule, uint32_t root) {
+    switch (collective) {
+        case MRV_ALL_REDUCE:
+            if (as_schedule(schedule) == kSchedRing && dt == MEGRAY_FLOAT16)
+                MEGRAY_THROW("the ring schedule is not offered for FLOAT16 (it would round at every hop)");
+            return plan_all_reduce(plan, sendbuffs, recvbuffs, nranks, count, reduce_elem_size(dt), as_order(order),
+                                   as_schedule(schedule));
+        case MRV_REDUCE_SCATTER:
+            return plan_reduce_scatter(plan, sendbuffs, recvbuffs, nranks, count, reduce_elem_size(dt),
+                                       as_order(order), as_schedule(schedule));
+        case MRV_ALL_GATHER:
+            return plan_all_gather(plan, sendbuffs, recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)));
+        case MRV_ALL_TO_ALL:
+            return plan_all_to_all(plan, sendbuffs, recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)));
+        case MRV_SCATTER:
+            if (root >= nranks) MEGRAY_THROW("root out of range");
+            return plan_scatter(plan, sendbuffs[root], recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)), root);
+        case MRV_GATHER:
+            if (root >= nranks) MEGRAY_THROW("root out of range");
+            return plan_gather(plan, sendbuffs, recvbuffs[root], nranks, count, uint32_t(get_dtype_size(dt)), root);
+        case MRV_BROADCAST:
+            if (root >= nranks) MEGRAY_THROW("root out of range");
+            return plan_broadcast(plan, sendbuffs[root], recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)),
+                                  root);
+        case MRV_REDUCE:
+            if (root >= nranks) MEGRAY_THROW("root out of range");
+            return plan_reduce(plan, sendbuffs, recvbuffs[root], nranks, count, reduce_elem_size(dt), as_order(order),
+                               root);
+        case MRV_REDUCE2:
+            return plan_reduce2(plan, sendbuffs[0], sendbuffs[1], recvbuffs[0], count, reduce_elem_size(dt));
+        default:
+            MEGRAY_THROW("unknown collective");
+    }
+}
+
+bool is_reduction(int collective) {
+    return collective == MRV_ALL_REDUCE || collective == MRV_REDUCE_SCATTER || collective == MRV_REDUCE ||
+           collective == MRV_REDUCE2;
+}
+
+}  // namespace
+
+struct mrv_plan {
+    Plan plan;
+    DType dtype;
+    ReduceOp op;
+    std::vector<KernelCall> calls;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+extern "C" {
+
+int mrv_plan_create(int collective, const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks,
+                    size_t count, int dtype, int op, int order, int schedule, uint32_t root, uint32_t flags,
+                    mrv_plan** out) {
+    return guarded([&] {
+        need(sendbuffs, "sendbuffs is null");
+        need(recvbuffs, "recvbuffs is null");
+        need(out, "plan is null");
+        *out = nullptr;
+        std::unique_ptr<mrv_plan> p(new mrv_plan);
+        p->dtype = static_cast<DType>(dtype);
+        p->op = is_reduction(collective) ? static_cast<ReduceOp>(op) : MEGRAY_SUM;
+        if (is_reduction(collective)) check_reduce_op(p->op);
+        Status st = build_plan(p->plan, collective, sendbuffs, recvbuffs, nranks, count, p->dtype, order, schedule, root);
+        if (st != MEGRAY_OK) return st;
+        st = resolve(p->plan, p->dtype, p->op, p->calls);
+        if (st != MEGRAY_OK) return st;
+        if ((flags & MRV_PLAN_GRAPH) && !p->calls.empty()) {
+            // a chain of kernel nodes, each depending on the one before it
+            HIP_CHECK(hipGraphCreate(&p->graph, 0));
+            hipGraphNode_t prev = nullptr;
+            for (const KernelCall& call : p->calls) {
+                if (!call.grid) continue;
+                void* args[] = {const_cast<void*>(call.launch)};
+                hipKernelNodeParams params;
+                std::memset(&params, 0, sizeof(params));
+                params.func = const_cast<void*>(call.kernel);
+                params.gridDim = dim3(call.grid);
+                params.blockDim = dim3(kThreads);
+                params.kernelParams = args;
+                hipGraphNode_t node = nullptr;
+                HIP_CHECK(hipGraphAddKernelNode(&node, p->graph, prev ? &prev : nullptr, prev ? 1 : 0, &params));
+                prev = node;
+            }
+            HIP_CHECK(hipGraphInstantiate(&p->exec, p->graph, nullptr, nullptr, 0));
+        }
+        *out = p.release();
+        return MEGRAY_OK;
+    });
+}
+
+int mrv_plan_launch(const mrv_plan* plan, void* stream) {
+    return guarded([&] {
+        need(plan, "plan is null");
+        if (plan->exec) {
+            HIP_CHECK(hipGraphLaunch(plan->exec, as_stream(stream)));
+            return MEGRAY_OK;
+        }
+        for (const KernelCall& call : plan->calls)
+            HIP_CHECK(enqueue(call.kernel, call.grid, call.launch, as_stream(stream)));
+        return MEGRAY_OK;
+    });
+}
+
+size_t mrv_plan_launch_count(const mrv_plan* plan) {
+    return plan ? plan->calls.size() : 0;
+}
+
+void mrv_plan_destroy(mrv_plan* plan) {
+    if (!plan) return;
+    if (plan->exec) (void)hipGraphExecDestroy(plan->exec);
+    if (plan->graph) (void)hipGraphDestroy(plan->graph);
+    delete plan;
+}
+
 int mrv_describe(int collective, const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks,
                  size_t count, int dtype, int order, int schedule, uint32_t root, mrv_plan_run* runs, size_t cap,
                  size_t* nruns, uint64_t* bytes_read, uint64_t* bytes_written) {
     return guarded([&] {
         need(sendbuffs, "sendbuffs is null");
         need(recvbuffs, "recvbuffs is null");
-        const DType dt = static_cast<DType>(dtype);
         Plan plan;
-        Status st = MEGRAY_OK;
-        switch (collective) {
-            case MRV_ALL_REDUCE:
-                st = plan_all_reduce(plan, sendbuffs, recvbuffs, nranks, count, reduce_elem_size(dt), as_order(order),
-                                     as_schedule(schedule));
-                break;
-            case MRV_REDUCE_SCATTER:
-                st = plan_reduce_scatter(plan, sendbuffs, recvbuffs, nranks, count, reduce_elem_size(dt),
-                                         as_order(order), as_schedule(schedule));
-                break;
-            case MRV_ALL_GATHER:
-                st = plan_all_gather(plan, sendbuffs, recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)));
-                break;
-            case MRV_ALL_TO_ALL:
-                st = plan_all_to_all(plan, sendbuffs, recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)));
-                break;
-            case MRV_SCATTER:
-                if (root >= nranks) MEGRAY_THROW("root out of range");
-                st = plan_scatter(plan, sendbuffs[root], recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)), root);
-                break;
-            case MRV_GATHER:
-                if (root >= nranks) MEGRAY_THROW("root out of range");
-                st = plan_gather(plan, sendbuffs, recvbuffs[root], nranks, count, uint32_t(get_dtype_size(dt)), root);
-                break;
-            case MRV_BROADCAST:
-                if (root >= nranks) MEGRAY_THROW("root out of range");
-                st = plan_broadcast(plan, sendbuffs[root], recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)),
-                                    root);
-                break;
-            case MRV_REDUCE:
-                if (root >= nranks) MEGRAY_THROW("root out of range");
-                st = plan_reduce(plan, sendbuffs, recvbuffs[root], nranks, count, reduce_elem_size(dt), as_order(order),
-                                 root);
-                break;
-            case MRV_REDUCE2:
-                st = plan_reduce2(plan, sendbuffs[0], sendbuffs[1], recvbuffs[0], count, reduce_elem_size(dt));
-                break;
-            default:
-                MEGRAY_THROW("unknown collective");
-        }
+        Status st = build_plan(plan, collective, sendbuffs, recvbuffs, nranks, count, static_cast<DType>(dtype), order,
+                               schedule, root);
         if (st != MEGRAY_OK) return st;
         size_t n = 0;
         auto emit = [&](const mrv_plan_run& run) {

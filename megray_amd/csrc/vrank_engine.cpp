@@ -30,16 +30,50 @@ void check_reduce_op(ReduceOp op) {
     if (op != MEGRAY_SUM && op != MEGRAY_MAX && op != MEGRAY_MIN) MEGRAY_THROW("unknown reduce op");
 }
 
+Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCall>& calls) {
+    calls.clear();
+    calls.reserve(plan.steps.size());
+    for (const Step& step : plan.steps) {
+        KernelCall call{nullptr, 0, nullptr};
+        switch (step.kind) {
+            case Step::kFold:
+                call = {fold_kernel_for(step.fold, dtype, op), step.fold.total_tiles, &step.fold};
+                break;
+            case Step::kFlat:
+                call = {flat_kernel_for(step.flat, dtype, op), step.flat.total_tiles, &step.flat};
+                break;
+            case Step::kTree:
+                call = {tree_kernel_for(step.tree, dtype, op), step.tree.total_tiles, &step.tree};
+                break;
+            case Step::kPack:
+                call = {pack_kernel_for(step.pack), step.pack.ncopies * step.pack.tiles_per_copy, &step.pack};
+                break;
+        }
+        if (!call.kernel) {
+            MEGRAY_ERROR("no kernel for dtype %d / op %d", int(dtype), int(op));
+            return MEGRAY_INVALID_ARGUMENT;
+        }
+        calls.push_back(call);
+    }
+    return MEGRAY_OK;
+}
+
 Status execute(const Plan& plan, DType dtype, ReduceOp op, hipStream_t stream) {
     for (const Step& step : plan.steps) {
-        if (step.kind == Step::kFold) {
-            HIP_CHECK(launch_fold(step.fold, dtype, op, stream));
-        } else if (step.kind == Step::kFlat) {
-            HIP_CHECK(launch_flat(step.flat, dtype, op, stream));
-        } else if (step.kind == Step::kTree) {
-            HIP_CHECK(launch_tree(step.tree, dtype, op, stream));
-        } else {
-            HIP_CHECK(launch_pack(step.pack, stream));
+        switch (step.kind) {
+            case Step::kFold:
+                HIP_CHECK(enqueue(fold_kernel_for(step.fold, dtype, op), step.fold.total_tiles, &step.fold, stream));
+                break;
+            case Step::kFlat:
+                HIP_CHECK(enqueue(flat_kernel_for(step.flat, dtype, op), step.flat.total_tiles, &step.flat, stream));
+                break;
+            case Step::kTree:
+                HIP_CHECK(enqueue(tree_kernel_for(step.tree, dtype, op), step.tree.total_tiles, &step.tree, stream));
+                break;
+            case Step::kPack:
+                HIP_CHECK(enqueue(pack_kernel_for(step.pack), step.pack.ncopies * step.pack.tiles_per_copy,
+                                  &step.pack, stream));
+                break;
         }
     }
     return MEGRAY_OK;

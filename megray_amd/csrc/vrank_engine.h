@@ -8,6 +8,8 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <vector>
+
 #include "megray/common.h"
 #include "vrank_plan.h"
 
@@ -20,8 +22,18 @@ uint32_t reduce_elem_size(DType dtype);
 // Throws "unknown reduce op" outside SUM / MAX / MIN.
 void check_reduce_op(ReduceOp op);
 
+// One kernel launch of a plan, ready for hipLaunchKernel or a graph node.  `launch` points into
+// the Plan it was resolved from.
+struct KernelCall {
+    const void* kernel;
+    uint32_t grid;
+    const void* launch;
+};
+
 // Enqueue every launch of `plan` on `stream`.
 Status execute(const Plan& plan, DType dtype, ReduceOp op, hipStream_t stream);
+// The same launches, resolved but not enqueued.
+Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCall>& calls);
 
 Status reduce2(const void* i0, const void* i1, void* o, size_t len, DType dtype, ReduceOp op,
                hipStream_t stream);

@@ -1,4 +1,4 @@
-// Launch entry points of the gfx950 kernels (vrank_kernels.hip).
+// Entry points of the gfx950 kernels (vrank_kernels.hip, vrank_fold_<type>.hip).
 #pragma once
 
 #include <hip/hip_runtime_api.h>
@@ -9,17 +9,15 @@
 namespace MegRay {
 namespace vrank {
 
-// Enqueue one fold launch on `stream`.  hipErrorInvalidValue for a dtype / op without a kernel.
-hipError_t launch_fold(const FoldLaunch& launch, DType dtype, ReduceOp op, hipStream_t stream);
+// The kernel that executes a launch descriptor, as a host-side function address usable with
+// hipLaunchKernel and hipGraphAddKernelNode; nullptr for a dtype / op without a kernel.
+const void* fold_kernel_for(const FoldLaunch& launch, DType dtype, ReduceOp op);
+const void* flat_kernel_for(const FlatLaunch& launch, DType dtype, ReduceOp op);  // rank count 2, 3, 4 or 8
+const void* tree_kernel_for(const TreeLaunch& launch, DType dtype, ReduceOp op);
+const void* pack_kernel_for(const PackLaunch& launch);
 
-// Enqueue one flat fold launch on `stream` (rank count 2, 3, 4 or 8).
-hipError_t launch_flat(const FlatLaunch& launch, DType dtype, ReduceOp op, hipStream_t stream);
-
-// Enqueue one element-wise binomial-tree launch on `stream`.
-hipError_t launch_tree(const TreeLaunch& launch, DType dtype, ReduceOp op, hipStream_t stream);
-
-// Enqueue one pack launch on `stream`.
-hipError_t launch_pack(const PackLaunch& launch, hipStream_t stream);
+// Enqueue `kernel` over `grid` one-wavefront workgroups with `*launch` as its only argument.
+hipError_t enqueue(const void* kernel, uint32_t grid, const void* launch, hipStream_t stream);
 
 }  // namespace vrank
 }  // namespace MegRay

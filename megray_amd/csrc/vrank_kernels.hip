@@ -9,10 +9,10 @@ namespace vrank {
 
 namespace detail {
 // instantiated in vrank_fold_<type>.hip
-#define MEGRAY_VRANK_EXTERN(T)                                                                 \
-    extern template hipError_t launch_fold_t<T>(const FoldLaunch&, int, hipStream_t);          \
-    extern template hipError_t launch_flat_t<T>(const FlatLaunch&, int, hipStream_t);          \
-    extern template hipError_t launch_tree_t<T>(const TreeLaunch&, int, hipStream_t);
+#define MEGRAY_VRANK_EXTERN(T)                                                \
+    extern template const void* fold_kernel_t<T>(const FoldLaunch&, int);     \
+    extern template const void* flat_kernel_t<T>(const FlatLaunch&, int);     \
+    extern template const void* tree_kernel_t<T>(int);
 MEGRAY_VRANK_EXTERN(int8_t)
 MEGRAY_VRANK_EXTERN(uint8_t)
 MEGRAY_VRANK_EXTERN(int32_t)
@@ -89,16 +89,16 @@ FoldFn pick_copy(uint32_t elem_size) {
     }
 }
 
-// Runs `call.template operator()<T>()` for the element type that carries out `op` on `dtype`:
-// integer SUM wraps, so both signs share the unsigned kernel.
+// Calls `call(T{}, k)` for the element type that carries out `op` on `dtype`: integer SUM wraps,
+// so both signs share the unsigned kernel.
 template <typename F>
-hipError_t with_type(DType dtype, ReduceOp op, F&& call) {
+const void* with_type(DType dtype, ReduceOp op, F&& call) {
     int k;
     switch (op) {
         case MEGRAY_SUM: k = kSum; break;
         case MEGRAY_MAX: k = kMax; break;
         case MEGRAY_MIN: k = kMin; break;
-        default: return hipErrorInvalidValue;
+        default: return nullptr;
     }
     const bool sum = k == kSum;
     switch (dtype) {
@@ -111,34 +111,26 @@ hipError_t with_type(DType dtype, ReduceOp op, F&& call) {
         case MEGRAY_FLOAT16: return call(_Float16{}, k);
         case MEGRAY_FLOAT32: return call(float{}, k);
         case MEGRAY_FLOAT64: return call(double{}, k);
-        default: return hipErrorInvalidValue;
+        default: return nullptr;
     }
 }
 
 }  // namespace
 
-hipError_t launch_fold(const FoldLaunch& L, DType dtype, ReduceOp op, hipStream_t stream) {
-    if (L.total_tiles == 0) return hipSuccess;
-    if (L.nfold == 1) {
-        hipLaunchKernelGGL(pick_copy(L.elem_size), dim3(L.total_tiles), dim3(kThreads), 0, stream, L);
-        return hipGetLastError();
-    }
-    return with_type(dtype, op, [&](auto tag, int k) { return launch_fold_t<decltype(tag)>(L, k, stream); });
+const void* fold_kernel_for(const FoldLaunch& L, DType dtype, ReduceOp op) {
+    if (L.nfold == 1) return reinterpret_cast<const void*>(pick_copy(L.elem_size));
+    return with_type(dtype, op, [&](auto tag, int k) { return fold_kernel_t<decltype(tag)>(L, k); });
 }
 
-hipError_t launch_flat(const FlatLaunch& L, DType dtype, ReduceOp op, hipStream_t stream) {
-    if (L.total_tiles == 0) return hipSuccess;
-    return with_type(dtype, op, [&](auto tag, int k) { return launch_flat_t<decltype(tag)>(L, k, stream); });
+const void* flat_kernel_for(const FlatLaunch& L, DType dtype, ReduceOp op) {
+    return with_type(dtype, op, [&](auto tag, int k) { return flat_kernel_t<decltype(tag)>(L, k); });
 }
 
-hipError_t launch_tree(const TreeLaunch& L, DType dtype, ReduceOp op, hipStream_t stream) {
-    if (L.total_tiles == 0) return hipSuccess;
-    return with_type(dtype, op, [&](auto tag, int k) { return launch_tree_t<decltype(tag)>(L, k, stream); });
+const void* tree_kernel_for(const TreeLaunch&, DType dtype, ReduceOp op) {
+    return with_type(dtype, op, [&](auto tag, int k) { return tree_kernel_t<decltype(tag)>(k); });
 }
 
-hipError_t launch_pack(const PackLaunch& L, hipStream_t stream) {
-    const uint64_t blocks = uint64_t(L.ncopies) * L.tiles_per_copy;
-    if (blocks == 0) return hipSuccess;
+const void* pack_kernel_for(const PackLaunch& L) {
     void (*fn)(const PackLaunch) = nullptr;
     switch (L.width) {
         case 16: fn = pack_kernel<u32x4, pack_unroll()>; break;
@@ -146,10 +138,16 @@ hipError_t launch_pack(const PackLaunch& L, hipStream_t stream) {
         case 4: fn = pack_kernel<uint32_t, pack_unroll()>; break;
         case 2: fn = pack_kernel<uint16_t, pack_unroll()>; break;
         case 1: fn = pack_kernel<uint8_t, pack_unroll()>; break;
-        default: return hipErrorInvalidValue;
+        default: break;
     }
-    hipLaunchKernelGGL(fn, dim3(uint32_t(blocks)), dim3(kThreads), 0, stream, L);
-    return hipGetLastError();
+    return reinterpret_cast<const void*>(fn);
+}
+
+hipError_t enqueue(const void* kernel, uint32_t grid, const void* launch, hipStream_t stream) {
+    if (!kernel) return hipErrorInvalidValue;
+    if (!grid) return hipSuccess;
+    void* args[] = {const_cast<void*>(launch)};
+    return hipLaunchKernel(kernel, dim3(grid), dim3(kThreads), args, 0, stream);
 }
 
 }  // namespace vrank

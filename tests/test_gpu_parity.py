@@ -323,3 +323,44 @@ def test_reduce_to_root(dtype):
                         torch.cuda.synchronize()
                         assert_same(to_host(d_out, ins[0].dtype), orc.fold_all_reduce(ins, dtype, op, order)[0],
                                     f"reduce order={order}")
+
+
+def test_planned_collectives_and_graph_replay():
+    """mrv_plan_*: a plan launched repeatedly, eagerly and as a HIP graph of kernel nodes, gives the
+    eager result on every replay, with other work and host syncs between the replays."""
+    rng = np.random.default_rng(11)
+    nranks, length = 8, 40000 + 3
+    for sched in (mr.Schedule.FUSED, mr.Schedule.TWO_PHASE, mr.Schedule.RING):
+        ins = [rand_array(orc.FLOAT32, length, rng) for _ in range(nranks)]
+        want = orc.ucx_all_reduce(ins, orc.FLOAT32, orc.SUM)
+        d_in = [to_device(x) for x in ins]
+        for graph in (False, True):
+            d_out = [empty_device(length * 4) for _ in range(nranks)]
+            plan = mr.CollectivePlan(mr.Collective.ALL_REDUCE, d_in, d_out, length, mr.DType.FLOAT32, mr.ReduceOp.SUM,
+                                     schedule=sched, graph=graph)
+            assert plan.launch_count == {mr.Schedule.FUSED: 1, mr.Schedule.TWO_PHASE: 2,
+                                         mr.Schedule.RING: 1 + 2 * (nranks - 1)}[sched]
+            for replay in range(4):
+                for o in d_out:
+                    o.fill_(replay)  # the program's own eager work between replays
+                torch.cuda.synchronize()
+                plan.launch()
+                torch.cuda.synchronize()
+                for r in range(nranks):
+                    assert_same(to_host(d_out[r], np.float32), want[r], f"sched={sched} graph={graph} replay={replay}")
+            plan.close()
+    # new data in the same buffers is picked up by a replay (the plan holds addresses, not values)
+    ins = [rand_array(orc.INT32, 5000, rng) for _ in range(4)]
+    d_in = [to_device(x) for x in ins]
+    d_out = [empty_device(5000 * 4) for _ in range(4)]
+    plan = mr.CollectivePlan(mr.Collective.ALL_REDUCE, d_in, d_out, 5000, mr.DType.INT32, mr.ReduceOp.MAX,
+                             schedule=mr.Schedule.TWO_PHASE, graph=True)
+    for _ in range(3):
+        ins = [rand_array(orc.INT32, 5000, rng) for _ in range(4)]
+        for d, x in zip(d_in, ins):
+            d.copy_(torch.from_numpy(x.view(np.uint8).copy()))
+        plan.launch()
+        torch.cuda.synchronize()
+        assert_same(to_host(d_out[2], np.int32), np.stack(ins).max(axis=0), "graph replay on new data")
+    with pytest.raises(mr.MegRayError, match="unknown reduce op"):
+        mr.CollectivePlan(mr.Collective.ALL_REDUCE, d_in, d_out, 5000, mr.DType.INT32, 9)
