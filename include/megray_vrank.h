@@ -156,7 +156,7 @@ typedef struct mrv_plan_run {
     uint32_t step;          /* launch index within the collective */
     uint32_t kind;          /* 0 = fold run, 1 = block copy of a pack launch */
     uint32_t nfold;         /* fold: inputs combined per element (1 = copy) */
-    uint32_t nout;          /* fold: destinations */
+    uint32_t nout;          /* destinations: ranks out_first .. out_first + nout - 1 (mod nranks) */
     uint32_t new_wins_ties; /* fold */
     uint32_t vector;        /* fold: 0 = element by element, 1 = 16-byte vectors, 2 = run of a flat launch
                                (vectors on the buffer's own 1 KiB tile grid); pack: bytes per lane access */

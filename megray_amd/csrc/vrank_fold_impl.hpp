@@ -268,7 +268,7 @@ __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
                 for (int j = 0; j < K; ++j) {
                     const char* src = static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off;
 #pragma unroll
-                    for (int u = 0; u < U; ++u) x[j][u] = load_vec(src + (u * kThreads + tid) * kVecBytes);
+                    for (int u = 0; u < U; ++u) x[j][u] = load_tile_vec(src + u * (kThreads * kVecBytes), tid);
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
@@ -280,7 +280,7 @@ __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
                 {
                     const char* src = static_cast<const char*>(L.in[start]) + in_off;
 #pragma unroll
-                    for (int u = 0; u < U; ++u) acc[u].seed(load_vec(src + (u * kThreads + tid) * kVecBytes));
+                    for (int u = 0; u < U; ++u) acc[u].seed(load_tile_vec(src + u * (kThreads * kVecBytes), tid));
                 }
                 uint32_t j = 1;
                 for (; j + 4 <= nfold; j += 4) {
@@ -290,7 +290,7 @@ __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
                         const char* src =
                                 static_cast<const char*>(L.in[rotate_rank(start, dir, j + q, nr)]) + in_off;
 #pragma unroll
-                        for (int u = 0; u < U; ++u) x[q][u] = load_vec(src + (u * kThreads + tid) * kVecBytes);
+                        for (int u = 0; u < U; ++u) x[q][u] = load_tile_vec(src + u * (kThreads * kVecBytes), tid);
                     }
 #pragma unroll
                     for (int q = 0; q < 4; ++q)
@@ -301,7 +301,7 @@ __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
                     const char* src = static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off;
 #pragma unroll
                     for (int u = 0; u < U; ++u)
-                        acc[u].fold(load_vec(src + (u * kThreads + tid) * kVecBytes), new_wins);
+                        acc[u].fold(load_tile_vec(src + u * (kThreads * kVecBytes), tid), new_wins);
                 }
             }
             u32x4 res[U];
@@ -310,7 +310,7 @@ __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
             for (uint32_t m = 0; m < nout; ++m) {
                 char* dst = static_cast<char*>(L.out[rotate_rank(out_first, 1, m, nr)]) + out_off;
 #pragma unroll
-                for (int u = 0; u < U; ++u) store_vec(dst + (u * kThreads + tid) * kVecBytes, res[u]);
+                for (int u = 0; u < U; ++u) store_tile_vec(dst + u * (kThreads * kVecBytes), tid, res[u]);
             }
         } else {
             // last tile of the segment: predicate every vector

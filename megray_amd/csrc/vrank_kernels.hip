@@ -42,7 +42,7 @@ __global__ void __launch_bounds__(kThreads) pack_kernel(const PackLaunch L) {
     const uint32_t copy = blockIdx.x / L.tiles_per_copy;
     const uint32_t tile = blockIdx.x - copy * L.tiles_per_copy;
     const uint32_t n = L.nranks;
-    uint32_t src_rank, dst_rank, src_block, dst_block;
+    uint32_t src_rank, dst_rank, src_block, dst_block, ndst = 1;
     if (L.mode == kPackAllToAll) {
         src_rank = copy / n;
         src_block = copy - src_rank * n;
@@ -53,32 +53,54 @@ __global__ void __launch_bounds__(kThreads) pack_kernel(const PackLaunch L) {
         src_block = copy;
         dst_rank = copy;
         dst_block = 0;
-    } else {
+    } else if (L.mode == kPackGather) {
         src_rank = copy;
         src_block = 0;
         dst_rank = L.root;
         dst_block = copy;
+    } else {  // kPackAllGather: read once, write the block into every rank's buffer
+        src_rank = copy;
+        src_block = 0;
+        dst_rank = 0;
+        dst_block = copy;
+        ndst = n;
     }
     const uint64_t base = uint64_t(tile) * (kThreads * U) * sizeof(W);
     const char* src = static_cast<const char*>(L.in[src_rank]) + src_block * L.block_bytes + base;
-    char* dst = static_cast<char*>(L.out[dst_rank]) + dst_block * L.block_bytes + base;
+    const uint64_t dst_off = dst_block * L.block_bytes + base;
     const uint64_t left = (L.block_bytes - base) / sizeof(W);
     const uint32_t tid = threadIdx.x;
     if (left >= uint64_t(kThreads) * U) {
         W x[U];
+        if constexpr (sizeof(W) == kVecBytes) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) x[u] = load_w<W>(src + (u * kThreads + tid) * sizeof(W));
+            for (int u = 0; u < U; ++u) x[u] = load_tile_vec(src + u * (kThreads * kVecBytes), tid);
+            for (uint32_t m = 0; m < ndst; ++m) {
+                char* dst = static_cast<char*>(L.out[dst_rank + m]) + dst_off;
 #pragma unroll
-        for (int u = 0; u < U; ++u) store_w<W>(dst + (u * kThreads + tid) * sizeof(W), x[u]);
+                for (int u = 0; u < U; ++u) store_tile_vec(dst + u * (kThreads * kVecBytes), tid, x[u]);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u) x[u] = load_w<W>(src + (u * kThreads + tid) * sizeof(W));
+            for (uint32_t m = 0; m < ndst; ++m) {
+                char* dst = static_cast<char*>(L.out[dst_rank + m]) + dst_off;
+#pragma unroll
+                for (int u = 0; u < U; ++u) store_w<W>(dst + (u * kThreads + tid) * sizeof(W), x[u]);
+            }
+        }
     } else {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const uint32_t i = u * kThreads + tid;
-            if (i < left) store_w<W>(dst + i * sizeof(W), load_w<W>(src + i * sizeof(W)));
+            if (i < left) {
+                const W x = load_w<W>(src + i * sizeof(W));
+                for (uint32_t m = 0; m < ndst; ++m)
+                    store_w<W>(static_cast<char*>(L.out[dst_rank + m]) + dst_off + i * sizeof(W), x);
+            }
         }
     }
 }
-
 
 FoldFn pick_copy(uint32_t elem_size) {
     switch (elem_size) {

@@ -417,6 +417,11 @@ Status plan_reduce_scatter(Plan& plan, const void* const* send, void* const* rec
     return MEGRAY_OK;
 }
 
+namespace {
+Status add_pack(Plan& plan, const void* const* in, void* const* out, uint32_t nranks, uint64_t block_bytes,
+                uint32_t mode, uint32_t root, uint32_t ncopies);
+}
+
 Status plan_all_gather(Plan& plan, const void* const* send, void* const* recv, uint32_t nranks,
                        uint64_t sendlen, uint32_t elem_size) {
     PLAN_TRY(check_ranks(nranks));
@@ -433,10 +438,12 @@ Status plan_all_gather(Plan& plan, const void* const* send, void* const* recv, u
             if (!in_place) return invalid("a receive buffer overlaps a send buffer out of place");
         }
     }
-    FoldBuilder copy(plan, send, recv, nranks, 1, nranks, elem_size, false);
-    for (uint32_t i = 0; i < nranks; ++i) copy.add_run(0, i * sendlen, sendlen, uint8_t(i), 1, 0);
-    copy.finish();
-    return MEGRAY_OK;
+    // one pack launch: block i is read once from rank i and written into slot i of every rank
+    const uint64_t before = plan.steps.size();
+    Status st = add_pack(plan, send, recv, nranks, sendlen * elem_size, kPackAllGather, 0, nranks);
+    if (st == MEGRAY_OK && plan.steps.size() > before)
+        plan.bytes_written += sendlen * elem_size * nranks * (nranks - 1);  // add_pack counted one copy per block
+    return st;
 }
 
 namespace {

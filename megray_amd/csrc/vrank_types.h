@@ -97,6 +97,7 @@ enum PackMode : uint32_t {
     kPackAllToAll = 0,  // copy b = i*N + j : in[i] block j  -> out[j] block i
     kPackScatter = 1,   // copy b = i       : in[root] block i -> out[i] block 0
     kPackGather = 2,    // copy b = i       : in[i] block 0    -> out[root] block i
+    kPackAllGather = 3, // copy b = i       : in[i] block 0    -> block i of EVERY out
 };
 
 // One launch of the pack kernel: `ncopies` equally sized block copies whose endpoints follow

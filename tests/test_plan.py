@@ -80,11 +80,13 @@ def execute(runs, sends, recvs, nranks, op, elem_size, send_ptrs, recv_ptrs):
                         dst = (run["out_first"] + m) % nranks
                         assert (recv_ptrs[dst] + run["out_begin"] * elem_size) % 16 == 0
             else:
-                s, d = run["start"], run["out_first"]
+                s = run["start"]
                 a, b, cnt = run["in_begin"], run["out_begin"], run["count"]
-                recvs[d].view(np.uint8)[b:b + cnt] = sends[s].view(np.uint8)[a:a + cnt]
                 width = run["vector"]
-                assert cnt % width == 0 and (send_ptrs[s] + a) % width == 0 and (recv_ptrs[d] + b) % width == 0
+                for m in range(run["nout"]):
+                    d = (run["out_first"] + m) % nranks
+                    recvs[d].view(np.uint8)[b:b + cnt] = sends[s].view(np.uint8)[a:a + cnt]
+                    assert cnt % width == 0 and (send_ptrs[s] + a) % width == 0 and (recv_ptrs[d] + b) % width == 0
     return recvs
 
 
