@@ -66,5 +66,21 @@ def build_library(verbose=True):
     return LIB_PATH
 
 
+CPP_TEST_SRC = os.path.join(ROOT, "tests", "cpp", "test_vrank_opr.cpp")
+CPP_TEST_BIN = os.path.join(ROOT, "tests", "cpp", "test_vrank_opr")
+
+
+def build_cpp_test():
+    """Compile the thread-per-rank C++ API test against the library just built."""
+    cmd = [HIPCC, "-std=c++17", "-O2", "-x", "c++", "-D__HIP_PLATFORM_AMD__=1", f"-I{os.path.join(ROOT, 'include')}",
+           f"-I{ROCM}/include", CPP_TEST_SRC, "-o", CPP_TEST_BIN, f"-L{HERE}", "-lmegray_vrank", f"-L{ROCM}/lib",
+           "-lamdhip64", "-pthread", "-Wl,-rpath,$ORIGIN/../../megray_amd", f"-Wl,-rpath,{ROCM}/lib"]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"building {CPP_TEST_SRC} failed:\n{proc.stdout}\n{proc.stderr}")
+    return CPP_TEST_BIN
+
+
 if __name__ == "__main__":
     print(build_library())
+    print(build_cpp_test())
