@@ -1,0 +1,255 @@
+// megray_performance: the benchmark of the MegRay API for the MEGRAY_VRANK backend.
+//
+// Command line and table follow the reference's test/performance.cpp (options :443-496, table
+// :342-362: bufsize / time(us) / speed(GB/s) / iters with speed = bufsize_bytes / avg_us / 1000, the
+// per-rank payload over wall time), so numbers line up with anyone's MegRay runs.  Two columns are
+// added: the HBM bytes the collective moves algorithmically per second, and that as a fraction of
+// the 8 TB/s peak.  "-d" is the number of virtual ranks; all of them live on GPU 0 of this node,
+// each driven by its own thread with its own stream, exactly like the reference's thread per device.
+#include <hip/hip_runtime.h>
+#include <unistd.h>
+
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <functional>
+#include <iomanip>
+#include <iostream>
+#include <memory>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "megray.h"
+
+namespace {
+
+struct Arguments {
+    std::string backends = "ALL";
+    std::string master_ip = "127.0.0.1";
+    int port = 2395;
+    int n_nodes = 1;
+    int node_rank = 0;
+    int n_devs = 2;
+    std::vector<size_t> sizes = {8, 1024, 512 * 1024, 1024 * 1024, 10 * 1024 * 1024};
+    int send_dev = 0;
+    int recv_dev = 1;
+    int warmup_iters = 100;
+    int iters = 100;
+    std::string func_select = "ALL";
+    size_t bufsize = 0, in_bufsize = 0, out_bufsize = 0;
+};
+
+using Kernel = std::function<void(std::shared_ptr<MegRay::Communicator>, void*, void*, std::shared_ptr<MegRay::Context>)>;
+
+struct Func {
+    std::string name;
+    // buffer sizes per rank as multiples of bufsize (N = ranks), and HBM bytes moved per collective
+    std::function<size_t(size_t, size_t)> in_bytes, out_bytes, hbm_bytes;
+    std::function<Kernel(const Arguments&, int)> make;
+};
+
+#define CHECK_HIP(expr)                                                                    \
+    do {                                                                                   \
+        hipError_t e_ = (expr);                                                            \
+        if (e_ != hipSuccess) {                                                            \
+            std::fprintf(stderr, "hip error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); \
+            std::exit(1);                                                                  \
+        }                                                                                  \
+    } while (0)
+
+size_t now_us() {
+    return size_t(std::chrono::duration_cast<std::chrono::microseconds>(
+                          std::chrono::steady_clock::now().time_since_epoch())
+                          .count());
+}
+
+// worker() of test/performance.cpp:103-137
+void worker(const Func& func, Arguments args, int dev, int port, double* res) {
+    CHECK_HIP(hipSetDevice(0));
+    hipStream_t stream;
+    CHECK_HIP(hipStreamCreate(&stream));
+    auto context = MegRay::HipContext::make(stream);
+    auto comm = MegRay::get_communicator(args.n_devs, dev, MegRay::MEGRAY_VRANK);
+    if (comm->init(args.master_ip.c_str(), port) != MegRay::MEGRAY_OK) std::exit(1);
+    void *in_ptr = nullptr, *out_ptr = nullptr;
+    CHECK_HIP(hipMalloc(&in_ptr, args.in_bufsize ? args.in_bufsize : 1));
+    CHECK_HIP(hipMalloc(&out_ptr, args.out_bufsize ? args.out_bufsize : 1));
+    CHECK_HIP(hipMemset(in_ptr, 0, args.in_bufsize));
+    Kernel kernel = func.make(args, dev);
+    for (int i = 0; i < args.warmup_iters; i++) kernel(comm, in_ptr, out_ptr, context);
+    CHECK_HIP(hipStreamSynchronize(stream));
+    size_t t0 = now_us();
+    for (int i = 0; i < args.iters; i++) kernel(comm, in_ptr, out_ptr, context);
+    CHECK_HIP(hipStreamSynchronize(stream));
+    size_t t1 = now_us();
+    CHECK_HIP(hipFree(in_ptr));
+    CHECK_HIP(hipFree(out_ptr));
+    CHECK_HIP(hipStreamDestroy(stream));
+    if (dev == 0) *res = double(t1 - t0) / args.iters;
+}
+
+double run_test(const Func& func, const Arguments& args) {
+    double res = 0;
+    int port = MegRay::get_free_port();
+    if (MegRay::create_server(args.n_devs, port) != MegRay::MEGRAY_OK) std::exit(1);
+    std::vector<std::thread> threads;
+    for (int i = 0; i < args.n_devs; i++) threads.emplace_back(worker, std::cref(func), args, i, port, &res);
+    for (auto& t : threads) t.join();
+    return res;
+}
+
+std::vector<Func> all_funcs() {
+    using A = const Arguments&;
+    const auto f32 = MegRay::MEGRAY_FLOAT32;
+    auto one = [](size_t b, size_t) { return b; };
+    auto all = [](size_t b, size_t n) { return b * n; };
+    std::vector<Func> f;
+    f.push_back({"send_recv", one, one, [](size_t b, size_t) { return 2 * b; }, [=](A a, int dev) -> Kernel {
+                     return [=](auto comm, void* in, void* out, auto ctx) {
+                         if (dev == a.send_dev) comm->send(in, a.bufsize / 4, f32, a.recv_dev, ctx);
+                         if (dev == a.recv_dev) comm->recv(out, a.bufsize / 4, f32, a.send_dev, ctx);
+                     };
+                 }});
+    f.push_back({"all_reduce_sum", one, one, [](size_t b, size_t n) { return 2 * n * b; }, [=](A a, int) -> Kernel {
+                     return [=](auto comm, void* in, void* out, auto ctx) {
+                         comm->all_reduce(in, out, a.bufsize / 4, f32, MegRay::MEGRAY_SUM, ctx);
+                     };
+                 }});
+    f.push_back({"scatter", all, one, [](size_t b, size_t n) { return 2 * n * b; }, [=](A a, int) -> Kernel {
+                     return [=](auto comm, void* in, void* out, auto ctx) {
+                         comm->scatter(in, out, a.bufsize / 4, f32, 0, ctx);
+                     };
+                 }});
+    f.push_back({"gather", one, all, [](size_t b, size_t n) { return 2 * n * b; }, [=](A a, int) -> Kernel {
+                     return [=](auto comm, void* in, void* out, auto ctx) {
+                         comm->gather(in, out, a.bufsize / 4, f32, 0, ctx);
+                     };
+                 }});
+    f.push_back({"all_to_all", all, all, [](size_t b, size_t n) { return 2 * n * n * b; }, [=](A a, int) -> Kernel {
+                     return [=](auto comm, void* in, void* out, auto ctx) {
+                         comm->all_to_all(in, out, a.bufsize / 4, f32, ctx);
+                     };
+                 }});
+    f.push_back({"all_gather", one, all, [](size_t b, size_t n) { return n * b + n * n * b; }, [=](A a, int) -> Kernel {
+                     return [=](auto comm, void* in, void* out, auto ctx) {
+                         comm->all_gather(in, out, a.bufsize / 4, f32, ctx);
+                     };
+                 }});
+    f.push_back({"reduce_scatter_sum", all, one, [](size_t b, size_t n) { return n * n * b + n * b; },
+                 [=](A a, int) -> Kernel {
+                     return [=](auto comm, void* in, void* out, auto ctx) {
+                         comm->reduce_scatter(in, out, a.bufsize / 4, f32, MegRay::MEGRAY_SUM, ctx);
+                     };
+                 }});
+    f.push_back({"broadcast", one, one, [](size_t b, size_t n) { return b + n * b; }, [=](A a, int) -> Kernel {
+                     return [=](auto comm, void* in, void* out, auto ctx) {
+                         comm->broadcast(in, out, a.bufsize / 4, f32, 0, ctx);
+                     };
+                 }});
+    f.push_back({"reduce_sum", one, one, [](size_t b, size_t n) { return n * b + b; }, [=](A a, int) -> Kernel {
+                     return [=](auto comm, void* in, void* out, auto ctx) {
+                         comm->reduce(in, out, a.bufsize / 4, f32, MegRay::MEGRAY_SUM, 0, ctx);
+                     };
+                 }});
+    return f;
+}
+
+void show_help(const char* argv0) {
+    std::cout << argv0
+              << " {OPTIONS}\n\n    Benchmark of the MegRay API on the MEGRAY_VRANK backend.\n\n  OPTIONS:\n"
+                 "      -h          this help\n"
+                 "      -d[int]     number of devs = virtual ranks on GPU 0 (default 2, at most 16)\n"
+                 "      -I[string]  master IP (default 127.0.0.1)\n"
+                 "      -P[int]     master port (accepted; every run draws a free port)\n"
+                 "      -n[int]     number of nodes: only 1 (all ranks share one GPU)\n"
+                 "      -r[int]     rank of node: only 0\n"
+                 "      -e[string]  backend: ALL or VRANK\n"
+                 "      -f[string]  function: ALL, all_reduce, send_recv, scatter, gather, all_to_all,\n"
+                 "                  all_gather, reduce_scatter, broadcast, reduce\n"
+                 "      -s[int]     packet size in bytes per rank (default: 8, 1 KiB, 512 KiB, 1 MiB, 10 MiB)\n"
+                 "      -w[int]     warm-up iterations (default 100)\n"
+                 "      -i[int]     timed iterations (default 100)\n"
+                 "      -A -B       send/recv: sending node rank / dev (default 0 / 0)\n"
+                 "      -C -D       send/recv: receiving node rank / dev (default 0 / 1)\n\n"
+                 "    example: "
+              << argv0 << " -d 8 -f all_reduce -s 1073741824 -w 5 -i 20\n";
+}
+
+template <typename T>
+void print(T value) {
+    std::cout << std::setw(16) << value;
+}
+
+}  // namespace
+
+int main(int argc, char* argv[]) {
+    Arguments args;
+    int ch;
+    while ((ch = getopt(argc, argv, "hd:I:P:n:r:e:f:s:w:i:A:B:C:D:")) != EOF) {
+        switch (ch) {
+            case 'h': show_help(argv[0]); return 0;
+            case 'd': args.n_devs = std::atoi(optarg); break;
+            case 'I': args.master_ip = optarg; break;
+            case 'P': args.port = std::atoi(optarg); break;
+            case 'n': args.n_nodes = std::atoi(optarg); break;
+            case 'r': args.node_rank = std::atoi(optarg); break;
+            case 'e': args.backends = optarg; break;
+            case 'f': args.func_select = optarg; break;
+            case 's': args.sizes = std::vector<size_t>(1, size_t(std::atoll(optarg))); break;
+            case 'w': args.warmup_iters = std::atoi(optarg); break;
+            case 'i': args.iters = std::atoi(optarg); break;
+            case 'A': break;  // node ranks of the send/recv pair: one node only
+            case 'C': break;
+            case 'B': args.send_dev = std::atoi(optarg); break;
+            case 'D': args.recv_dev = std::atoi(optarg); break;
+            default: std::cerr << "Error arguments\n"; show_help(argv[0]); return 1;
+        }
+    }
+    if (args.n_nodes != 1 || args.node_rank != 0) {
+        std::cerr << "the vrank backend keeps all ranks on one GPU of one node: use -n 1 -r 0\n";
+        return 1;
+    }
+    if (args.backends != "ALL" && args.backends != "VRANK") {
+        std::cerr << "this build has one backend: VRANK\n";
+        return 1;
+    }
+    if (args.n_devs < 1 || args.n_devs > 16 || args.iters < 1) {
+        std::cerr << "need 1 <= -d <= 16 and -i >= 1\n";
+        return 1;
+    }
+    int devices = 0;
+    if (hipGetDeviceCount(&devices) != hipSuccess || devices < 1) {
+        std::cerr << "no GPU\n";
+        return 2;
+    }
+    const std::string want = args.func_select;
+    for (const Func& func : all_funcs()) {
+        if (want != "ALL" && func.name.rfind(want, 0) != 0) continue;
+        if (func.name == "send_recv" && (args.n_devs < 2 || args.send_dev == args.recv_dev)) continue;
+        std::cout << "\nTesting " << func.name << " on backend VRANK (" << args.n_devs << " virtual ranks)\n";
+        print("bufsize");
+        print("time(us)");
+        print("speed(GB/s)");
+        print("iters");
+        print("hbm(GB/s)");
+        print("hbm(%peak)");
+        std::cout << std::endl;
+        for (size_t size : args.sizes) {
+            Arguments run = args;
+            run.bufsize = size / 4 * 4;
+            run.in_bufsize = func.in_bytes(run.bufsize, args.n_devs);
+            run.out_bufsize = func.out_bytes(run.bufsize, args.n_devs);
+            double avg_us = run_test(func, run);
+            double hbm = func.hbm_bytes(run.bufsize, args.n_devs) / avg_us / 1000.0;
+            print(size);
+            print(avg_us);
+            print(1.0 * size / avg_us / 1000);
+            print(args.iters);
+            print(hbm);
+            print(hbm / 80.0);
+            std::cout << std::endl;
+        }
+    }
+    return 0;
+}

@@ -57,10 +57,14 @@ struct PendingP2P {
 // The process-local meeting point of the N rank objects of one communicator group.
 class Group {
 public:
-    explicit Group(uint32_t nranks) : m_nranks(nranks), m_slots(nranks), m_mail(size_t(nranks) * nranks) {}
+    explicit Group(uint32_t nranks)
+            : m_nranks(nranks), m_slots(nranks), m_arrive(nranks, nullptr), m_mail(size_t(nranks) * nranks) {}
 
     ~Group() {
         for (hipEvent_t ev : m_events) (void)hipEventDestroy(ev);
+        for (hipEvent_t ev : m_arrive)
+            if (ev) (void)hipEventDestroy(ev);
+        if (m_done) (void)hipEventDestroy(m_done);
     }
 
     // Groups are found by the 128-bit id rank 0 drew and the bootstrap broadcast.
@@ -82,9 +86,14 @@ public:
     // Deposit `call` for `rank` and wait until every rank of the group has done the same; the last
     // to arrive enqueues the collective for all.  Every rank returns the same Status.
     Status collective(uint32_t rank, const Call& call) {
+        // Every rank marks, on its own stream and from its own thread, the point its buffers are
+        // ready at; the N records run in parallel instead of one after the other in the leader.
+        if (!m_arrive[rank]) HIP_CHECK(hipEventCreateWithFlags(&m_arrive[rank], hipEventDisableTiming));
+        HIP_CHECK(hipEventRecord(m_arrive[rank], call.stream));
+
         std::unique_lock<std::mutex> lock(m_mutex);
         m_slots[rank] = call;
-        const uint64_t gen = m_generation;
+        const uint64_t gen = m_generation.load(std::memory_order_relaxed);
         if (++m_arrived == m_nranks) {
             Status st;
             try {
@@ -94,13 +103,32 @@ public:
                 st = MEGRAY_INVALID_ARGUMENT;
             }
             m_result[gen & 1] = st;
+            m_lead_stream[gen & 1] = call.stream;
             m_arrived = 0;
-            ++m_generation;
+            m_generation.store(gen + 1, std::memory_order_release);
+            lock.unlock();
             m_cv.notify_all();
             return st;
         }
-        m_cv.wait(lock, [&] { return m_generation != gen; });
-        return m_result[gen & 1];
+        lock.unlock();
+        // The other ranks are usually a few microseconds away: poll the generation for a while before
+        // going to sleep on the condition variable (a sleeping thread costs tens of microseconds to wake).
+        bool released = false;
+        for (int spin = 0; spin < kSpinPolls && !released; ++spin) {
+            released = m_generation.load(std::memory_order_acquire) != gen;
+            if (!released) __builtin_ia32_pause();
+        }
+        if (!released) {
+            lock.lock();
+            m_cv.wait(lock, [&] { return m_generation.load(std::memory_order_acquire) != gen; });
+            lock.unlock();
+        }
+        // ... and orders its own stream behind the result.  The done event is not recorded again before
+        // every rank has passed this point: the next collective needs all of them to arrive first.
+        const Status st = m_result[gen & 1];
+        if (st == MEGRAY_OK && call.stream != m_lead_stream[gen & 1])
+            HIP_CHECK(hipStreamWaitEvent(call.stream, m_done, 0));
+        return st;
     }
 
     // Post one side of a point-to-point transfer; the side that finds its counterpart already
@@ -163,9 +191,8 @@ private:
         // order the leader's stream behind everything already enqueued on the other ranks' streams
         hipStream_t stream = lead.stream;
         for (uint32_t r = 0; r < m_nranks; ++r) {
-            if (m_slots[r].stream == stream || seen_before(r)) continue;
-            HIP_CHECK(hipEventRecord(event(r), m_slots[r].stream));
-            HIP_CHECK(hipStreamWaitEvent(stream, event(r), 0));
+            if (m_slots[r].stream == stream) continue;
+            HIP_CHECK(hipStreamWaitEvent(stream, m_arrive[r], 0));
         }
         Status st = MEGRAY_OK;
         const uint32_t n = m_nranks;
@@ -197,19 +224,10 @@ private:
                 break;
         }
         if (st == MEGRAY_INVALID_ARGUMENT) MEGRAY_ERROR("collective rejected: %s", plan_error());
-        // ... and every other rank's stream behind the result
-        HIP_CHECK(hipEventRecord(event(m_nranks), stream));
-        for (uint32_t r = 0; r < m_nranks; ++r) {
-            if (m_slots[r].stream == stream || seen_before(r)) continue;
-            HIP_CHECK(hipStreamWaitEvent(m_slots[r].stream, event(m_nranks), 0));
-        }
+        // the other ranks order their streams behind this point themselves
+        if (!m_done) HIP_CHECK(hipEventCreateWithFlags(&m_done, hipEventDisableTiming));
+        HIP_CHECK(hipEventRecord(m_done, stream));
         return st;
-    }
-
-    bool seen_before(uint32_t r) const {
-        for (uint32_t q = 0; q < r; ++q)
-            if (m_slots[q].stream == m_slots[r].stream) return true;
-        return false;
     }
 
     // Enqueue the copy of a matched send / receive pair: on the receiver's stream, after the
@@ -220,7 +238,7 @@ private:
             return MEGRAY_INVALID_USAGE;
         }
         if (!s.size) return MEGRAY_OK;
-        const size_t base = m_nranks + 1;
+        const size_t base = 0;
         if (s.stream != r.stream) {
             HIP_CHECK(hipEventRecord(event(base), s.stream));
             HIP_CHECK(hipStreamWaitEvent(r.stream, event(base), 0));
@@ -238,9 +256,13 @@ private:
     std::condition_variable m_cv;
     std::vector<Call> m_slots;
     uint32_t m_arrived = 0;
-    uint64_t m_generation = 0;
+    std::atomic<uint64_t> m_generation{0};
+    static constexpr int kSpinPolls = 20000;
     Status m_result[2] = {MEGRAY_OK, MEGRAY_OK};
-    std::vector<hipEvent_t> m_events;  // [0, N): arrivals, N: collective done, N+1, N+2: p2p
+    hipStream_t m_lead_stream[2] = {nullptr, nullptr};
+    std::vector<hipEvent_t> m_arrive;  // per rank: "my buffers are ready", recorded by the rank itself
+    hipEvent_t m_done = nullptr;       // recorded by the leader behind the collective
+    std::vector<hipEvent_t> m_events;  // point-to-point transfers
     std::vector<Mailbox> m_mail;
 };
 
