@@ -183,3 +183,14 @@ def test_sum_special_values():
         assert np.isnan(got[2]) and np.isnan(want[2])
         keep = [0, 1, 3, 4, 5, 6]
         assert _bits(got[keep]) == _bits(want[keep])  # denormal kept, overflow -> inf, -0 + -0 = -0
+
+
+def test_oracle_selftest_under_sanitizers():
+    """The oracle itself, driven over ragged shapes under AddressSanitizer + UBSan (host only)."""
+    import os
+    import subprocess
+    here = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle")
+    subprocess.check_call(["make", "-s", "-C", here, "selftest_asan"])
+    proc = subprocess.run([os.path.join(here, "selftest_asan")], capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert "selftest ok" in proc.stdout
