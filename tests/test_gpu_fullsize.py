@@ -180,3 +180,28 @@ def test_small_message_sizes_are_exact():
         want = orc.ucx_all_reduce(host, orc.FLOAT32, orc.SUM)
         for r in range(8):
             assert np.array_equal(outs[r].cpu().numpy().view(np.uint32), want[r].view(np.uint32))
+
+
+def test_offsets_beyond_4_gib():
+    """A rank buffer larger than 4 GiB: every offset computation must be 64-bit."""
+    n = (1 << 32) + 4099
+    ins = [gen(n, torch.uint8, r) for r in range(2)]
+    outs = [torch.empty_like(t) for t in ins]
+    mr.all_reduce(ins, outs, n, mr.DType.UINT8, mr.ReduceOp.SUM)
+    torch.cuda.synchronize()
+    want = ins[0] + ins[1]  # torch wraps uint8
+    assert torch.equal(want, outs[0]) and torch.equal(want, outs[1])
+    # the copy path as well (general kernel, one source, two destinations)
+    for o in outs:
+        o.zero_()
+    mr.broadcast(ins[1], outs, n, mr.DType.UINT8, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(ins[1], outs[0]) and torch.equal(ins[1], outs[1])
+    # and a reduce_scatter whose second half starts beyond 4 GiB
+    half = n // 2
+    parts = [torch.empty(half, dtype=torch.uint8, device=DEV) for _ in range(2)]
+    mr.reduce_scatter(ins, parts, half, mr.DType.UINT8, mr.ReduceOp.MAX)
+    torch.cuda.synchronize()
+    for r in range(2):
+        sl = slice(r * half, (r + 1) * half)
+        assert torch.equal(torch.maximum(ins[0][sl], ins[1][sl]), parts[r])

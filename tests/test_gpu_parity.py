@@ -364,3 +364,30 @@ def test_planned_collectives_and_graph_replay():
         assert_same(to_host(d_out[2], np.int32), np.stack(ins).max(axis=0), "graph replay on new data")
     with pytest.raises(mr.MegRayError, match="unknown reduce op"):
         mr.CollectivePlan(mr.Collective.ALL_REDUCE, d_in, d_out, 5000, mr.DType.INT32, 9)
+
+
+def test_sixteen_ranks_many_segments():
+    """16 ranks with ragged, unaligned pieces: more runs than one launch descriptor holds, so the
+    planner splits the collective over several launches."""
+    rng = np.random.default_rng(16)
+    nranks, recvlen = 16, 1031
+    for dtype in (orc.FLOAT32, orc.INT8):
+        size = orc.dtype_size(dtype)
+        ins = [rand_array(dtype, nranks * recvlen, rng) for _ in range(nranks)]
+        for order in ORDERS:
+            want = orc.fold_reduce_scatter(ins, dtype, orc.SUM, order)
+            d_in = [to_device(x, size * (r % 3)) for r, x in enumerate(ins)]
+            d_out = [empty_device(recvlen * size, size * (r % 2)) for r in range(nranks)]
+            runs, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, d_in, d_out, recvlen, dtype, order)
+            mr.reduce_scatter(d_in, d_out, recvlen, dtype, orc.SUM, order)
+            torch.cuda.synchronize()
+            for r in range(nranks):
+                assert_same(to_host(d_out[r], ins[0].dtype), want[r], f"N=16 reduce_scatter dtype={dtype} order={order}")
+            if order == orc.ORDER_SHM:
+                assert len({run["step"] for run in runs}) == 1 or len(runs) > 96
+            want = orc.fold_all_reduce(ins, dtype, orc.MAX, order)
+            d_out = [empty_device(nranks * recvlen * size, size * (r % 2)) for r in range(nranks)]
+            mr.all_reduce(d_in, d_out, nranks * recvlen, dtype, orc.MAX, order)
+            torch.cuda.synchronize()
+            for r in (0, 7, 15):
+                assert_same(to_host(d_out[r], ins[0].dtype), want[r], f"N=16 all_reduce dtype={dtype} order={order}")
