@@ -23,10 +23,6 @@ Status invalid(const char* what) {
     return MEGRAY_INVALID_ARGUMENT;
 }
 
-bool aligned16(const void* p) {
-    return (reinterpret_cast<uintptr_t>(p) & (kVecBytes - 1)) == 0;
-}
-
 bool overlaps(const void* a, uint64_t a_bytes, const void* b, uint64_t b_bytes) {
     if (!a || !b || !a_bytes || !b_bytes) return false;
     const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
@@ -43,12 +39,25 @@ public:
                 uint32_t nout, uint32_t elem_size, bool new_wins)
             : m_plan(plan), m_nranks(nranks), m_nfold(nfold), m_nout(nout), m_elem(elem_size),
               m_new_wins(new_wins) {
+        // Vector access needs every buffer at the same offset from a 16-byte boundary (usually 0;
+        // a common non-zero offset, in whole elements, only lengthens the scalar head of each run).
         m_aligned = true;
+        m_misalign = 0;
+        bool first = true;
         for (uint32_t r = 0; r < kMaxRanks; ++r) {
             m_in[r] = r < nranks ? in[r] : nullptr;
             m_out[r] = r < nranks ? out[r] : nullptr;
-            m_aligned = m_aligned && aligned16(m_in[r]) && aligned16(m_out[r]);  // null counts as aligned
+            for (const void* p : {m_in[r], static_cast<const void*>(m_out[r])}) {
+                if (!p) continue;  // unused slot
+                const uint32_t mis = uint32_t(reinterpret_cast<uintptr_t>(p) & (kVecBytes - 1));
+                if (first) {
+                    m_misalign = mis;
+                    first = false;
+                }
+                m_aligned = m_aligned && mis == m_misalign;
+            }
         }
+        if (m_misalign % elem_size) m_aligned = false;
     }
 
     void add_run(uint64_t in_begin, uint64_t out_begin, uint64_t count, uint8_t start, int8_t dir,
@@ -86,7 +95,7 @@ private:
     static bool flat_width(uint32_t n) { return n == 2 || n == 3 || n == 4 || n == 8; }
 
     bool emit_flat() {
-        if (!m_aligned || m_nfold != m_nranks || !flat_width(m_nranks) || m_runs.size() > kMaxFlatRuns)
+        if (!m_aligned || m_misalign || m_nfold != m_nranks || !flat_width(m_nranks) || m_runs.size() > kMaxFlatRuns)
             return false;
         const uint64_t epv = kVecBytes / m_elem;
         const uint64_t tile = uint64_t(kThreads) * epv;  // elements per tile
@@ -134,11 +143,12 @@ private:
     void emit_general() {
         open_launch();
         const uint64_t epv = kVecBytes / m_elem;
+        const uint64_t shift = m_misalign / m_elem;  // elements between a 16-byte boundary and each base
         for (const Run& r : m_runs) {
             const bool vector = m_aligned && (r.in_begin % epv == r.out_begin % epv);
             uint64_t head = 0, body = 0;
             if (vector) {
-                head = std::min<uint64_t>((epv - r.in_begin % epv) % epv, r.count);
+                head = std::min<uint64_t>((epv - (r.in_begin + shift) % epv) % epv, r.count);
                 body = (r.count - head) / epv * epv;
             }
             if (!body) {
@@ -210,6 +220,7 @@ private:
     uint32_t m_nranks, m_nfold, m_nout, m_elem;
     bool m_new_wins;
     bool m_aligned;
+    uint32_t m_misalign = 0;
     bool m_tree = false;
     std::vector<Run> m_runs;
     FoldLaunch m_launch;

@@ -94,6 +94,10 @@ def test_all_reduce_in_place_and_misaligned():
                 got = run_all_reduce(ins, dtype, orc.SUM, orc.ORDER_UCX, sched, offsets=offs)
                 for r in range(nranks):
                     assert_same(got[r], want[r], f"misaligned dtype={dtype} sched={sched}")
+                # all buffers off by the same element count: vector body behind a longer scalar head
+                got = run_all_reduce(ins, dtype, orc.SUM, orc.ORDER_UCX, sched, offsets=[size * 3] * nranks)
+                for r in range(nranks):
+                    assert_same(got[r], want[r], f"common offset dtype={dtype} sched={sched}")
 
 
 def test_float_special_values_and_tie_conventions():
