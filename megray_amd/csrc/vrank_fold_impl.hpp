@@ -254,11 +254,15 @@ __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
     const uint32_t tid = threadIdx.x;
 
     if (vector) {
+        // A tile is kVecIters groups of kThreads * U vectors, taken one after the other: the segment
+        // lookup above is paid once per tile while the registers of one group suffice.
         const uint64_t nvec = count / EPV;
-        const uint64_t vbase = uint64_t(local_tile) * (kThreads * U);
+        for (uint32_t it = 0; it < kVecIters; ++it) {
+        const uint64_t vbase = (uint64_t(local_tile) * kVecIters + it) * (kThreads * U);
+        if (vbase >= nvec) break;
         const uint64_t in_off = in_begin * sizeof(T) + vbase * kVecBytes;
         const uint64_t out_off = out_begin * sizeof(T) + vbase * kVecBytes;
-        const uint64_t left = nvec - vbase;  // vectors from this tile's start to the segment's end
+        const uint64_t left = nvec - vbase;  // vectors from this group's start to the segment's end
         AccFor<T, OP> acc[U];
         if (left >= uint64_t(kThreads) * U) {
             // full tile: no predicates
@@ -332,28 +336,54 @@ __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
                 }
             }
         }
+        }  // groups of the tile
     } else {
-        // element tiles: chunk heads / tails and buffers that are not 16-byte aligned
-        const uint64_t ebase = uint64_t(local_tile) * (kThreads * U);
-        const uint64_t left = count - ebase;
+        // element tiles: run heads / tails and buffers that are not 16-byte aligned.  A lane takes
+        // kElemsPerLane elements, a wavefront's lanes consecutive ones, four at a time in flight.
+        constexpr uint32_t G = 4;
+        const uint64_t ebase = uint64_t(local_tile) * (kThreads * kElemsPerLane);
+        for (uint32_t g = 0; g < kElemsPerLane; g += G) {
+            const uint64_t gbase = ebase + uint64_t(g) * kThreads;
+            if (gbase >= count) break;
+            const uint64_t left = count - gbase;
+            const uint64_t ie = in_begin + gbase + tid;
+            const uint64_t oe = out_begin + gbase + tid;
+            if (left >= uint64_t(G) * kThreads) {
+                A a[G];
+                const T* seed = static_cast<const T*>(L.in[start]) + ie;
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const uint32_t e = u * kThreads + tid;
-            if (e < left) {
-                const uint64_t ie = in_begin + ebase + e;
-                const uint64_t oe = out_begin + ebase + e;
-                A a = static_cast<A>(static_cast<const T*>(L.in[start])[ie]);
-                for (uint32_t j = 1; j < nfold; ++j)
-                    a = combine<OP, A>(
-                            a, static_cast<A>(static_cast<const T*>(L.in[rotate_rank(start, dir, j, nr)])[ie]),
-                            new_wins);
-                const T r = static_cast<T>(a);
-                for (uint32_t m = 0; m < nout; ++m) static_cast<T*>(L.out[rotate_rank(out_first, 1, m, nr)])[oe] = r;
+                for (uint32_t q = 0; q < G; ++q) a[q] = static_cast<A>(seed[q * kThreads]);
+                for (uint32_t j = 1; j < nfold; ++j) {
+                    const T* src = static_cast<const T*>(L.in[rotate_rank(start, dir, j, nr)]) + ie;
+                    T x[G];
+#pragma unroll
+                    for (uint32_t q = 0; q < G; ++q) x[q] = src[q * kThreads];
+#pragma unroll
+                    for (uint32_t q = 0; q < G; ++q) a[q] = combine<OP, A>(a[q], static_cast<A>(x[q]), new_wins);
+                }
+                for (uint32_t m = 0; m < nout; ++m) {
+                    T* dst = static_cast<T*>(L.out[rotate_rank(out_first, 1, m, nr)]) + oe;
+#pragma unroll
+                    for (uint32_t q = 0; q < G; ++q) dst[q * kThreads] = static_cast<T>(a[q]);
+                }
+            } else {
+                for (uint32_t q = 0; q < G; ++q) {
+                    const uint32_t e = q * kThreads + tid;
+                    if (e >= left) break;
+                    A a = static_cast<A>(static_cast<const T*>(L.in[start])[ie + q * kThreads]);
+                    for (uint32_t j = 1; j < nfold; ++j)
+                        a = combine<OP, A>(
+                                a,
+                                static_cast<A>(static_cast<const T*>(L.in[rotate_rank(start, dir, j, nr)])[ie + q * kThreads]),
+                                new_wins);
+                    const T r = static_cast<T>(a);
+                    for (uint32_t m = 0; m < nout; ++m)
+                        static_cast<T*>(L.out[rotate_rank(out_first, 1, m, nr)])[oe + q * kThreads] = r;
+                }
             }
         }
     }
 }
-
 
 // ---------------------------------------------------------------------------------------------
 // Flat fold: tile t covers bytes [1024 t, 1024 t + 1024) of every input, whatever run it is in.

@@ -39,24 +39,29 @@ public:
                 uint32_t nout, uint32_t elem_size, bool new_wins)
             : m_plan(plan), m_nranks(nranks), m_nfold(nfold), m_nout(nout), m_elem(elem_size),
               m_new_wins(new_wins) {
-        // Vector access needs every buffer at the same offset from a 16-byte boundary (usually 0;
-        // a common non-zero offset, in whole elements, only lengthens the scalar head of each run).
-        m_aligned = true;
-        m_misalign = 0;
+        // Vector access needs every buffer at the same offset from a 16-byte boundary (usually 0; a
+        // common non-zero offset, in whole elements, only lengthens the scalar head of each run).
+        // m_grid is the largest power of two up to one tile (1 KiB) modulo which all buffers still
+        // agree: vector bodies start on that grid so that neighbouring wavefronts do not share
+        // cache lines.
+        uintptr_t differ = 0, first_ptr = 0;
         bool first = true;
         for (uint32_t r = 0; r < kMaxRanks; ++r) {
             m_in[r] = r < nranks ? in[r] : nullptr;
             m_out[r] = r < nranks ? out[r] : nullptr;
             for (const void* p : {m_in[r], static_cast<const void*>(m_out[r])}) {
                 if (!p) continue;  // unused slot
-                const uint32_t mis = uint32_t(reinterpret_cast<uintptr_t>(p) & (kVecBytes - 1));
                 if (first) {
-                    m_misalign = mis;
+                    first_ptr = reinterpret_cast<uintptr_t>(p);
                     first = false;
                 }
-                m_aligned = m_aligned && mis == m_misalign;
+                differ |= first_ptr ^ reinterpret_cast<uintptr_t>(p);
             }
         }
+        m_grid = kThreads * kVecBytes;
+        while (m_grid > 1 && (differ & (m_grid - 1))) m_grid >>= 1;
+        m_aligned = m_grid >= kVecBytes;
+        m_misalign = uint32_t(first_ptr & (m_grid - 1));  // offset of every base from the grid
         if (m_misalign % elem_size) m_aligned = false;
     }
 
@@ -95,7 +100,7 @@ private:
     static bool flat_width(uint32_t n) { return n == 2 || n == 3 || n == 4 || n == 8; }
 
     bool emit_flat() {
-        if (!m_aligned || m_misalign || m_nfold != m_nranks || !flat_width(m_nranks) || m_runs.size() > kMaxFlatRuns)
+        if (!m_aligned || (m_misalign & (kVecBytes - 1)) || m_nfold != m_nranks || !flat_width(m_nranks) || m_runs.size() > kMaxFlatRuns)
             return false;
         const uint64_t epv = kVecBytes / m_elem;
         const uint64_t tile = uint64_t(kThreads) * epv;  // elements per tile
@@ -143,12 +148,16 @@ private:
     void emit_general() {
         open_launch();
         const uint64_t epv = kVecBytes / m_elem;
-        const uint64_t shift = m_misalign / m_elem;  // elements between a 16-byte boundary and each base
         for (const Run& r : m_runs) {
             const bool vector = m_aligned && (r.in_begin % epv == r.out_begin % epv);
             uint64_t head = 0, body = 0;
             if (vector) {
-                head = std::min<uint64_t>((epv - (r.in_begin + shift) % epv) % epv, r.count);
+                // the body starts where inputs and outputs both sit on the coarsest grid they share
+                uint64_t grid = m_grid;
+                const uint64_t skew = (r.in_begin - r.out_begin) * m_elem;  // unsigned wrap is fine mod 2^k
+                while (grid > kVecBytes && (skew & (grid - 1))) grid >>= 1;
+                const uint64_t at = (m_misalign + r.in_begin * m_elem) & (grid - 1);
+                head = std::min<uint64_t>(((grid - at) & (grid - 1)) / m_elem, r.count);
                 body = (r.count - head) / epv * epv;
             }
             if (!body) {
@@ -221,6 +230,7 @@ private:
     bool m_new_wins;
     bool m_aligned;
     uint32_t m_misalign = 0;
+    uint64_t m_grid = kVecBytes;
     bool m_tree = false;
     std::vector<Run> m_runs;
     FoldLaunch m_launch;

@@ -125,9 +125,14 @@ constexpr uint32_t pack_unroll() {
     return 1u;
 }
 
+// Elements each lane handles in an element-wise tile (unaligned buffers, run heads and tails), and
+// vector groups a lane walks through, one after the other, in a vector tile of the general kernel.
+constexpr uint32_t kElemsPerLane = 16;
+constexpr uint32_t kVecIters = 4;
+
 inline uint64_t tile_elems(const FoldLaunch& L, bool vector) {
-    uint64_t per_lane = vector ? (kVecBytes / L.elem_size) : 1;
-    return uint64_t(kThreads) * L.unroll * per_lane;
+    uint64_t per_lane = vector ? uint64_t(L.unroll) * kVecIters * (kVecBytes / L.elem_size) : kElemsPerLane;
+    return uint64_t(kThreads) * per_lane;
 }
 
 }  // namespace vrank

@@ -99,13 +99,13 @@ def bits_equal(a, b):
 def test_all_reduce_plans_reproduce_the_replays(dtype, nranks):
     rng = np.random.default_rng(dtype * 100 + nranks)
     size = orc.dtype_size(dtype)
-    for length in (0, 1, nranks - 1, 3 * nranks + 1, 300, 4099):
+    for length in (0, 1, nranks - 1, 3 * nranks + 1, 300, 4099, 20011):
         ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
         for misalign in (0, 1, 2):
             # 1: every rank off by a different element count; 2: all buffers off by the same count
             offs = {0: [0] * nranks, 1: [size * (r % 3) for r in range(nranks)], 2: [size] * nranks}[misalign]
             sp, rp = fake_ptrs(SEND_BASE, nranks, offs), fake_ptrs(RECV_BASE, nranks, offs)
-            if misalign == 2 and size < 16 and length >= 64:
+            if misalign == 2 and length * size >= 2048 * nranks:  # every chunk outgrows its scalar head
                 runs, _, _ = mr.describe(mr.Collective.ALL_REDUCE, sp, rp, length, dtype)
                 assert any(r["vector"] == 1 for r in runs), "a common offset must keep the vector path"
             for op in (orc.SUM, orc.MAX, orc.MIN):
