@@ -23,7 +23,6 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-BASE_SEED = 0x4D656752  # "MegR"; rank r draws from seed BASE_SEED + r
 
 # HBM bytes per launch of the fold kernel on the headline workload, from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE runs scaled by the same counters on a plain copy of known size; the
@@ -52,14 +51,9 @@ def parse_args():
 
 
 def make_inputs(torch, nranks, n):
-    ins = []
-    for r in range(nranks):
-        g = torch.Generator(device="cuda:0")
-        g.manual_seed(BASE_SEED + r)
-        t = torch.rand(n, generator=g, device="cuda:0", dtype=torch.float32)
-        t.mul_(2.0).sub_(1.0)  # uniform[-1, 1)
-        ins.append(t)
-    return ins
+    """uniform[-1, 1) fp32 from the counter-based generator: element i of rank r depends only on (seed, r, i)."""
+    from megray_amd import synth
+    return [synth.fill_torch(torch.float32, n, r) for r in range(nranks)]
 
 
 def check_small(torch, mr, orc, np):
@@ -69,7 +63,8 @@ def check_small(torch, mr, orc, np):
     outs = [torch.empty_like(t) for t in ins]
     mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream=torch.cuda.current_stream())
     torch.cuda.synchronize()
-    host = [t.cpu().numpy() for t in ins]
+    from megray_amd import synth
+    host = [synth.fill_np(np.float32, n, r) for r in range(nranks)]  # regenerated, not copied back
     want = orc.ucx_all_reduce(host, orc.FLOAT32, orc.SUM)
     for r in range(nranks):
         got = outs[r].cpu().numpy()
@@ -101,7 +96,7 @@ def small_message_sweep(torch, mr):
     """
     out = {}
     st = torch.cuda.current_stream()
-    for nbytes in (4096, 16384, 65536, 262144, 1048576):
+    for nbytes in (4096, 4096, 16384, 65536, 262144, 1048576):  # the first pass only warms the path up
         n = nbytes // 4
         ins = make_inputs(torch, 8, n)
         outs = [torch.empty_like(t) for t in ins]
@@ -123,7 +118,7 @@ def small_message_sweep(torch, mr):
         stream_us = timed(lambda: plan.launch(raw), 2000)
         unplanned_us = timed(lambda: mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream=raw), 1000)
         lat = []
-        for _ in range(500):
+        for _ in range(1000):
             t0 = time.perf_counter()
             plan.launch(raw)
             torch.cuda.synchronize()
@@ -165,9 +160,9 @@ def cpu_baseline(orc, np, nranks):
     """The reference tests' expected-value loop on the host: single thread (as the reference runs
     it) on a 2^25-element-per-rank sample of the headline workload, plus the same loop split over
     all host cores for scale."""
+    from megray_amd import synth
     n = 1 << 25
-    rng = np.random.default_rng(BASE_SEED)
-    ins = [rng.random(n, dtype=np.float32) * 2 - 1 for _ in range(nranks)]
+    ins = [synth.fill_np(np.float32, n, r) for r in range(nranks)]  # the first 2^25 elements of the GPU's buffers
     bmin = 2 * nranks * n * 4
 
     def timed(threads, reps):
@@ -183,11 +178,21 @@ def cpu_baseline(orc, np, nranks):
     t1 = timed(0, 5)
     cores = min(os.cpu_count() or 1, 16)
     tn = timed(cores, 5)
+    # the reference's own schedule on the host: 2(N-1) ring steps of the two-input reduce loop
+    # (src/ucx/all_reduce.cpp:53-101 over src/ucx/kernel.cu:16-22), single thread, 2^24 elements per rank
+    m = 1 << 24
+    part = [a[:m] for a in ins]
+    orc.ucx_all_reduce(part, orc.FLOAT32, orc.SUM)
+    t0 = time.perf_counter()
+    orc.ucx_all_reduce(part, orc.FLOAT32, orc.SUM)
+    tr = time.perf_counter() - t0
     return {
         "value": round(bmin / t1 / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
         "sample": f"all_reduce SUM fp32, {nranks} ranks x 2^25 elements, test/test_opr.cpp:321-330 loop, "
                   f"median of 5, {t1 * 1e3:.1f} ms per pass",
         "all_cores": {"value": round(bmin / tn / 1e9, 3), "cores": cores, "ms": round(tn * 1e3, 1)},
+        "ring_replay": {"value": round(2 * nranks * m * 4 / tr / 1e9, 3), "cores": 1, "ms": round(tr * 1e3, 1),
+                        "sample": f"literal 2(N-1)-step ring replay, {nranks} ranks x 2^24 elements, B_min / t"},
     }
 
 
@@ -198,13 +203,9 @@ def run_other_workload(args, torch, mr):
     n8 = 8
     w = args.workload
 
-    def rnd(n, dtype, seed):
-        g = torch.Generator(device=dev)
-        g.manual_seed(BASE_SEED + seed)
-        if dtype.is_floating_point:
-            return (torch.randn(n, generator=g, device=dev, dtype=torch.float32) * 0.01).to(dtype)
-        info = torch.iinfo(dtype)
-        return torch.randint(info.min, info.max, (n,), generator=g, device=dev, dtype=dtype)
+    def rnd(n, dtype, rank):
+        from megray_amd import synth
+        return synth.fill_torch(dtype, n, rank, "normal" if dtype.is_floating_point else "uniform", device=dev)
 
     if w == "copy":
         n = 1 << 30
@@ -352,7 +353,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
-        "data": "synthetic: uniform[-1,1) fp32, torch generator seeded 0x4D656752 + rank",
+        "data": "synthetic: uniform[-1,1) fp32, counter-based splitmix64 of (0x4D656752 + rank) xor golden*index",
         "config": {
             "workload": f"all_reduce SUM fp32, {nranks} virtual ranks x 2^{args.log2n} elements, ucx ring order, "
                         f"{args.schedule} schedule, buffers resident in HBM",
@@ -371,6 +372,9 @@ def main():
     }
     del ins, outs
     torch.cuda.empty_cache()
+    props = torch.cuda.get_device_properties(0)
+    result["device"] = {"name": props.name, "compute_units": props.multi_processor_count,
+                        "hbm_gib": round(props.total_memory / 2 ** 30, 1)}
     result["copy_yardstick"] = copy_yardstick(torch, mr)
     if not args.no_small:
         result["small_msg_us"] = small_message_sweep(torch, mr)

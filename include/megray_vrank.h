@@ -165,7 +165,7 @@ typedef struct mrv_plan_run {
     uint32_t out_first;     /* fold: first destination rank; pack: destination rank */
     uint32_t tiles;         /* workgroups this run occupies (flat: those wholly inside it) */
     uint32_t reads_recv;    /* 1 = the launch reads the receive buffers (a later step of a multi-launch plan) */
-    uint32_t reserved;
+    uint32_t waves;         /* wavefronts per workgroup of the launch (4: the group form, four tiles per workgroup) */
     uint64_t in_begin;      /* fold: first element in the inputs; pack: source byte offset */
     uint64_t out_begin;     /* fold: first element in the outputs; pack: destination byte offset */
     uint64_t count;         /* fold: elements; pack: bytes */

@@ -16,7 +16,7 @@ class PlanRun(ctypes.Structure):
         ("step", ctypes.c_uint32), ("kind", ctypes.c_uint32), ("nfold", ctypes.c_uint32),
         ("nout", ctypes.c_uint32), ("new_wins_ties", ctypes.c_uint32), ("vector", ctypes.c_uint32),
         ("start", ctypes.c_uint32), ("dir", ctypes.c_int32), ("out_first", ctypes.c_uint32),
-        ("tiles", ctypes.c_uint32), ("reads_recv", ctypes.c_uint32), ("reserved", ctypes.c_uint32),
+        ("tiles", ctypes.c_uint32), ("reads_recv", ctypes.c_uint32), ("waves", ctypes.c_uint32),
         ("in_begin", ctypes.c_uint64), ("out_begin", ctypes.c_uint64),
         ("count", ctypes.c_uint64),
     ]

@@ -292,7 +292,7 @@ int mrv_plan_create(int collective, const void* const* sendbuffs, void* const* r
                 std::memset(&params, 0, sizeof(params));
                 params.func = const_cast<void*>(call.kernel);
                 params.gridDim = dim3(call.grid);
-                params.blockDim = dim3(kThreads);
+                params.blockDim = dim3(call.block);
                 params.kernelParams = args;
                 hipGraphNode_t node = nullptr;
                 HIP_CHECK(hipGraphAddKernelNode(&node, p->graph, prev ? &prev : nullptr, prev ? 1 : 0, &params));
@@ -313,7 +313,7 @@ int mrv_plan_launch(const mrv_plan* plan, void* stream) {
             return MEGRAY_OK;
         }
         for (const KernelCall& call : plan->calls)
-            HIP_CHECK(enqueue(call.kernel, call.grid, call.launch, as_stream(stream)));
+            HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, as_stream(stream)));
         return MEGRAY_OK;
     });
 }
@@ -358,6 +358,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.nout = L.nout;
                     run.new_wins_ties = L.new_wins_ties;
                     run.vector = (sg.flags & kSegVector) ? 1 : 0;
+                    run.waves = 1;
                     run.start = sg.start;
                     run.dir = sg.dir;
                     run.out_first = sg.out_first;
@@ -384,6 +385,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.nout = L.nout;
                     run.new_wins_ties = L.new_wins_ties;
                     run.vector = 2;
+                    run.waves = L.waves;
                     run.start = fr.start;
                     run.dir = L.tree ? 0 : fr.dir;
                     run.out_first = fr.out_first;
@@ -404,6 +406,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                 run.step = uint32_t(i);
                 run.nfold = L.nranks;
                 run.nout = 1;
+                run.waves = 1;
                 run.start = L.root;
                 run.dir = 0;
                 run.out_first = L.root;
@@ -420,6 +423,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.nfold = 1;
                     run.nout = 1;
                     run.vector = L.width;
+                    run.waves = 1;
                     run.dir = 1;
                     run.tiles = L.tiles_per_copy;
                     run.count = L.block_bytes;

@@ -34,19 +34,24 @@ Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCal
     calls.clear();
     calls.reserve(plan.steps.size());
     for (const Step& step : plan.steps) {
-        KernelCall call{nullptr, 0, nullptr};
+        KernelCall call{nullptr, 0, kThreads, nullptr};
         switch (step.kind) {
             case Step::kFold:
-                call = {fold_kernel_for(step.fold, dtype, op), step.fold.total_tiles, &step.fold};
+                call = {fold_kernel_for(step.fold, dtype, op), step.fold.total_tiles, kThreads, &step.fold};
                 break;
             case Step::kFlat:
-                call = {flat_kernel_for(step.flat, dtype, op), step.flat.total_tiles, &step.flat};
+                if (step.flat.waves == kGroupWaves)
+                    call = {flat_kernel_for(step.flat, dtype, op), group_grid(step.flat.total_tiles),
+                            kThreads * kGroupWaves, &step.flat};
+                else
+                    call = {flat_kernel_for(step.flat, dtype, op), step.flat.total_tiles, kThreads, &step.flat};
                 break;
             case Step::kTree:
-                call = {tree_kernel_for(step.tree, dtype, op), step.tree.total_tiles, &step.tree};
+                call = {tree_kernel_for(step.tree, dtype, op), step.tree.total_tiles, kThreads, &step.tree};
                 break;
             case Step::kPack:
-                call = {pack_kernel_for(step.pack), step.pack.ncopies * step.pack.tiles_per_copy, &step.pack};
+                call = {pack_kernel_for(step.pack), step.pack.ncopies * step.pack.tiles_per_copy, kThreads,
+                        &step.pack};
                 break;
         }
         if (!call.kernel) {
@@ -59,23 +64,10 @@ Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCal
 }
 
 Status execute(const Plan& plan, DType dtype, ReduceOp op, hipStream_t stream) {
-    for (const Step& step : plan.steps) {
-        switch (step.kind) {
-            case Step::kFold:
-                HIP_CHECK(enqueue(fold_kernel_for(step.fold, dtype, op), step.fold.total_tiles, &step.fold, stream));
-                break;
-            case Step::kFlat:
-                HIP_CHECK(enqueue(flat_kernel_for(step.flat, dtype, op), step.flat.total_tiles, &step.flat, stream));
-                break;
-            case Step::kTree:
-                HIP_CHECK(enqueue(tree_kernel_for(step.tree, dtype, op), step.tree.total_tiles, &step.tree, stream));
-                break;
-            case Step::kPack:
-                HIP_CHECK(enqueue(pack_kernel_for(step.pack), step.pack.ncopies * step.pack.tiles_per_copy,
-                                  &step.pack, stream));
-                break;
-        }
-    }
+    std::vector<KernelCall> calls;
+    const Status st = resolve(plan, dtype, op, calls);
+    if (st != MEGRAY_OK) return st;
+    for (const KernelCall& call : calls) HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, stream));
     return MEGRAY_OK;
 }
 

@@ -27,6 +27,7 @@ void check_reduce_op(ReduceOp op);
 struct KernelCall {
     const void* kernel;
     uint32_t grid;
+    uint32_t block;  // threads per workgroup
     const void* launch;
 };
 

@@ -258,85 +258,85 @@ __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
         // lookup above is paid once per tile while the registers of one group suffice.
         const uint64_t nvec = count / EPV;
         for (uint32_t it = 0; it < kVecIters; ++it) {
-        const uint64_t vbase = (uint64_t(local_tile) * kVecIters + it) * (kThreads * U);
-        if (vbase >= nvec) break;
-        const uint64_t in_off = in_begin * sizeof(T) + vbase * kVecBytes;
-        const uint64_t out_off = out_begin * sizeof(T) + vbase * kVecBytes;
-        const uint64_t left = nvec - vbase;  // vectors from this group's start to the segment's end
-        AccFor<T, OP> acc[U];
-        if (left >= uint64_t(kThreads) * U) {
-            // full tile: no predicates
-            if constexpr (K > 0) {
-                u32x4 x[K][U];
+            const uint64_t vbase = (uint64_t(local_tile) * kVecIters + it) * (kThreads * U);
+            if (vbase >= nvec) break;
+            const uint64_t in_off = in_begin * sizeof(T) + vbase * kVecBytes;
+            const uint64_t out_off = out_begin * sizeof(T) + vbase * kVecBytes;
+            const uint64_t left = nvec - vbase;  // vectors from this group's start to the segment's end
+            AccFor<T, OP> acc[U];
+            if (left >= uint64_t(kThreads) * U) {
+                // full tile: no predicates
+                if constexpr (K > 0) {
+                    u32x4 x[K][U];
 #pragma unroll
-                for (int j = 0; j < K; ++j) {
-                    const char* src = static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off;
+                    for (int j = 0; j < K; ++j) {
+                        const char* src = static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off;
 #pragma unroll
-                    for (int u = 0; u < U; ++u) x[j][u] = load_tile_vec(src + u * (kThreads * kVecBytes), tid);
-                }
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    acc[u].seed(x[0][u]);
-#pragma unroll
-                    for (int j = 1; j < K; ++j) acc[u].fold(x[j][u], new_wins);
-                }
-            } else {
-                {
-                    const char* src = static_cast<const char*>(L.in[start]) + in_off;
-#pragma unroll
-                    for (int u = 0; u < U; ++u) acc[u].seed(load_tile_vec(src + u * (kThreads * kVecBytes), tid));
-                }
-                uint32_t j = 1;
-                for (; j + 4 <= nfold; j += 4) {
-                    u32x4 x[4][U];
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const char* src =
-                                static_cast<const char*>(L.in[rotate_rank(start, dir, j + q, nr)]) + in_off;
-#pragma unroll
-                        for (int u = 0; u < U; ++u) x[q][u] = load_tile_vec(src + u * (kThreads * kVecBytes), tid);
+                        for (int u = 0; u < U; ++u) x[j][u] = load_tile_vec(src + u * (kThreads * kVecBytes), tid);
                     }
 #pragma unroll
-                    for (int q = 0; q < 4; ++q)
+                    for (int u = 0; u < U; ++u) {
+                        acc[u].seed(x[0][u]);
 #pragma unroll
-                        for (int u = 0; u < U; ++u) acc[u].fold(x[q][u], new_wins);
+                        for (int j = 1; j < K; ++j) acc[u].fold(x[j][u], new_wins);
+                    }
+                } else {
+                    {
+                        const char* src = static_cast<const char*>(L.in[start]) + in_off;
+#pragma unroll
+                        for (int u = 0; u < U; ++u) acc[u].seed(load_tile_vec(src + u * (kThreads * kVecBytes), tid));
+                    }
+                    uint32_t j = 1;
+                    for (; j + 4 <= nfold; j += 4) {
+                        u32x4 x[4][U];
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const char* src =
+                                    static_cast<const char*>(L.in[rotate_rank(start, dir, j + q, nr)]) + in_off;
+#pragma unroll
+                            for (int u = 0; u < U; ++u) x[q][u] = load_tile_vec(src + u * (kThreads * kVecBytes), tid);
+                        }
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+#pragma unroll
+                            for (int u = 0; u < U; ++u) acc[u].fold(x[q][u], new_wins);
+                    }
+                    for (; j < nfold; ++j) {
+                        const char* src = static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off;
+#pragma unroll
+                        for (int u = 0; u < U; ++u)
+                            acc[u].fold(load_tile_vec(src + u * (kThreads * kVecBytes), tid), new_wins);
+                    }
                 }
-                for (; j < nfold; ++j) {
-                    const char* src = static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off;
+                u32x4 res[U];
 #pragma unroll
-                    for (int u = 0; u < U; ++u)
-                        acc[u].fold(load_tile_vec(src + u * (kThreads * kVecBytes), tid), new_wins);
+                for (int u = 0; u < U; ++u) res[u] = acc[u].finish();
+                for (uint32_t m = 0; m < nout; ++m) {
+                    char* dst = static_cast<char*>(L.out[rotate_rank(out_first, 1, m, nr)]) + out_off;
+#pragma unroll
+                    for (int u = 0; u < U; ++u) store_tile_vec(dst + u * (kThreads * kVecBytes), tid, res[u]);
                 }
-            }
-            u32x4 res[U];
+            } else {
+                // last tile of the segment: predicate every vector
 #pragma unroll
-            for (int u = 0; u < U; ++u) res[u] = acc[u].finish();
-            for (uint32_t m = 0; m < nout; ++m) {
-                char* dst = static_cast<char*>(L.out[rotate_rank(out_first, 1, m, nr)]) + out_off;
-#pragma unroll
-                for (int u = 0; u < U; ++u) store_tile_vec(dst + u * (kThreads * kVecBytes), tid, res[u]);
-            }
-        } else {
-            // last tile of the segment: predicate every vector
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const uint32_t v = u * kThreads + tid;
-                if (v < left) {
-                    AccFor<T, OP> a;
-                    a.seed(load_vec(static_cast<const char*>(L.in[start]) + in_off + v * kVecBytes));
-                    for (uint32_t j = 1; j < nfold; ++j)
-                        a.fold(load_vec(static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off +
-                                        v * kVecBytes),
-                               new_wins);
-                    const u32x4 r = a.finish();
-                    for (uint32_t m = 0; m < nout; ++m)
-                        store_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, nr)]) + out_off +
-                                          v * kVecBytes,
-                                  r);
+                for (int u = 0; u < U; ++u) {
+                    const uint32_t v = u * kThreads + tid;
+                    if (v < left) {
+                        AccFor<T, OP> a;
+                        a.seed(load_vec(static_cast<const char*>(L.in[start]) + in_off + v * kVecBytes));
+                        for (uint32_t j = 1; j < nfold; ++j)
+                            a.fold(load_vec(static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off +
+                                            v * kVecBytes),
+                                   new_wins);
+                        const u32x4 r = a.finish();
+                        for (uint32_t m = 0; m < nout; ++m)
+                            store_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, nr)]) + out_off +
+                                              v * kVecBytes,
+                                      r);
+                    }
                 }
             }
         }
-        }  // groups of the tile
     } else {
         // element tiles: run heads / tails and buffers that are not 16-byte aligned.  A lane takes
         // kElemsPerLane elements, a wavefront's lanes consecutive ones, four at a time in flight.
@@ -463,11 +463,49 @@ __global__ void __launch_bounds__(kThreads) fold_tree_kernel(const TreeLaunch L)
     if (el < L.count) static_cast<T*>(L.out)[el] = tree_element<T, OP, 0>(L, L.nranks, L.root, el);
 }
 
+// One tile of a flat launch element by element: a tile that straddles a run border or the end of
+// the buffers.  One run at a time, so that ranks and destinations stay uniform.
+template <typename T, int OP, int K, bool TREE>
+__device__ __forceinline__ void flat_tile_by_element(const FlatLaunch& L, uint32_t tile, uint32_t tid) {
+    using A = typename Wide<T>::type;
+    constexpr uint32_t EPV = kVecBytes / sizeof(T);
+    constexpr uint32_t TILE = kThreads * EPV;
+    const bool new_wins = L.new_wins_ties != 0;
+    const uint32_t nout = L.nout;
+    const uint64_t e_lo = uint64_t(tile) * TILE;
+    const uint64_t e_hi = e_lo + TILE < L.count ? e_lo + TILE : L.count;
+    for (uint32_t i = 0; i < L.nruns; ++i) {
+        const uint64_t b = L.run[i].begin > e_lo ? L.run[i].begin : e_lo;
+        const uint64_t e = L.run[i].end < e_hi ? L.run[i].end : e_hi;
+        if (b >= e) continue;
+        const uint32_t start = L.run[i].start;
+        const int dir = L.run[i].dir;
+        const uint32_t out_first = L.run[i].out_first;
+        const uint64_t shift = uint64_t(L.run[i].out_shift);
+        for (uint32_t k = 0; k < EPV; ++k) {
+            const uint64_t el = e_lo + uint64_t(tid) * EPV + k;
+            if (el < b || el >= e) continue;
+            T r;
+            if constexpr (TREE) {
+                r = tree_element<T, OP, K>(L, K, start, el);
+            } else {
+                A a = static_cast<A>(static_cast<const T*>(L.in[start])[el]);
+                for (uint32_t j = 1; j < uint32_t(K); ++j)
+                    a = combine<OP, A>(
+                            a, static_cast<A>(static_cast<const T*>(L.in[rotate_rank(start, dir, j, K)])[el]),
+                            new_wins);
+                r = static_cast<T>(a);
+            }
+            for (uint32_t m = 0; m < nout; ++m)
+                static_cast<T*>(L.out[rotate_rank(out_first, 1, m, K)])[el - shift] = r;
+        }
+    }
+}
+
 // TREE selects the binomial-tree combination; it is a template parameter, not a run-time branch,
 // so that the tree's K live accumulators do not cost the left fold any registers.
 template <typename T, int OP, int K, bool TREE>
 __global__ void __launch_bounds__(kThreads) fold_flat_kernel(const FlatLaunch L) {
-    using A = typename Wide<T>::type;
     constexpr uint32_t EPV = kVecBytes / sizeof(T);
     constexpr uint32_t TILE = kThreads * EPV;  // elements per tile
     const uint32_t tile = blockIdx.x;
@@ -513,38 +551,74 @@ __global__ void __launch_bounds__(kThreads) fold_flat_kernel(const FlatLaunch L)
         return;
     }
 
-    // A tile that straddles a run border or the end of the buffer: element by element, one run at a
-    // time so that ranks and destinations stay uniform.
-    const uint64_t e_lo = uint64_t(tile) * TILE;
-    const uint64_t e_hi = e_lo + TILE < L.count ? e_lo + TILE : L.count;
-    for (uint32_t i = 0; i < L.nruns; ++i) {
-        const uint64_t b = L.run[i].begin > e_lo ? L.run[i].begin : e_lo;
-        const uint64_t e = L.run[i].end < e_hi ? L.run[i].end : e_hi;
-        if (b >= e) continue;
-        const uint32_t start = L.run[i].start;
-        const int dir = L.run[i].dir;
-        const uint32_t out_first = L.run[i].out_first;
-        const uint64_t shift = uint64_t(L.run[i].out_shift);
-        for (uint32_t k = 0; k < EPV; ++k) {
-            const uint64_t el = e_lo + uint64_t(tid) * EPV + k;
-            if (el < b || el >= e) continue;
-            T r;
-            if constexpr (TREE) {
-                r = tree_element<T, OP, K>(L, K, start, el);
-            } else {
-                A a = static_cast<A>(static_cast<const T*>(L.in[start])[el]);
-                for (uint32_t j = 1; j < uint32_t(K); ++j)
-                    a = combine<OP, A>(
-                            a, static_cast<A>(static_cast<const T*>(L.in[rotate_rank(start, dir, j, K)])[el]),
-                            new_wins);
-                r = static_cast<T>(a);
-            }
-            for (uint32_t m = 0; m < nout; ++m)
-                static_cast<T*>(L.out[rotate_rank(out_first, 1, m, K)])[el - shift] = r;
+    flat_tile_by_element<T, OP, K, TREE>(L, tile, tid);
+}
+
+// Group form of the flat left fold for all_reduce shapes (every rank an output, outputs at the
+// inputs' offsets).  A workgroup of kGroupWaves wavefronts owns kGroupWaves tiles that lie
+// kGroupStride tiles apart.  Wavefront w loads input r of tile (w + r) % kGroupWaves, so the K loads
+// it issues together go to different tiles; the tiles are exchanged through LDS, wavefront w folds
+// tile w, the results are exchanged again, and wavefront w stores output m of tile
+// (w + m) % kGroupWaves.  Measured on MI355X with 8 + 8 fp32 buffers, over several buffer sizes
+// and placements: 80 - 85 % of the HBM peak where one wavefront per tile reaches 64 - 76 % and
+// swings with the placement; strides of 32 and 64 tiles are the good ones, 128 and more lose the gain.
+template <typename T, int OP, int K>
+__global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(const FlatLaunch L) {
+    constexpr uint32_t EPV = kVecBytes / sizeof(T);
+    constexpr uint32_t TILE = kThreads * EPV;
+    constexpr uint32_t W = kGroupWaves;
+    __shared__ u32x4 stage[W][K][kThreads];
+    __shared__ u32x4 result[W][kThreads];
+    __shared__ uint32_t folded[W];
+    const uint32_t tid = threadIdx.x % kThreads;
+    // wavefront index, made known to be uniform so that it selects pointers in scalar registers
+    const uint32_t wave = uint32_t(__builtin_amdgcn_readfirstlane(int(threadIdx.x / kThreads)));
+    const uint32_t first = (blockIdx.x / kGroupStride) * (W * kGroupStride) + blockIdx.x % kGroupStride;
+
+    // tile k of the group is first + k * kGroupStride; it is loaded if it lies inside the buffers
+    {
+        u32x4 x[K];
+#pragma unroll
+        for (int r = 0; r < K; ++r) {
+            const uint64_t tile = uint64_t(first) + ((wave + r) % W) * kGroupStride;
+            if ((tile + 1) * TILE <= L.count)
+                x[r] = load_tile_vec(static_cast<const char*>(L.in[r]) + tile * (kThreads * kVecBytes), tid);
+            else
+                x[r] = u32x4{0u, 0u, 0u, 0u};  // never folded: such a tile goes element by element
+        }
+#pragma unroll
+        for (int r = 0; r < K; ++r) stage[(wave + r) % W][r][tid] = x[r];
+    }
+    __syncthreads();
+
+    const uint32_t mine = first + wave * kGroupStride;
+    int run = -1;
+    for (uint32_t base = 0; base < L.nruns; base += 8) {
+#pragma unroll
+        for (uint32_t i = 0; i < 8; ++i)
+            if (mine >= L.tile_lo[base + i] && mine < L.tile_hi[base + i]) run = int(base + i);
+    }
+    if (run >= 0) {
+        // the whole tile shares one fold order (and lies inside the buffers)
+        u32x4 x[K];
+#pragma unroll
+        for (int r = 0; r < K; ++r) x[r] = stage[wave][r][tid];
+        result[wave][tid] = fold_from<T, OP, K>(x, L.run[run].start, L.run[run].dir, L.new_wins_ties != 0);
+    } else if (mine < L.total_tiles) {
+        flat_tile_by_element<T, OP, K, false>(L, mine, tid);  // reads and writes global memory itself
+    }
+    if (tid == 0) folded[wave] = run >= 0 ? 1u : 0u;
+    __syncthreads();
+
+#pragma unroll
+    for (int m = 0; m < K; ++m) {
+        const uint32_t k = (wave + m) % W;
+        if (folded[k]) {
+            const uint64_t tile = uint64_t(first) + k * kGroupStride;
+            store_tile_vec(static_cast<char*>(L.out[m]) + tile * (kThreads * kVecBytes), tid, result[k][tid]);
         }
     }
 }
-
 
 // ---------------------------------------------------------------------------------------------
 // Launchers for one element type.  `op` is kSum / kMax / kMin; SUM exists for the unsigned and the
@@ -583,6 +657,16 @@ FlatFn pick_flat_k(uint32_t nranks) {
 
 template <typename T, int OP>
 FlatFn pick_flat(const FlatLaunch& L) {
+    if (L.waves == kGroupWaves) {  // asked for by the planner on all_reduce shapes only
+        if (L.tree || L.nout != L.nranks) return nullptr;
+        switch (L.nranks) {
+            case 2: return fold_group_kernel<T, OP, 2>;
+            case 3: return fold_group_kernel<T, OP, 3>;
+            case 4: return fold_group_kernel<T, OP, 4>;
+            case 8: return fold_group_kernel<T, OP, 8>;
+            default: return nullptr;
+        }
+    }
     return L.tree ? pick_flat_k<T, OP, true>(L.nranks) : pick_flat_k<T, OP, false>(L.nranks);
 }
 

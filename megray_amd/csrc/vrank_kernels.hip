@@ -165,11 +165,11 @@ const void* pack_kernel_for(const PackLaunch& L) {
     return reinterpret_cast<const void*>(fn);
 }
 
-hipError_t enqueue(const void* kernel, uint32_t grid, const void* launch, hipStream_t stream) {
+hipError_t enqueue(const void* kernel, uint32_t grid, uint32_t block, const void* launch, hipStream_t stream) {
     if (!kernel) return hipErrorInvalidValue;
     if (!grid) return hipSuccess;
     void* args[] = {const_cast<void*>(launch)};
-    return hipLaunchKernel(kernel, dim3(grid), dim3(kThreads), args, 0, stream);
+    return hipLaunchKernel(kernel, dim3(grid), dim3(block), args, 0, stream);
 }
 
 }  // namespace vrank

@@ -79,7 +79,17 @@ struct FlatLaunch {
     uint32_t new_wins_ties;
     uint32_t elem_size;
     uint32_t tree;  // 1: combine in binomial-tree order towards rank run.start instead of a left fold
+    uint32_t waves;  // wavefronts per workgroup: 1, or kGroupWaves for the group form (all_reduce shapes)
 };
+
+// Group form of the flat fold: a workgroup of kGroupWaves wavefronts owns kGroupWaves tiles that lie
+// kGroupStride tiles apart; launches of fewer than kGroupMinTiles tiles keep one wavefront per tile.
+constexpr uint32_t kGroupWaves = 4;
+constexpr uint32_t kGroupStride = 32;
+constexpr uint32_t kGroupMinTiles = 1024;
+constexpr uint32_t group_grid(uint32_t total_tiles) {
+    return (total_tiles + kGroupWaves * kGroupStride - 1) / (kGroupWaves * kGroupStride) * kGroupStride;
+}
 
 // One launch of the element-wise tree kernel: out[e] = binomial-tree combination of in[*][e]
 // towards `root`, any rank count, any alignment.

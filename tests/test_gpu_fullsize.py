@@ -11,37 +11,38 @@ torch = pytest.importorskip("torch")
 pytestmark = pytest.mark.gpu
 
 import megray_amd as mr  # noqa: E402
+from megray_amd import synth  # noqa: E402
 
 DEV = "cuda:0"
-SEED = 0x4D656752
+NP_OF = {torch.float16: np.float16, torch.float32: np.float32, torch.int32: np.int32, torch.int64: np.int64,
+         torch.uint8: np.uint8, torch.int8: np.int8}
 
 
-def gen(n, dtype, rank, kind="full"):
-    g = torch.Generator(device=DEV)
-    g.manual_seed(SEED + rank)
-    if dtype.is_floating_point:
-        if kind == "normal":  # normal(0, 0.01)
-            return (torch.randn(n, generator=g, device=DEV, dtype=torch.float32) * 0.01).to(dtype)
-        return (torch.rand(n, generator=g, device=DEV, dtype=torch.float32) * 2 - 1).to(dtype)
-    info = torch.iinfo(dtype)
-    if dtype == torch.int64:  # randint cannot span the whole int64 range in one call
-        hi = torch.randint(-2 ** 31, 2 ** 31, (n,), generator=g, device=DEV, dtype=torch.int64)
-        lo = torch.randint(0, 2 ** 32, (n,), generator=g, device=DEV, dtype=torch.int64)
-        return (hi << 32) | lo
-    return torch.randint(info.min, info.max + 1, (n,), generator=g, device=DEV, dtype=dtype)
+def gen(n, dtype, rank, kind="uniform"):
+    """Rank `rank`'s buffer from the counter-based generator (uniform[-1,1) / full-range integers /
+    approximately normal(0, 0.01)), filled on the device."""
+    return synth.fill_torch(dtype, n, rank, kind, device=DEV)
+
+
+def regen(n, dtype, rank, start, kind="uniform"):
+    """The same elements computed on the host, without touching the device buffer."""
+    return synth.fill_np(NP_OF[dtype], n, rank, kind, start)
 
 
 def bits(t):
     return t.view(torch.uint8) if t.element_size() == 1 else t.view({2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()])
 
 
-def window_problem(ins, nranks, chunk_len, offset, width):
-    """Host copies of [chunk*chunk_len + offset, +width) of every input for every chunk, laid out as a
-    small collective of length nranks*width whose chunk c is the window of chunk c."""
+def window_problem(ins, nranks, chunk_len, offset, width, kind="uniform"):
+    """[chunk*chunk_len + offset, +width) of every input for every chunk, laid out as a small collective
+    of length nranks*width whose chunk c is the window of chunk c.  The windows are regenerated on the
+    host; the first of each rank is also compared with what the device buffer holds."""
     mini = []
-    for t in ins:
-        parts = [t[c * chunk_len + offset: c * chunk_len + offset + width] for c in range(nranks)]
-        mini.append(torch.cat(parts).cpu().numpy())
+    for r, t in enumerate(ins):
+        parts = [regen(width, t.dtype, r, c * chunk_len + offset, kind) for c in range(nranks)]
+        on_device = t[offset:offset + width].cpu().numpy()
+        assert np.array_equal(on_device.view(np.uint8), parts[0].view(np.uint8)), "device data is not the generator's"
+        mini.append(np.concatenate(parts))
     return mini
 
 
@@ -121,7 +122,7 @@ def test_c2_reduce_scatter_then_all_gather_fp16():
     # windows against the oracle (tolerance stated by the task: 1 ulp; asserted: 0)
     width = 1 << 13
     for offset in (0, recvlen // 3, recvlen - width):
-        mini = window_problem(ins, nranks, recvlen, offset, width)
+        mini = window_problem(ins, nranks, recvlen, offset, width, "normal")
         want = orc.fold_reduce_scatter(mini, orc.FLOAT16, orc.SUM, orc.ORDER_UCX)
         for r in range(nranks):
             got = parts[r][offset:offset + width].cpu().numpy()
@@ -167,12 +168,31 @@ def test_c5_all_to_all_uint8_and_int8_wraparound():
     assert torch.equal(((wide + 128) % 256 - 128).to(torch.int8), souts[0][:1 << 20])
 
 
+def test_c1_all_reduce_fp32_4x2p20_rank_order():
+    """4 ranks x 2^20 fp32 SUM folded rank 0 -> 3: the reference tests' own expectation loop
+    (test/test_opr.cpp:321-330), compared in full."""
+    nranks, n = 4, 1 << 20
+    host = [regen(n, torch.float32, r, 0) for r in range(nranks)]
+    ins = [gen(n, torch.float32, r) for r in range(nranks)]
+    outs = [torch.empty_like(t) for t in ins]
+    mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, mr.FoldOrder.RANK0)
+    torch.cuda.synchronize()
+    want = orc.test_all_reduce_f32(host, orc.SUM)
+    for r in range(nranks):
+        assert np.array_equal(outs[r].cpu().numpy().view(np.uint32), want[r].view(np.uint32)), f"rank {r}"
+    # the default (ucx ring) order differs from it somewhere on this data, or the test would not tell them apart
+    mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM)
+    torch.cuda.synchronize()
+    assert not np.array_equal(outs[0].cpu().numpy().view(np.uint32), want[0].view(np.uint32))
+    ring = orc.ucx_all_reduce(host, orc.FLOAT32, orc.SUM)
+    assert np.array_equal(outs[2].cpu().numpy().view(np.uint32), ring[2].view(np.uint32))
+
+
 def test_small_message_sizes_are_exact():
     # the latency sweep's shapes: 8 ranks, 4 KiB .. 1 MiB per rank
-    rng = np.random.default_rng(4)
     for nbytes in (4096, 16384, 65536, 262144, 1048576):
         n = nbytes // 4
-        host = [rng.uniform(-1, 1, n).astype(np.float32) for _ in range(8)]
+        host = [regen(n, torch.float32, r, 0) for r in range(8)]
         ins = [torch.from_numpy(h).to(DEV) for h in host]
         outs = [torch.empty_like(t) for t in ins]
         mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM)

@@ -51,6 +51,30 @@ def test_all_reduce_fused_all_orders(dtype, nranks):
                                                  f"order={order} rank={r}")
 
 
+@pytest.mark.parametrize("dtype", REDUCE_TYPES)
+def test_all_reduce_group_form(dtype):
+    """Launches of 1024 tiles and more take the group form of the flat kernel (four wavefronts per
+    workgroup, four tiles 32 tiles apart): ragged lengths, so that chunk borders fall inside tiles and the
+    last group of tiles is incomplete; out of place and in place."""
+    size = orc.dtype_size(dtype)
+    rng = np.random.default_rng(77 + dtype)
+    for nranks, tiles in ((2, 1024), (3, 1500), (4, 1301), (8, 2051)):
+        length = (tiles * 1024 + 1024 - 16 * (nranks - 1)) // size - 3
+        ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+        d_in = [to_device(x) for x in ins]
+        runs, _, _ = mr.describe(mr.Collective.ALL_REDUCE, d_in, [empty_device(length * size) for _ in range(nranks)],
+                                 length, dtype)
+        assert runs and all(r["waves"] == 4 for r in runs), "the group form is not what runs here"
+        for op, order in ((orc.SUM, orc.ORDER_UCX), (orc.MAX, orc.ORDER_SHM), (orc.MIN, orc.ORDER_RANK0),
+                          (orc.SUM, orc.ORDER_SHM)):
+            want = orc.fold_all_reduce(ins, dtype, op, order)
+            for inplace in (False, True):
+                got = run_all_reduce(ins, dtype, op, order, mr.Schedule.FUSED, inplace=inplace)
+                for r in range(nranks):
+                    assert_same(got[r], want[r], f"group form dtype={dtype} N={nranks} len={length} op={op} "
+                                                 f"order={order} inplace={inplace} rank={r}")
+
+
 @pytest.mark.parametrize("dtype", [orc.INT8, orc.INT32, orc.FLOAT32, orc.FLOAT64, orc.UINT64])
 def test_all_reduce_equals_literal_ring_replay(dtype):
     """Against the oracle's literal replay of src/ucx/all_reduce.cpp, not only its fold form."""
