@@ -216,13 +216,35 @@ struct ByteAcc {
     }
 };
 
-// Left folds keep one accumulator, and for bytes the plain element-wise form measured faster; the
-// tree keeps K accumulators alive, where the packed byte form is what fits the register file.
+// int8 / uint8 SUM: four bytes per 32-bit register are added at once.  The low seven bits of every
+// byte are added with the top bits masked off, so no carry crosses a byte border, and the top bits
+// are put back with an exclusive or: exactly the byte-wise sum mod 256.
+struct ByteSumAcc {
+    u32x4 raw;
+    static __device__ __forceinline__ u32x4 add(u32x4 a, u32x4 b) {
+        const u32x4 low = (a & 0x7f7f7f7fu) + (b & 0x7f7f7f7fu);
+        return low ^ ((a ^ b) & 0x80808080u);
+    }
+    __device__ __forceinline__ void seed(u32x4 r) { raw = r; }
+    __device__ __forceinline__ void fold(u32x4 r, bool) { raw = add(raw, r); }
+    __device__ __forceinline__ void merge(const ByteSumAcc& other) { raw = add(raw, other.raw); }
+    __device__ __forceinline__ u32x4 finish() const { return raw; }
+};
+
+// Accumulator of a left fold: bytes in packed form (element by element they compile to several
+// instructions per byte and spill), FLOAT16 in fp32, everything else element-wise in its own type.
 template <typename T, int OP>
-using AccFor = typename std::conditional<std::is_same<T, _Float16>::value, HalfAcc<OP>, VecAcc<T, OP>>::type;
+using ByteAccFor = typename std::conditional<
+        OP == kSum, ByteSumAcc,
+        typename std::conditional<OP == kMax || OP == kMin, ByteAcc<T, OP>, VecAcc<T, OP>>::type>::type;
 
 template <typename T, int OP>
-using TreeAccFor = typename std::conditional<sizeof(T) == 1, ByteAcc<T, OP>, AccFor<T, OP>>::type;
+using AccFor = typename std::conditional<
+        sizeof(T) == 1, ByteAccFor<T, OP>,
+        typename std::conditional<std::is_same<T, _Float16>::value, HalfAcc<OP>, VecAcc<T, OP>>::type>::type;
+
+template <typename T, int OP>
+using TreeAccFor = AccFor<T, OP>;
 
 // K > 0: fold count known at compile time, all K loads of a lane are issued before the first use.
 // K == 0: fold count read from the launch, loads issued in groups of four.

@@ -86,7 +86,7 @@ struct FlatLaunch {
 // kGroupStride tiles apart; launches of fewer than kGroupMinTiles tiles keep one wavefront per tile.
 constexpr uint32_t kGroupWaves = 4;
 constexpr uint32_t kGroupStride = 32;
-constexpr uint32_t kGroupMinTiles = 1024;
+constexpr uint32_t kGroupMinTiles = 4096;
 constexpr uint32_t group_grid(uint32_t total_tiles) {
     return (total_tiles + kGroupWaves * kGroupStride - 1) / (kGroupWaves * kGroupStride) * kGroupStride;
 }

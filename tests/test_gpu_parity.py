@@ -53,12 +53,12 @@ def test_all_reduce_fused_all_orders(dtype, nranks):
 
 @pytest.mark.parametrize("dtype", REDUCE_TYPES)
 def test_all_reduce_group_form(dtype):
-    """Launches of 1024 tiles and more take the group form of the flat kernel (four wavefronts per
+    """Launches of 4096 tiles and more take the group form of the flat kernel (four wavefronts per
     workgroup, four tiles 32 tiles apart): ragged lengths, so that chunk borders fall inside tiles and the
     last group of tiles is incomplete; out of place and in place."""
     size = orc.dtype_size(dtype)
     rng = np.random.default_rng(77 + dtype)
-    for nranks, tiles in ((2, 1024), (3, 1500), (4, 1301), (8, 2051)):
+    for nranks, tiles in ((2, 4096), (3, 4500), (4, 4301), (8, 5051)):
         length = (tiles * 1024 + 1024 - 16 * (nranks - 1)) // size - 3
         ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
         d_in = [to_device(x) for x in ins]

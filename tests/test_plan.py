@@ -249,7 +249,7 @@ def test_full_size_plan_shapes():
     assert br == bw == 8 * n * 4
     assert all(r["waves"] == 4 for r in runs)  # the group form: four wavefronts, four tiles per workgroup
     # short launches, reduce_scatter shapes and tree reductions keep one wavefront per tile
-    small, _, _ = mr.describe(mr.Collective.ALL_REDUCE, sp, rp, 1 << 17, orc.FLOAT32)
+    small, _, _ = mr.describe(mr.Collective.ALL_REDUCE, sp, rp, 1 << 19, orc.FLOAT32)
     assert small and all(r["waves"] == 1 for r in small)
     rs, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, sp, rp, 1 << 22, orc.FLOAT32)
     assert rs and all(r["waves"] == 1 and r["vector"] == 2 for r in rs)
