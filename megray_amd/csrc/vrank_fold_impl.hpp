@@ -576,15 +576,16 @@ __global__ void __launch_bounds__(kThreads) fold_flat_kernel(const FlatLaunch L)
     flat_tile_by_element<T, OP, K, TREE>(L, tile, tid);
 }
 
-// Group form of the flat left fold for all_reduce shapes (every rank an output, outputs at the
-// inputs' offsets).  A workgroup of kGroupWaves wavefronts owns kGroupWaves tiles that lie
-// kGroupStride tiles apart.  Wavefront w loads input r of tile (w + r) % kGroupWaves, so the K loads
-// it issues together go to different tiles; the tiles are exchanged through LDS, wavefront w folds
-// tile w, the results are exchanged again, and wavefront w stores output m of tile
-// (w + m) % kGroupWaves.  Measured on MI355X with 8 + 8 fp32 buffers, over several buffer sizes
-// and placements: 80 - 85 % of the HBM peak where one wavefront per tile reaches 64 - 76 % and
-// swings with the placement; strides of 32 and 64 tiles are the good ones, 128 and more lose the gain.
-template <typename T, int OP, int K>
+// Group form of the flat fold for launches of many tiles.  A workgroup of kGroupWaves wavefronts
+// owns kGroupWaves tiles that lie kGroupStride tiles apart.  Wavefront w loads input r of tile
+// (w + r) % kGroupWaves, so the K loads it issues together go to different tiles; the tiles are
+// exchanged through LDS and wavefront w folds tile w.  Where every rank is an output at the inputs'
+// offsets (all_reduce, L.exchange) the results are exchanged again and wavefront w stores output m
+// of tile (w + m) % kGroupWaves; otherwise wavefront w stores its own tile.  Measured on MI355X,
+// fp32, over several buffer sizes and placements, against one wavefront per tile on the same
+// device: 8 in + 8 out 83 % of the HBM peak against 70 - 76 %, 8 in + 1 out 85 % against 75 - 79 %;
+// strides of 32 and 64 tiles are the good ones, 16 and 128 lose most of the gain.
+template <typename T, int OP, int K, bool TREE>
 __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(const FlatLaunch L) {
     constexpr uint32_t EPV = kVecBytes / sizeof(T);
     constexpr uint32_t TILE = kThreads * EPV;
@@ -614,6 +615,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
     __syncthreads();
 
     const uint32_t mine = first + wave * kGroupStride;
+    const bool exchange = L.exchange != 0;
     int run = -1;
     for (uint32_t base = 0; base < L.nruns; base += 8) {
 #pragma unroll
@@ -625,10 +627,25 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
         u32x4 x[K];
 #pragma unroll
         for (int r = 0; r < K; ++r) x[r] = stage[wave][r][tid];
-        result[wave][tid] = fold_from<T, OP, K>(x, L.run[run].start, L.run[run].dir, L.new_wins_ties != 0);
+        u32x4 res;
+        if constexpr (TREE) {
+            res = tree_from<T, OP, K>(x, L.run[run].start);
+        } else {
+            res = fold_from<T, OP, K>(x, L.run[run].start, L.run[run].dir, L.new_wins_ties != 0);
+        }
+        if (exchange) {
+            result[wave][tid] = res;
+        } else {
+            const uint64_t out_off =
+                    uint64_t(mine) * (kThreads * kVecBytes) - uint64_t(L.run[run].out_shift) * sizeof(T);
+            const uint32_t out_first = L.run[run].out_first;
+            for (uint32_t m = 0; m < L.nout; ++m)
+                store_tile_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, K)]) + out_off, tid, res);
+        }
     } else if (mine < L.total_tiles) {
-        flat_tile_by_element<T, OP, K, false>(L, mine, tid);  // reads and writes global memory itself
+        flat_tile_by_element<T, OP, K, TREE>(L, mine, tid);  // reads and writes global memory itself
     }
+    if (!exchange) return;
     if (tid == 0) folded[wave] = run >= 0 ? 1u : 0u;
     __syncthreads();
 
@@ -677,18 +694,20 @@ FlatFn pick_flat_k(uint32_t nranks) {
     }
 }
 
+template <typename T, int OP, bool TREE>
+FlatFn pick_group_k(uint32_t nranks) {
+    switch (nranks) {
+        case 2: return fold_group_kernel<T, OP, 2, TREE>;
+        case 3: return fold_group_kernel<T, OP, 3, TREE>;
+        case 4: return fold_group_kernel<T, OP, 4, TREE>;
+        case 8: return fold_group_kernel<T, OP, 8, TREE>;
+        default: return nullptr;
+    }
+}
+
 template <typename T, int OP>
 FlatFn pick_flat(const FlatLaunch& L) {
-    if (L.waves == kGroupWaves) {  // asked for by the planner on all_reduce shapes only
-        if (L.tree || L.nout != L.nranks) return nullptr;
-        switch (L.nranks) {
-            case 2: return fold_group_kernel<T, OP, 2>;
-            case 3: return fold_group_kernel<T, OP, 3>;
-            case 4: return fold_group_kernel<T, OP, 4>;
-            case 8: return fold_group_kernel<T, OP, 8>;
-            default: return nullptr;
-        }
-    }
+    if (L.waves == kGroupWaves) return L.tree ? pick_group_k<T, OP, true>(L.nranks) : pick_group_k<T, OP, false>(L.nranks);
     return L.tree ? pick_flat_k<T, OP, true>(L.nranks) : pick_flat_k<T, OP, false>(L.nranks);
 }
 

@@ -141,10 +141,12 @@ private:
         L.new_wins_ties = m_new_wins ? 1 : 0;
         L.elem_size = m_elem;
         L.tree = m_tree ? 1 : 0;
-        // all_reduce shapes (every rank an output, outputs at the inputs' offsets) take the group form
+        // launches of many tiles take the group form; all_reduce shapes (every rank an output, outputs at
+        // the inputs' offsets) also exchange the results between the wavefronts of a group
         bool unshifted = true;
         for (const Run& r : m_runs) unshifted = unshifted && r.in_begin == r.out_begin;
-        L.waves = (!m_tree && m_nout == m_nranks && unshifted && total >= kGroupMinTiles) ? kGroupWaves : 1;
+        L.waves = total >= kGroupMinTiles ? kGroupWaves : 1;
+        L.exchange = (L.waves == kGroupWaves && !m_tree && m_nout == m_nranks && unshifted) ? 1 : 0;
         m_plan.steps.push_back(step);
         return true;
     }

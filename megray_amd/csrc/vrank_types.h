@@ -79,7 +79,8 @@ struct FlatLaunch {
     uint32_t new_wins_ties;
     uint32_t elem_size;
     uint32_t tree;  // 1: combine in binomial-tree order towards rank run.start instead of a left fold
-    uint32_t waves;  // wavefronts per workgroup: 1, or kGroupWaves for the group form (all_reduce shapes)
+    uint32_t waves;     // wavefronts per workgroup: 1, or kGroupWaves for the group form (launches of many tiles)
+    uint32_t exchange;  // group form: 1 = every rank is an output at the inputs' offsets, results are exchanged too
 };
 
 // Group form of the flat fold: a workgroup of kGroupWaves wavefronts owns kGroupWaves tiles that lie

@@ -75,6 +75,70 @@ def test_all_reduce_group_form(dtype):
                                                  f"order={order} inplace={inplace} rank={r}")
 
 
+def tree_expectation(ins, dtype, op, root):
+    """reduce towards `root`: the oracle's literal replay of the binomial tree; FLOAT16 (which the
+    reference cannot reduce) as the same tree in fp32 with one rounding."""
+    nranks = len(ins)
+    if dtype != orc.FLOAT16:
+        return orc.ucx_reduce(ins, dtype, op, root)[root]
+    a = [ins[(root + v) % nranks].astype(np.float32) for v in range(nranks)]
+    bit = 1
+    while bit < nranks:
+        for v in range(0, nranks - bit, 2 * bit):
+            x, y = a[v], a[v + bit]
+            with np.errstate(over="ignore"):
+                a[v] = {orc.SUM: x + y, orc.MAX: np.where(y > x, y, x), orc.MIN: np.where(y < x, y, x)}[op]
+        bit *= 2
+    with np.errstate(over="ignore"):
+        return a[0].astype(np.float16)
+
+
+@pytest.mark.parametrize("dtype", REDUCE_TYPES)
+def test_group_form_with_one_output(dtype):
+    """reduce_scatter, reduce towards a root and the two-phase all_reduce at 4096 tiles and more: the
+    group form in which every wavefront stores the tile it folded (shifted outputs, one destination)."""
+    size = orc.dtype_size(dtype)
+    rng = np.random.default_rng(177 + dtype)
+    for nranks, tiles in ((3, 4200), (8, 4999)):
+        recvlen = (tiles * 1024 // size) // nranks // 16 * 16 + 16  # keeps chunk r of rank r on a 16-byte boundary
+        length = recvlen * nranks
+        ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+        d_in = [to_device(x) for x in ins]
+        parts = [empty_device(recvlen * size) for _ in range(nranks)]
+        runs, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, d_in, parts, recvlen, dtype)
+        assert runs and all(r["waves"] == 4 for r in runs), "the group form is not what runs here"
+        for op, order in ((orc.SUM, orc.ORDER_UCX), (orc.MAX, orc.ORDER_UCX), (orc.MIN, orc.ORDER_SHM)):
+            want = orc.fold_reduce_scatter(ins, dtype, op, order)
+            mr.reduce_scatter(d_in, parts, recvlen, dtype, op, order)
+            torch.cuda.synchronize()
+            for r in range(nranks):
+                assert_same(to_host(parts[r], ins[0].dtype), want[r],
+                            f"reduce_scatter group form dtype={dtype} N={nranks} op={op} order={order} rank={r}")
+            # in place: rank r's result lands on its own chunk r
+            d_io = [to_device(x) for x in ins]
+            mr.reduce_scatter(d_io, [d_io[r][r * recvlen * size:(r + 1) * recvlen * size] for r in range(nranks)],
+                              recvlen, dtype, op, order)
+            torch.cuda.synchronize()
+            for r in range(nranks):
+                got = to_host(d_io[r], ins[0].dtype)[r * recvlen:(r + 1) * recvlen]
+                assert_same(got, want[r], f"in-place reduce_scatter group form dtype={dtype} N={nranks} rank={r}")
+        for op in (orc.SUM, orc.MAX):
+            root = nranks - 2
+            out = empty_device(length * size)
+            mr.reduce_to_root(d_in, out, length, dtype, op, root)
+            torch.cuda.synchronize()
+            assert_same(to_host(out, ins[0].dtype), tree_expectation(ins, dtype, op, root),
+                        f"tree reduce group form dtype={dtype} N={nranks} op={op}")
+            mr.reduce_to_root(d_in, out, length, dtype, op, root, orc.ORDER_RANK0)
+            torch.cuda.synchronize()
+            assert_same(to_host(out, ins[0].dtype), orc.fold_all_reduce(ins, dtype, op, orc.ORDER_RANK0)[0],
+                        f"left-fold reduce group form dtype={dtype} N={nranks} op={op}")
+        want = orc.fold_all_reduce(ins, dtype, orc.SUM, orc.ORDER_UCX)
+        got = run_all_reduce(ins, dtype, orc.SUM, orc.ORDER_UCX, mr.Schedule.TWO_PHASE)
+        for r in range(nranks):
+            assert_same(got[r], want[r], f"two-phase group form dtype={dtype} N={nranks} rank={r}")
+
+
 @pytest.mark.parametrize("dtype", [orc.INT8, orc.INT32, orc.FLOAT32, orc.FLOAT64, orc.UINT64])
 def test_all_reduce_equals_literal_ring_replay(dtype):
     """Against the oracle's literal replay of src/ucx/all_reduce.cpp, not only its fold form."""
@@ -329,20 +393,7 @@ def test_reduce_to_root(dtype):
                         mr.reduce_to_root(d_in, d_out, length, dtype, op, root)
                         torch.cuda.synchronize()
                         got = to_host(d_out, ins[0].dtype)
-                        if dtype == orc.FLOAT16:
-                            a = [ins[(root + v) % nranks].astype(np.float32) for v in range(nranks)]
-                            bit = 1
-                            while bit < nranks:
-                                for v in range(0, nranks - bit, 2 * bit):
-                                    x, y = a[v], a[v + bit]
-                                    with np.errstate(over="ignore"):
-                                        a[v] = {orc.SUM: x + y, orc.MAX: np.where(y > x, y, x),
-                                                orc.MIN: np.where(y < x, y, x)}[op]
-                                bit *= 2
-                            with np.errstate(over="ignore"):
-                                want = a[0].astype(np.float16)
-                        else:
-                            want = orc.ucx_reduce(ins, dtype, op, root)[root]
+                        want = tree_expectation(ins, dtype, op, root)
                         assert_same(got, want, f"reduce dtype={dtype} N={nranks} len={length} root={root} op={op}")
                     for order in (orc.ORDER_SHM, orc.ORDER_RANK0):
                         d_in = [to_device(x) for x in ins]

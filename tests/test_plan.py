@@ -248,13 +248,15 @@ def test_full_size_plan_shapes():
     assert sum(r["count"] for r in runs) == n
     assert br == bw == 8 * n * 4
     assert all(r["waves"] == 4 for r in runs)  # the group form: four wavefronts, four tiles per workgroup
-    # short launches, reduce_scatter shapes and tree reductions keep one wavefront per tile
-    small, _, _ = mr.describe(mr.Collective.ALL_REDUCE, sp, rp, 1 << 19, orc.FLOAT32)
-    assert small and all(r["waves"] == 1 for r in small)
+    # so do long reduce_scatter and tree launches; short launches keep one wavefront per tile
     rs, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, sp, rp, 1 << 22, orc.FLOAT32)
-    assert rs and all(r["waves"] == 1 and r["vector"] == 2 for r in rs)
+    assert rs and all(r["waves"] == 4 and r["vector"] == 2 for r in rs)
     tree, _, _ = mr.describe(mr.Collective.REDUCE, sp, rp, 1 << 22, orc.FLOAT32, root=3)
-    assert tree and all(r["waves"] == 1 for r in tree)
+    assert tree and all(r["waves"] == 4 and r["dir"] == 0 for r in tree)
+    for coll, count in ((mr.Collective.ALL_REDUCE, 1 << 19), (mr.Collective.REDUCE_SCATTER, 1 << 16),
+                        (mr.Collective.REDUCE, 1 << 19)):
+        small, _, _ = mr.describe(coll, sp, rp, count, orc.FLOAT32)
+        assert small and all(r["waves"] == 1 for r in small)
     # a buffer far beyond one launch's grid is split into several launches, nothing lost
     big = 1 << 41
     runs, br, bw = mr.describe(mr.Collective.ALL_REDUCE, [SEND_BASE, SEND_BASE + (1 << 42)],
