@@ -423,7 +423,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.nfold = 1;
                     run.nout = 1;
                     run.vector = L.width;
-                    run.waves = 1;
+                    run.waves = L.waves;
                     run.dir = 1;
                     run.tiles = L.tiles_per_copy;
                     run.count = L.block_bytes;

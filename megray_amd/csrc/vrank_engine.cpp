@@ -50,8 +50,12 @@ Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCal
                 call = {tree_kernel_for(step.tree, dtype, op), step.tree.total_tiles, kThreads, &step.tree};
                 break;
             case Step::kPack:
-                call = {pack_kernel_for(step.pack), step.pack.ncopies * step.pack.tiles_per_copy, kThreads,
-                        &step.pack};
+                if (step.pack.waves == kGroupWaves)
+                    call = {pack_kernel_for(step.pack), step.pack.ncopies * step.pack.groups_per_copy,
+                            kThreads * kGroupWaves, &step.pack};
+                else
+                    call = {pack_kernel_for(step.pack), step.pack.ncopies * step.pack.tiles_per_copy, kThreads,
+                            &step.pack};
                 break;
         }
         if (!call.kernel) {

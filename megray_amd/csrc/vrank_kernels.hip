@@ -102,6 +102,70 @@ __global__ void __launch_bounds__(kThreads) pack_kernel(const PackLaunch L) {
     }
 }
 
+// Decodes copy `copy` of a pack launch into its endpoints.
+struct PackEnds {
+    uint32_t src_rank, src_block, dst_rank, dst_block, ndst;
+};
+__device__ __forceinline__ PackEnds pack_ends(const PackLaunch& L, uint32_t copy) {
+    const uint32_t n = L.nranks;
+    if (L.mode == kPackAllToAll) return {copy / n, copy % n, copy % n, copy / n, 1};
+    if (L.mode == kPackScatter) return {L.root, copy, copy, 0, 1};
+    if (L.mode == kPackGather) return {copy, 0, L.root, copy, 1};
+    return {copy, 0, 0, copy, n};  // kPackAllGather: read once, write the block into every rank's buffer
+}
+
+// Group form of the pack kernel for long blocks of 16-byte accesses: a workgroup of kGroupWaves
+// wavefronts owns kGroupWaves tiles of one block copy, kGroupStride tiles apart; wavefront w loads
+// tile w.  With one destination it stores that tile; with N destinations (all_gather) the tiles are
+// exchanged through LDS and wavefront w stores destination m of tile (w + m) % kGroupWaves, so the
+// N stores it issues together go to different tiles.  Measured on MI355X (1 GiB and 128 MiB
+// buffers): 1 -> 8 copies 82 % of the HBM peak against 65 - 69 % with one wavefront per tile,
+// 1 -> 1 copies 84 - 87 % against 83 - 84 %.
+__global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(const PackLaunch L) {
+    constexpr uint32_t W = kGroupWaves;
+    constexpr uint32_t kTileBytes = kThreads * kVecBytes;
+    __shared__ u32x4 stage[W][kThreads];
+    __shared__ uint32_t staged[W];
+    const uint32_t tid = threadIdx.x % kThreads;
+    const uint32_t wave = uint32_t(__builtin_amdgcn_readfirstlane(int(threadIdx.x / kThreads)));
+    const uint32_t copy = blockIdx.x / L.groups_per_copy;
+    const uint32_t group = blockIdx.x - copy * L.groups_per_copy;
+    const uint32_t first = (group / kGroupStride) * (W * kGroupStride) + group % kGroupStride;
+    const PackEnds e = pack_ends(L, copy);
+    const char* src = static_cast<const char*>(L.in[e.src_rank]) + e.src_block * L.block_bytes;
+    const uint64_t dst_base = e.dst_block * L.block_bytes;
+
+    const uint32_t mine = first + wave * kGroupStride;
+    const uint64_t mine_off = uint64_t(mine) * kTileBytes;
+    const bool whole = mine_off + kTileBytes <= L.block_bytes;
+    u32x4 x = {0u, 0u, 0u, 0u};
+    if (whole) {
+        x = load_tile_vec(src + mine_off, tid);
+    } else if (mine_off < L.block_bytes) {
+        // the block's last, partial tile: this wavefront copies it to every destination itself
+        const uint64_t off = mine_off + tid * kVecBytes;
+        if (off < L.block_bytes) {
+            const u32x4 v = load_w<u32x4>(src + off);
+            for (uint32_t m = 0; m < e.ndst; ++m)
+                store_w<u32x4>(static_cast<char*>(L.out[e.dst_rank + m]) + dst_base + off, v);
+        }
+    }
+    if (e.ndst == 1) {
+        if (whole) store_tile_vec(static_cast<char*>(L.out[e.dst_rank]) + dst_base + mine_off, tid, x);
+        return;
+    }
+    stage[wave][tid] = x;
+    if (tid == 0) staged[wave] = whole ? 1u : 0u;
+    __syncthreads();
+    for (uint32_t m = 0; m < e.ndst; ++m) {
+        const uint32_t k = (wave + m) % W;
+        if (staged[k]) {
+            const uint64_t off = (uint64_t(first) + k * kGroupStride) * kTileBytes;
+            store_tile_vec(static_cast<char*>(L.out[e.dst_rank + m]) + dst_base + off, tid, stage[k][tid]);
+        }
+    }
+}
+
 FoldFn pick_copy(uint32_t elem_size) {
     switch (elem_size) {
         case 1: return fold_kernel<uint8_t, kCopy, 1, fold_unroll(1)>;
@@ -154,6 +218,7 @@ const void* tree_kernel_for(const TreeLaunch&, DType dtype, ReduceOp op) {
 
 const void* pack_kernel_for(const PackLaunch& L) {
     void (*fn)(const PackLaunch) = nullptr;
+    if (L.waves == kGroupWaves) return L.width == kVecBytes ? reinterpret_cast<const void*>(&pack_group_kernel) : nullptr;
     switch (L.width) {
         case 16: fn = pack_kernel<u32x4, pack_unroll()>; break;
         case 8: fn = pack_kernel<u32x2, pack_unroll()>; break;

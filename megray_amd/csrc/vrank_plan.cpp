@@ -507,6 +507,10 @@ Status add_pack(Plan& plan, const void* const* in, void* const* out, uint32_t nr
     const uint64_t tiles = (block_bytes + per_tile - 1) / per_tile;
     if (tiles * ncopies > 0x7fffffffull) return invalid("block too large for one pack launch");
     L.tiles_per_copy = uint32_t(tiles);
+    // long blocks of 16-byte accesses take the group form
+    L.waves = (L.width == kVecBytes && tiles >= kGroupMinTiles / 4) ? kGroupWaves : 1;
+    L.groups_per_copy = group_grid(L.tiles_per_copy);
+    if (L.waves == kGroupWaves && uint64_t(L.groups_per_copy) * ncopies > 0x7fffffffull) L.waves = 1;
     plan.steps.push_back(step);
     plan.bytes_read += block_bytes * ncopies;
     plan.bytes_written += block_bytes * ncopies;

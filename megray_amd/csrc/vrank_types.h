@@ -124,6 +124,8 @@ struct PackLaunch {
     uint32_t tiles_per_copy;
     uint32_t width;   // bytes per lane access: 16, 8, 4, 2 or 1
     uint32_t unroll;  // accesses per lane per tile
+    uint32_t waves;   // wavefronts per workgroup: 1, or kGroupWaves (16-byte accesses, long blocks)
+    uint32_t groups_per_copy;  // group form: workgroups per block copy
 };
 
 // Vectors (or elements) each lane moves per tile.  The kernels are instantiated with these values;

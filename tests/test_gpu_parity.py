@@ -254,53 +254,72 @@ COPY_TYPES = [orc.UINT8, orc.FLOAT16, orc.FLOAT32, orc.INT64, orc.CHAR]
 def test_pack_collectives(dtype):
     rng = np.random.default_rng(90 + dtype)
     size = orc.dtype_size(dtype)
-    gen = orc.UINT8 if dtype == orc.CHAR else dtype
     for nranks in (1, 2, 3, 8, 16):
         for length in (0, 1, 6, 1000, 4096 + 3):
             for misalign in (0, size):
-                ins = [rand_array(gen, nranks * length, rng) for _ in range(nranks)]
-                npdt = ins[0].dtype
-                # all_to_all
-                want = orc.ucx_all_to_all(ins, dtype)
-                d_in = [to_device(x, misalign) for x in ins]
-                d_out = [empty_device(nranks * length * size, misalign) for _ in range(nranks)]
-                mr.all_to_all(d_in, d_out, length, dtype)
-                torch.cuda.synchronize()
-                for r in range(nranks):
-                    assert_same(to_host(d_out[r], npdt), want[r], f"all_to_all dtype={dtype} N={nranks} len={length}")
-                # all_gather
-                parts = [x[:length] for x in ins]
-                want = orc.ucx_all_gather(parts, dtype)
-                d_in = [to_device(x, misalign) for x in parts]
-                d_out = [empty_device(nranks * length * size, misalign) for _ in range(nranks)]
-                mr.all_gather(d_in, d_out, length, dtype)
-                torch.cuda.synchronize()
-                for r in range(nranks):
-                    assert_same(to_host(d_out[r], npdt), want[r], f"all_gather dtype={dtype} N={nranks} len={length}")
-                root = nranks // 2
-                # scatter: only the root has a send buffer
-                want = orc.ucx_scatter([ins[root] if r == root else None for r in range(nranks)], dtype, root)
-                d_root = to_device(ins[root], misalign)
-                d_out = [empty_device(length * size, misalign) for _ in range(nranks)]
-                mr.scatter(d_root, d_out, length, dtype, root)
-                torch.cuda.synchronize()
-                for r in range(nranks):
-                    assert_same(to_host(d_out[r], npdt), want[r], f"scatter dtype={dtype} N={nranks} len={length}")
-                # gather: only the root has a receive buffer
-                want = orc.ucx_gather(parts, dtype, root)[root]
-                d_in = [to_device(x, misalign) for x in parts]
-                d_root = empty_device(nranks * length * size, misalign)
-                mr.gather(d_in, d_root, length, dtype, root)
-                torch.cuda.synchronize()
-                assert_same(to_host(d_root, npdt), want, f"gather dtype={dtype} N={nranks} len={length}")
-                # broadcast
-                want = orc.ucx_broadcast(parts, dtype, root)
-                d_root = to_device(parts[root], misalign)
-                d_out = [empty_device(length * size, misalign) for _ in range(nranks)]
-                mr.broadcast(d_root, d_out, length, dtype, root)
-                torch.cuda.synchronize()
-                for r in range(nranks):
-                    assert_same(to_host(d_out[r], npdt), want[r], f"broadcast dtype={dtype} N={nranks} len={length}")
+                check_pack_collectives(dtype, nranks, length, misalign, rng)
+
+
+@pytest.mark.parametrize("dtype", [orc.UINT8, orc.FLOAT16, orc.INT64])
+def test_pack_collectives_group_form(dtype):
+    """Blocks of 1024 tiles and more go through the group form of the pack kernel (four wavefronts, four
+    tiles per workgroup); the block ends in a partial tile."""
+    rng = np.random.default_rng(190 + dtype)
+    size = orc.dtype_size(dtype)
+    length = (1030 * 1024 + 48) // size
+    for nranks in (3, 8):
+        runs, _, _ = mr.describe(mr.Collective.ALL_GATHER, [(1 << 40) + (r << 30) for r in range(nranks)],
+                                 [(2 << 40) + (r << 34) for r in range(nranks)], length, dtype)
+        assert runs and all(r["waves"] == 4 and r["vector"] == 16 for r in runs), "the group form is not what runs here"
+        check_pack_collectives(dtype, nranks, length, 0, rng)
+
+
+def check_pack_collectives(dtype, nranks, length, misalign, rng):
+    size = orc.dtype_size(dtype)
+    gen = orc.UINT8 if dtype == orc.CHAR else dtype
+    ins = [rand_array(gen, nranks * length, rng) for _ in range(nranks)]
+    npdt = ins[0].dtype
+    # all_to_all
+    want = orc.ucx_all_to_all(ins, dtype)
+    d_in = [to_device(x, misalign) for x in ins]
+    d_out = [empty_device(nranks * length * size, misalign) for _ in range(nranks)]
+    mr.all_to_all(d_in, d_out, length, dtype)
+    torch.cuda.synchronize()
+    for r in range(nranks):
+        assert_same(to_host(d_out[r], npdt), want[r], f"all_to_all dtype={dtype} N={nranks} len={length}")
+    # all_gather
+    parts = [x[:length] for x in ins]
+    want = orc.ucx_all_gather(parts, dtype)
+    d_in = [to_device(x, misalign) for x in parts]
+    d_out = [empty_device(nranks * length * size, misalign) for _ in range(nranks)]
+    mr.all_gather(d_in, d_out, length, dtype)
+    torch.cuda.synchronize()
+    for r in range(nranks):
+        assert_same(to_host(d_out[r], npdt), want[r], f"all_gather dtype={dtype} N={nranks} len={length}")
+    root = nranks // 2
+    # scatter: only the root has a send buffer
+    want = orc.ucx_scatter([ins[root] if r == root else None for r in range(nranks)], dtype, root)
+    d_root = to_device(ins[root], misalign)
+    d_out = [empty_device(length * size, misalign) for _ in range(nranks)]
+    mr.scatter(d_root, d_out, length, dtype, root)
+    torch.cuda.synchronize()
+    for r in range(nranks):
+        assert_same(to_host(d_out[r], npdt), want[r], f"scatter dtype={dtype} N={nranks} len={length}")
+    # gather: only the root has a receive buffer
+    want = orc.ucx_gather(parts, dtype, root)[root]
+    d_in = [to_device(x, misalign) for x in parts]
+    d_root = empty_device(nranks * length * size, misalign)
+    mr.gather(d_in, d_root, length, dtype, root)
+    torch.cuda.synchronize()
+    assert_same(to_host(d_root, npdt), want, f"gather dtype={dtype} N={nranks} len={length}")
+    # broadcast
+    want = orc.ucx_broadcast(parts, dtype, root)
+    d_root = to_device(parts[root], misalign)
+    d_out = [empty_device(length * size, misalign) for _ in range(nranks)]
+    mr.broadcast(d_root, d_out, length, dtype, root)
+    torch.cuda.synchronize()
+    for r in range(nranks):
+        assert_same(to_host(d_out[r], npdt), want[r], f"broadcast dtype={dtype} N={nranks} len={length}")
 
 
 @pytest.mark.parametrize("dtype", REDUCE_TYPES)
