@@ -366,7 +366,7 @@ def main():
         "roofline": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(key),
-            "kernel": "fold_flat_kernel<float, SUM, K=8>" if args.schedule == "fused" else "fold kernels (several)",
+            "kernel": "fold_group_kernel<float, SUM, K=8>" if args.schedule == "fused" else "fold kernels (several)",
             "kernel_ms": round(kernel_ms, 4), "algorithmic_bytes_per_launch": executed // launches,
         },
     }

@@ -437,6 +437,12 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                         run.in_begin = uint64_t(c) * L.block_bytes;
                         run.out_first = c;
                         run.out_begin = 0;
+                    } else if (L.mode == kPackBroadcast) {
+                        run.start = L.root;
+                        run.in_begin = 0;
+                        run.out_first = 0;
+                        run.nout = L.nranks;
+                        run.out_begin = 0;
                     } else if (L.mode == kPackAllGather) {
                         run.start = c;
                         run.in_begin = 0;

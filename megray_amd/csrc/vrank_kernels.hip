@@ -37,34 +37,26 @@ __device__ __forceinline__ void store_w(char* p, W x) {
     __builtin_nontemporal_store(x, reinterpret_cast<W*>(p));
 }
 
+// Decodes copy `copy` of a pack launch into its endpoints.
+struct PackEnds {
+    uint32_t src_rank, src_block, dst_rank, dst_block, ndst;
+};
+__device__ __forceinline__ PackEnds pack_ends(const PackLaunch& L, uint32_t copy) {
+    const uint32_t n = L.nranks;
+    if (L.mode == kPackAllToAll) return {copy / n, copy % n, copy % n, copy / n, 1};
+    if (L.mode == kPackScatter) return {L.root, copy, copy, 0, 1};
+    if (L.mode == kPackGather) return {copy, 0, L.root, copy, 1};
+    if (L.mode == kPackBroadcast) return {L.root, 0, 0, 0, n};
+    return {copy, 0, 0, copy, n};  // kPackAllGather: read once, write the block into every rank's buffer
+}
+
 template <typename W, int U>
 __global__ void __launch_bounds__(kThreads) pack_kernel(const PackLaunch L) {
     const uint32_t copy = blockIdx.x / L.tiles_per_copy;
     const uint32_t tile = blockIdx.x - copy * L.tiles_per_copy;
-    const uint32_t n = L.nranks;
-    uint32_t src_rank, dst_rank, src_block, dst_block, ndst = 1;
-    if (L.mode == kPackAllToAll) {
-        src_rank = copy / n;
-        src_block = copy - src_rank * n;
-        dst_rank = src_block;
-        dst_block = src_rank;
-    } else if (L.mode == kPackScatter) {
-        src_rank = L.root;
-        src_block = copy;
-        dst_rank = copy;
-        dst_block = 0;
-    } else if (L.mode == kPackGather) {
-        src_rank = copy;
-        src_block = 0;
-        dst_rank = L.root;
-        dst_block = copy;
-    } else {  // kPackAllGather: read once, write the block into every rank's buffer
-        src_rank = copy;
-        src_block = 0;
-        dst_rank = 0;
-        dst_block = copy;
-        ndst = n;
-    }
+    const PackEnds e = pack_ends(L, copy);
+    const uint32_t src_rank = e.src_rank, src_block = e.src_block, dst_rank = e.dst_rank, dst_block = e.dst_block;
+    const uint32_t ndst = e.ndst;
     const uint64_t base = uint64_t(tile) * (kThreads * U) * sizeof(W);
     const char* src = static_cast<const char*>(L.in[src_rank]) + src_block * L.block_bytes + base;
     const uint64_t dst_off = dst_block * L.block_bytes + base;
@@ -100,18 +92,6 @@ __global__ void __launch_bounds__(kThreads) pack_kernel(const PackLaunch L) {
             }
         }
     }
-}
-
-// Decodes copy `copy` of a pack launch into its endpoints.
-struct PackEnds {
-    uint32_t src_rank, src_block, dst_rank, dst_block, ndst;
-};
-__device__ __forceinline__ PackEnds pack_ends(const PackLaunch& L, uint32_t copy) {
-    const uint32_t n = L.nranks;
-    if (L.mode == kPackAllToAll) return {copy / n, copy % n, copy % n, copy / n, 1};
-    if (L.mode == kPackScatter) return {L.root, copy, copy, 0, 1};
-    if (L.mode == kPackGather) return {copy, 0, L.root, copy, 1};
-    return {copy, 0, 0, copy, n};  // kPackAllGather: read once, write the block into every rank's buffer
 }
 
 // Group form of the pack kernel for long blocks of 16-byte accesses: a workgroup of kGroupWaves

@@ -585,6 +585,15 @@ Status plan_broadcast(Plan& plan, const void* send_root, void* const* recv, uint
     }
     const void* in[kMaxRanks] = {};
     in[root] = send_root;
+    // 16-byte aligned everywhere: one pack copy, read once and written into every rank's buffer
+    const void* recv_c[kMaxRanks] = {};
+    for (uint32_t r = 0; r < nranks; ++r) recv_c[r] = recv[r];
+    if (bytes && common_width(bytes, in, recv_c, nranks) == kVecBytes) {
+        const uint64_t before = plan.steps.size();
+        Status st = add_pack(plan, in, recv, nranks, bytes, kPackBroadcast, root, 1);
+        if (st == MEGRAY_OK && plan.steps.size() > before) plan.bytes_written += bytes * (nranks - 1);
+        return st;
+    }
     FoldBuilder copy(plan, in, recv, nranks, 1, nranks, elem_size, false);
     copy.add_run(0, 0, len, uint8_t(root), 1, 0);
     copy.finish();

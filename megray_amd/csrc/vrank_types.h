@@ -109,6 +109,7 @@ enum PackMode : uint32_t {
     kPackScatter = 1,   // copy b = i       : in[root] block i -> out[i] block 0
     kPackGather = 2,    // copy b = i       : in[i] block 0    -> out[root] block i
     kPackAllGather = 3, // copy b = i       : in[i] block 0    -> block i of EVERY out
+    kPackBroadcast = 4, // one copy         : in[root] block 0 -> block 0 of EVERY out
 };
 
 // One launch of the pack kernel: `ncopies` equally sized block copies whose endpoints follow
