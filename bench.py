@@ -27,8 +27,8 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the fold kernel on the headline workload, from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE runs scaled by the same counters on a plain copy of known size; the
 # summaries those figures come from are kept as text next to the kernel-trace summaries.
-# FETCH_SIZE counts 2 KiB per unit on this part (scale 1.99992), WRITE_SIZE 1 KiB (scale 0.99997).
-MEASURED_TRAFFIC_BYTES = {"all_reduce_f32_n8_2p28_fused": 17180153376}
+# FETCH_SIZE counts 2 KiB per unit on this part (scale 1.99990), WRITE_SIZE 1 KiB (scale 1.00000).
+MEASURED_TRAFFIC_BYTES = {"all_reduce_f32_n8_2p28_fused": 17179567119}
 
 
 def parse_args():
