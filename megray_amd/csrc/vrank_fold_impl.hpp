@@ -497,6 +497,9 @@ __device__ __forceinline__ void flat_tile_by_element(const FlatLaunch& L, uint32
     const uint64_t e_lo = uint64_t(tile) * TILE;
     const uint64_t e_hi = e_lo + TILE < L.count ? e_lo + TILE : L.count;
     for (uint32_t i = 0; i < L.nruns; ++i) {
+        // tile_lo = ceil(begin / TILE) and tile_hi >= floor(end / TILE): a run outside this window cannot
+        // touch the tile, and the two small tables are already in the scalar cache from the run lookup
+        if (L.tile_lo[i] > tile + 1 || L.tile_hi[i] < tile) continue;
         const uint64_t b = L.run[i].begin > e_lo ? L.run[i].begin : e_lo;
         const uint64_t e = L.run[i].end < e_hi ? L.run[i].end : e_hi;
         if (b >= e) continue;
@@ -520,6 +523,48 @@ __device__ __forceinline__ void flat_tile_by_element(const FlatLaunch& L, uint32
             }
             for (uint32_t m = 0; m < nout; ++m)
                 static_cast<T*>(L.out[rotate_rank(out_first, 1, m, K)])[el - shift] = r;
+        }
+    }
+}
+
+// A tile that lies inside the buffers but straddles run borders, its K input vectors already in
+// registers: folded once per run that touches it (uniform, registers only), and each lane stores
+// the elements that belong to that run.
+template <typename T, int OP, int K, bool TREE>
+__device__ __forceinline__ void flat_tile_across_runs(const FlatLaunch& L, uint32_t tile, uint32_t tid,
+                                                      const u32x4 (&x)[K]) {
+    constexpr uint32_t EPV = kVecBytes / sizeof(T);
+    constexpr uint32_t TILE = kThreads * EPV;
+    const uint64_t e_lo = uint64_t(tile) * TILE, e_hi = e_lo + TILE;
+    for (uint32_t i = 0; i < L.nruns; ++i) {
+        // tile_lo = ceil(begin / TILE) and tile_hi >= floor(end / TILE): a run outside this window cannot
+        // touch the tile, and the two small tables are already in the scalar cache from the run lookup
+        if (L.tile_lo[i] > tile + 1 || L.tile_hi[i] < tile) continue;
+        const uint64_t b = L.run[i].begin > e_lo ? L.run[i].begin : e_lo;
+        const uint64_t e = L.run[i].end < e_hi ? L.run[i].end : e_hi;
+        if (b >= e) continue;
+        VecOf<T> res;
+        if constexpr (TREE) {
+            res.raw = tree_from<T, OP, K>(x, L.run[i].start);
+        } else {
+            res.raw = fold_from<T, OP, K>(x, L.run[i].start, L.run[i].dir, L.new_wins_ties != 0);
+        }
+        const uint32_t out_first = L.run[i].out_first;
+        const uint64_t shift = uint64_t(L.run[i].out_shift);
+        // a lane's vector usually lies wholly inside or outside the run: one 16-byte store then
+        const uint64_t lane_lo = e_lo + uint64_t(tid) * EPV;
+        const bool inside = lane_lo >= b && lane_lo + EPV <= e;
+        const bool outside = lane_lo + EPV <= b || lane_lo >= e;
+        const bool vector_ok = shift % EPV == 0;  // flat launches shift by whole vectors
+        for (uint32_t m = 0; m < L.nout; ++m) {
+            T* dst = static_cast<T*>(L.out[rotate_rank(out_first, 1, m, K)]);
+            if (inside && vector_ok) {
+                store_vec(reinterpret_cast<char*>(dst + (lane_lo - shift)), res.raw);
+            } else if (!outside) {
+#pragma unroll
+                for (uint32_t k = 0; k < EPV; ++k)
+                    if (lane_lo + k >= b && lane_lo + k < e) dst[lane_lo + k - shift] = res.v[k];
+            }
         }
     }
 }
@@ -573,7 +618,10 @@ __global__ void __launch_bounds__(kThreads) fold_flat_kernel(const FlatLaunch L)
         return;
     }
 
-    flat_tile_by_element<T, OP, K, TREE>(L, tile, tid);
+    if (whole)
+        flat_tile_across_runs<T, OP, K, TREE>(L, tile, tid, x);
+    else
+        flat_tile_by_element<T, OP, K, TREE>(L, tile, tid);
 }
 
 // Group form of the flat fold for launches of many tiles.  A workgroup of kGroupWaves wavefronts
@@ -642,8 +690,14 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
             for (uint32_t m = 0; m < L.nout; ++m)
                 store_tile_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, K)]) + out_off, tid, res);
         }
+    } else if ((uint64_t(mine) + 1) * TILE <= L.count) {
+        // inside the buffers but across run borders: from the staged vectors, stored by this wavefront
+        u32x4 x[K];
+#pragma unroll
+        for (int r = 0; r < K; ++r) x[r] = stage[wave][r][tid];
+        flat_tile_across_runs<T, OP, K, TREE>(L, mine, tid, x);
     } else if (mine < L.total_tiles) {
-        flat_tile_by_element<T, OP, K, TREE>(L, mine, tid);  // reads and writes global memory itself
+        flat_tile_by_element<T, OP, K, TREE>(L, mine, tid);  // the buffers' last, partial tile
     }
     if (!exchange) return;
     if (tid == 0) folded[wave] = run >= 0 ? 1u : 0u;

@@ -225,7 +225,7 @@ def test_reduce_scatter(dtype):
     rng = np.random.default_rng(50 + dtype)
     size = orc.dtype_size(dtype)
     for nranks in (1, 2, 3, 8):
-        for recvlen in (0, 1, 5, 1024, 4099):
+        for recvlen in (0, 1, 5, 144, 1024, 4099):  # 144: aligned chunks whose borders fall inside tiles
             ins = [rand_array(dtype, nranks * recvlen, rng) for _ in range(nranks)]
             for op in OPS:
                 for order in ORDERS:
