@@ -358,7 +358,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.nout = L.nout;
                     run.new_wins_ties = L.new_wins_ties;
                     run.vector = (sg.flags & kSegVector) ? 1 : 0;
-                    run.waves = 1;
+                    run.waves = L.waves;
                     run.start = sg.start;
                     run.dir = sg.dir;
                     run.out_first = sg.out_first;

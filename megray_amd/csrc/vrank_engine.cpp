@@ -37,7 +37,8 @@ Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCal
         KernelCall call{nullptr, 0, kThreads, nullptr};
         switch (step.kind) {
             case Step::kFold:
-                call = {fold_kernel_for(step.fold, dtype, op), step.fold.total_tiles, kThreads, &step.fold};
+                call = {fold_kernel_for(step.fold, dtype, op), step.fold.total_tiles, kThreads * step.fold.waves,
+                        &step.fold};
                 break;
             case Step::kFlat:
                 if (step.flat.waves == kGroupWaves)

@@ -246,29 +246,117 @@ using AccFor = typename std::conditional<
 template <typename T, int OP>
 using TreeAccFor = AccFor<T, OP>;
 
-// K > 0: fold count known at compile time, all K loads of a lane are issued before the first use.
-// K == 0: fold count read from the launch, loads issued in groups of four.
-template <typename T, int OP, int K, int U>
-__global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
-    using A = typename Wide<T>::type;
-    constexpr uint32_t EPV = kVecBytes / sizeof(T);
-    const uint32_t tile = blockIdx.x;
-    // segment lookup: first_tile is ascending and padded with 0xffffffff, so the segment is the
-    // number of entries <= tile, minus one; eight entries per scalar load
+// The segment a workgroup works in, found from its tile number: first_tile is ascending and padded
+// with 0xffffffff, so the segment is the number of entries <= tile, minus one; eight entries per
+// scalar load.
+struct SegmentView {
+    uint64_t in_begin, out_begin, count;
+    uint32_t local_tile, start, out_first;
+    int dir;
+    bool vector;
+};
+__device__ __forceinline__ SegmentView find_segment(const FoldLaunch& L, uint32_t tile) {
     uint32_t s = 0;
     for (uint32_t base = 0; base < L.nseg; base += 8) {
 #pragma unroll
         for (uint32_t i = 0; i < 8; ++i) s += L.first_tile[base + i] <= tile ? 1u : 0u;
     }
     s -= 1;
-    const uint64_t in_begin = L.seg[s].in_begin;
-    const uint64_t out_begin = L.seg[s].out_begin;
-    const uint64_t count = L.seg[s].count;
-    const uint32_t local_tile = tile - L.first_tile[s];
-    const uint32_t start = L.seg[s].start;
-    const int dir = L.seg[s].dir;
-    const uint32_t out_first = L.seg[s].out_first;
-    const bool vector = (L.seg[s].flags & kSegVector) != 0;
+    SegmentView sv;
+    sv.in_begin = L.seg[s].in_begin;
+    sv.out_begin = L.seg[s].out_begin;
+    sv.count = L.seg[s].count;
+    sv.local_tile = tile - L.first_tile[s];
+    sv.start = L.seg[s].start;
+    sv.dir = L.seg[s].dir;
+    sv.out_first = L.seg[s].out_first;
+    sv.vector = (L.seg[s].flags & kSegVector) != 0;
+    return sv;
+}
+
+// Element tiles: run heads / tails and buffers that are not 16-byte aligned.  A lane takes
+// kElemsPerLane elements, a wavefront's lanes consecutive ones, four at a time in flight.
+template <typename T, int OP>
+__device__ __forceinline__ void fold_element_tile(const FoldLaunch& L, const SegmentView& sv, uint32_t nfold,
+                                                  uint32_t local_tile, uint32_t tid) {
+    using A = typename Wide<T>::type;
+    constexpr uint32_t G = 4;
+    const uint64_t in_begin = sv.in_begin, out_begin = sv.out_begin, count = sv.count;
+    const uint32_t start = sv.start, out_first = sv.out_first, nr = L.nranks, nout = L.nout;
+    const int dir = sv.dir;
+    const bool new_wins = L.new_wins_ties != 0;
+    const uint64_t ebase = uint64_t(local_tile) * (kThreads * kElemsPerLane);
+    for (uint32_t g = 0; g < kElemsPerLane; g += G) {
+        const uint64_t gbase = ebase + uint64_t(g) * kThreads;
+        if (gbase >= count) break;
+        const uint64_t left = count - gbase;
+        const uint64_t ie = in_begin + gbase + tid;
+        const uint64_t oe = out_begin + gbase + tid;
+        if (left >= uint64_t(G) * kThreads) {
+            A a[G];
+            const T* seed = static_cast<const T*>(L.in[start]) + ie;
+#pragma unroll
+            for (uint32_t q = 0; q < G; ++q) a[q] = static_cast<A>(seed[q * kThreads]);
+            for (uint32_t j = 1; j < nfold; ++j) {
+                const T* src = static_cast<const T*>(L.in[rotate_rank(start, dir, j, nr)]) + ie;
+                T x[G];
+#pragma unroll
+                for (uint32_t q = 0; q < G; ++q) x[q] = src[q * kThreads];
+#pragma unroll
+                for (uint32_t q = 0; q < G; ++q) a[q] = combine<OP, A>(a[q], static_cast<A>(x[q]), new_wins);
+            }
+            for (uint32_t m = 0; m < nout; ++m) {
+                T* dst = static_cast<T*>(L.out[rotate_rank(out_first, 1, m, nr)]) + oe;
+#pragma unroll
+                for (uint32_t q = 0; q < G; ++q) dst[q * kThreads] = static_cast<T>(a[q]);
+            }
+        } else {
+            for (uint32_t q = 0; q < G; ++q) {
+                const uint32_t e = q * kThreads + tid;
+                if (e >= left) break;
+                A a = static_cast<A>(static_cast<const T*>(L.in[start])[ie + q * kThreads]);
+                for (uint32_t j = 1; j < nfold; ++j)
+                    a = combine<OP, A>(
+                            a,
+                            static_cast<A>(static_cast<const T*>(L.in[rotate_rank(start, dir, j, nr)])[ie + q * kThreads]),
+                            new_wins);
+                const T r = static_cast<T>(a);
+                for (uint32_t m = 0; m < nout; ++m)
+                    static_cast<T*>(L.out[rotate_rank(out_first, 1, m, nr)])[oe + q * kThreads] = r;
+            }
+        }
+    }
+}
+
+// Up to kThreads vectors at vector index `vbase` of a segment, each lane folding one vector by itself
+// with plain global accesses: the incomplete last group of a segment's vector body.
+template <typename T, int OP>
+__device__ __forceinline__ void fold_vector_remainder(const FoldLaunch& L, const SegmentView& sv, uint32_t nfold,
+                                                      uint64_t vbase, uint64_t left, uint32_t tid) {
+    if (tid >= left) return;
+    const uint32_t nr = L.nranks;
+    const bool new_wins = L.new_wins_ties != 0;
+    const uint64_t in_off = sv.in_begin * sizeof(T) + (vbase + tid) * kVecBytes;
+    const uint64_t out_off = sv.out_begin * sizeof(T) + (vbase + tid) * kVecBytes;
+    AccFor<T, OP> a;
+    a.seed(load_vec(static_cast<const char*>(L.in[sv.start]) + in_off));
+    for (uint32_t j = 1; j < nfold; ++j)
+        a.fold(load_vec(static_cast<const char*>(L.in[rotate_rank(sv.start, sv.dir, j, nr)]) + in_off), new_wins);
+    const u32x4 r = a.finish();
+    for (uint32_t m = 0; m < L.nout; ++m)
+        store_vec(static_cast<char*>(L.out[rotate_rank(sv.out_first, 1, m, nr)]) + out_off, r);
+}
+
+// K > 0: fold count known at compile time, all K loads of a lane are issued before the first use.
+// K == 0: fold count read from the launch, loads issued in groups of four.
+template <typename T, int OP, int K, int U>
+__global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
+    constexpr uint32_t EPV = kVecBytes / sizeof(T);
+    const SegmentView sv = find_segment(L, blockIdx.x);
+    const uint64_t in_begin = sv.in_begin, out_begin = sv.out_begin, count = sv.count;
+    const uint32_t local_tile = sv.local_tile, start = sv.start, out_first = sv.out_first;
+    const int dir = sv.dir;
+    const bool vector = sv.vector;
     const uint32_t nr = L.nranks;
     const uint32_t nfold = K > 0 ? uint32_t(K) : L.nfold;
     const uint32_t nout = L.nout;
@@ -360,50 +448,96 @@ __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
             }
         }
     } else {
-        // element tiles: run heads / tails and buffers that are not 16-byte aligned.  A lane takes
-        // kElemsPerLane elements, a wavefront's lanes consecutive ones, four at a time in flight.
-        constexpr uint32_t G = 4;
-        const uint64_t ebase = uint64_t(local_tile) * (kThreads * kElemsPerLane);
-        for (uint32_t g = 0; g < kElemsPerLane; g += G) {
-            const uint64_t gbase = ebase + uint64_t(g) * kThreads;
-            if (gbase >= count) break;
-            const uint64_t left = count - gbase;
-            const uint64_t ie = in_begin + gbase + tid;
-            const uint64_t oe = out_begin + gbase + tid;
-            if (left >= uint64_t(G) * kThreads) {
-                A a[G];
-                const T* seed = static_cast<const T*>(L.in[start]) + ie;
+        fold_element_tile<T, OP>(L, sv, nfold, local_tile, tid);
+    }
+}
+
+// Group form of the segment fold for launches whose vector bodies are long (L.waves == kGroupWaves).
+// A workgroup of kGroupWaves wavefronts owns kGroupWaves groups of kThreads vectors of one segment
+// (1 KiB per buffer each) that lie kGroupStride such groups apart.  Wavefront w loads fold position
+// j of group (w + j) % kGroupWaves, the groups are exchanged through LDS, wavefront w folds group
+// w, and with several destinations the results are exchanged again so that wavefront w stores
+// destination m of group (w + m) % kGroupWaves.  With the fold count read from the launch (K == 0)
+// the inputs pass through LDS four at a time.  Element segments are the work of wavefront 0 alone.
+template <typename T, int OP, int K>
+__global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_kernel(const FoldLaunch L) {
+    constexpr uint32_t EPV = kVecBytes / sizeof(T);
+    constexpr uint32_t W = kGroupWaves;
+    constexpr uint32_t SK = K > 0 ? uint32_t(K) : 4u;  // inputs staged at a time
+    constexpr uint32_t kGroupBytes = kThreads * kVecBytes;
+    __shared__ u32x4 stage[W][SK][kThreads];
+    __shared__ u32x4 result[W][kThreads];
+    __shared__ uint32_t folded[W];
+    const SegmentView sv = find_segment(L, blockIdx.x);
+    const uint32_t tid = threadIdx.x % kThreads;
+    const uint32_t wave = uint32_t(__builtin_amdgcn_readfirstlane(int(threadIdx.x / kThreads)));
+    const uint32_t nr = L.nranks;
+    const uint32_t nfold = K > 0 ? uint32_t(K) : L.nfold;
+    const uint32_t nout = L.nout;
+    const bool new_wins = L.new_wins_ties != 0;
+    if (!sv.vector) {
+        if (wave == 0) fold_element_tile<T, OP>(L, sv, nfold, sv.local_tile, tid);
+        return;
+    }
+    const uint64_t nvec = sv.count / EPV;
+    const uint64_t whole_groups = nvec / kThreads;  // groups of kThreads vectors that are complete
+    const uint64_t first =
+            uint64_t(sv.local_tile / kGroupStride) * (W * kGroupStride) + sv.local_tile % kGroupStride;
+    const uint64_t mine = first + wave * kGroupStride;
+    const bool have = mine < whole_groups;
+    const uint64_t in_base = sv.in_begin * sizeof(T), out_base = sv.out_begin * sizeof(T);
+
+    AccFor<T, OP> acc;
+    if constexpr (K == 1) {
+        // a copy: nothing to skew on the load side
+        if (have) acc.seed(load_tile_vec(static_cast<const char*>(L.in[sv.start]) + in_base + mine * kGroupBytes, tid));
+    } else {
+        for (uint32_t j0 = 0; j0 < nfold; j0 += SK) {
+            u32x4 x[SK];
 #pragma unroll
-                for (uint32_t q = 0; q < G; ++q) a[q] = static_cast<A>(seed[q * kThreads]);
-                for (uint32_t j = 1; j < nfold; ++j) {
-                    const T* src = static_cast<const T*>(L.in[rotate_rank(start, dir, j, nr)]) + ie;
-                    T x[G];
+            for (uint32_t q = 0; q < SK; ++q) {
+                const uint64_t group = first + ((wave + q) % W) * kGroupStride;
+                if (j0 + q < nfold && group < whole_groups)
+                    x[q] = load_tile_vec(static_cast<const char*>(L.in[rotate_rank(sv.start, sv.dir, j0 + q, nr)]) +
+                                                 in_base + group * kGroupBytes,
+                                         tid);
+                else
+                    x[q] = u32x4{0u, 0u, 0u, 0u};
+            }
+            if (K == 0 && j0) __syncthreads();  // the previous four have been folded by everyone
 #pragma unroll
-                    for (uint32_t q = 0; q < G; ++q) x[q] = src[q * kThreads];
+            for (uint32_t q = 0; q < SK; ++q) stage[(wave + q) % W][q][tid] = x[q];
+            __syncthreads();
+            if (have) {
 #pragma unroll
-                    for (uint32_t q = 0; q < G; ++q) a[q] = combine<OP, A>(a[q], static_cast<A>(x[q]), new_wins);
-                }
-                for (uint32_t m = 0; m < nout; ++m) {
-                    T* dst = static_cast<T*>(L.out[rotate_rank(out_first, 1, m, nr)]) + oe;
-#pragma unroll
-                    for (uint32_t q = 0; q < G; ++q) dst[q * kThreads] = static_cast<T>(a[q]);
-                }
-            } else {
-                for (uint32_t q = 0; q < G; ++q) {
-                    const uint32_t e = q * kThreads + tid;
-                    if (e >= left) break;
-                    A a = static_cast<A>(static_cast<const T*>(L.in[start])[ie + q * kThreads]);
-                    for (uint32_t j = 1; j < nfold; ++j)
-                        a = combine<OP, A>(
-                                a,
-                                static_cast<A>(static_cast<const T*>(L.in[rotate_rank(start, dir, j, nr)])[ie + q * kThreads]),
-                                new_wins);
-                    const T r = static_cast<T>(a);
-                    for (uint32_t m = 0; m < nout; ++m)
-                        static_cast<T*>(L.out[rotate_rank(out_first, 1, m, nr)])[oe + q * kThreads] = r;
+                for (uint32_t q = 0; q < SK; ++q) {
+                    if (j0 + q >= nfold) break;
+                    if (j0 + q == 0)
+                        acc.seed(stage[wave][q][tid]);
+                    else
+                        acc.fold(stage[wave][q][tid], new_wins);
                 }
             }
         }
+    }
+    // the segment's incomplete last group of vectors belongs to whoever owns its index
+    if (mine == whole_groups && nvec % kThreads)
+        fold_vector_remainder<T, OP>(L, sv, nfold, mine * kThreads, nvec % kThreads, tid);
+
+    if (nout == 1) {
+        if (have)
+            store_tile_vec(static_cast<char*>(L.out[sv.out_first]) + out_base + mine * kGroupBytes, tid, acc.finish());
+        return;
+    }
+    if (have) result[wave][tid] = acc.finish();
+    if (tid == 0) folded[wave] = have ? 1u : 0u;
+    __syncthreads();
+    for (uint32_t m = 0; m < nout; ++m) {
+        const uint32_t k = (wave + m) % W;
+        if (folded[k])
+            store_tile_vec(static_cast<char*>(L.out[rotate_rank(sv.out_first, 1, m, nr)]) + out_base +
+                                   (first + uint64_t(k) * kGroupStride) * kGroupBytes,
+                           tid, result[k][tid]);
     }
 }
 
@@ -727,6 +861,18 @@ constexpr bool has_sum() {
 }
 
 template <typename T, int OP>
+FoldFn pick_fold_group(uint32_t nfold) {
+    switch (nfold) {
+        case 1: return fold_segment_group_kernel<T, OP, 1>;
+        case 2: return fold_segment_group_kernel<T, OP, 2>;
+        case 3: return fold_segment_group_kernel<T, OP, 3>;
+        case 4: return fold_segment_group_kernel<T, OP, 4>;
+        case 8: return fold_segment_group_kernel<T, OP, 8>;
+        default: return fold_segment_group_kernel<T, OP, 0>;
+    }
+}
+
+template <typename T, int OP>
 FoldFn pick_fold(uint32_t nfold) {
     switch (nfold) {
         case 2: return fold_kernel<T, OP, 2, fold_unroll(2)>;
@@ -770,10 +916,11 @@ FlatFn pick_flat(const FlatLaunch& L) {
 template <typename T>
 const void* fold_kernel_t(const FoldLaunch& L, int op) {
     FoldFn fn = nullptr;
-    if (op == kMax) fn = pick_fold<T, kMax>(L.nfold);
-    if (op == kMin) fn = pick_fold<T, kMin>(L.nfold);
+    const bool group = L.waves == kGroupWaves;
+    if (op == kMax) fn = group ? pick_fold_group<T, kMax>(L.nfold) : pick_fold<T, kMax>(L.nfold);
+    if (op == kMin) fn = group ? pick_fold_group<T, kMin>(L.nfold) : pick_fold<T, kMin>(L.nfold);
     if constexpr (has_sum<T>()) {
-        if (op == kSum) fn = pick_fold<T, kSum>(L.nfold);
+        if (op == kSum) fn = group ? pick_fold_group<T, kSum>(L.nfold) : pick_fold<T, kSum>(L.nfold);
     }
     return reinterpret_cast<const void*>(fn);
 }

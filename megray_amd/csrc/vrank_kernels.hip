@@ -146,6 +146,15 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
     }
 }
 
+FoldFn pick_copy_group(uint32_t elem_size) {
+    switch (elem_size) {
+        case 1: return fold_segment_group_kernel<uint8_t, kCopy, 1>;
+        case 2: return fold_segment_group_kernel<uint16_t, kCopy, 1>;
+        case 4: return fold_segment_group_kernel<uint32_t, kCopy, 1>;
+        default: return fold_segment_group_kernel<uint64_t, kCopy, 1>;
+    }
+}
+
 FoldFn pick_copy(uint32_t elem_size) {
     switch (elem_size) {
         case 1: return fold_kernel<uint8_t, kCopy, 1, fold_unroll(1)>;
@@ -184,7 +193,8 @@ const void* with_type(DType dtype, ReduceOp op, F&& call) {
 }  // namespace
 
 const void* fold_kernel_for(const FoldLaunch& L, DType dtype, ReduceOp op) {
-    if (L.nfold == 1) return reinterpret_cast<const void*>(pick_copy(L.elem_size));
+    if (L.nfold == 1)
+        return reinterpret_cast<const void*>(L.waves == kGroupWaves ? pick_copy_group(L.elem_size) : pick_copy(L.elem_size));
     return with_type(dtype, op, [&](auto tag, int k) { return fold_kernel_t<decltype(tag)>(L, k); });
 }
 

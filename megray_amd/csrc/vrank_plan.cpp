@@ -152,8 +152,14 @@ private:
     }
 
     void emit_general() {
-        open_launch();
         const uint64_t epv = kVecBytes / m_elem;
+        // long vector bodies take the group form (four wavefronts per workgroup)
+        uint64_t vector_elems = 0;
+        if (m_aligned)
+            for (const Run& r : m_runs)
+                if (r.in_begin % epv == r.out_begin % epv) vector_elems += r.count;
+        m_waves = vector_elems / (kThreads * epv) >= kGroupMinTiles ? kGroupWaves : 1;
+        open_launch();
         for (const Run& r : m_runs) {
             const bool vector = m_aligned && (r.in_begin % epv == r.out_begin % epv);
             uint64_t head = 0, body = 0;
@@ -191,6 +197,7 @@ private:
         m_launch.new_wins_ties = m_new_wins ? 1 : 0;
         m_launch.unroll = fold_unroll(m_nfold);
         m_launch.elem_size = m_elem;
+        m_launch.waves = m_waves;
     }
 
     void close_launch() {
@@ -212,7 +219,8 @@ private:
             }
             // a segment never takes more tiles than one launch's grid has left
             const uint64_t room = max_tiles - m_launch.total_tiles;
-            const uint64_t take = std::min(count, room * per_tile);
+            uint64_t take = std::min(count, room * per_tile);
+            if (take < count) take = take / per_tile * per_tile;  // cut between workgroups (room > 0: never empty)
             m_launch.first_tile[m_launch.nseg] = m_launch.total_tiles;
             FoldSegment& sg = m_launch.seg[m_launch.nseg++];
             sg.in_begin = in_begin;
@@ -222,7 +230,7 @@ private:
             sg.dir = r.dir;
             sg.out_first = r.out_first;
             sg.flags = flags;
-            m_launch.total_tiles += uint32_t((take + per_tile - 1) / per_tile);
+            m_launch.total_tiles += uint32_t(segment_tiles(m_launch, flags & kSegVector, take));
             in_begin += take;
             out_begin += take;
             count -= take;
@@ -238,6 +246,7 @@ private:
     uint32_t m_misalign = 0;
     uint64_t m_grid = kVecBytes;
     bool m_tree = false;
+    uint32_t m_waves = 1;
     std::vector<Run> m_runs;
     FoldLaunch m_launch;
 };

@@ -45,6 +45,7 @@ struct FoldLaunch {
     uint32_t new_wins_ties;  // float MAX/MIN: an equal / unordered compare keeps the newcomer
     uint32_t unroll;         // vectors (or elements) per lane per tile; fixes the tile size
     uint32_t elem_size;
+    uint32_t waves;          // wavefronts per workgroup: 1, or 4 for the group form (long vector bodies)
 };
 
 constexpr uint32_t kMaxFlatRuns = 48;  // 2N chunks cut again at N-1 rank borders
@@ -144,9 +145,24 @@ constexpr uint32_t pack_unroll() {
 constexpr uint32_t kElemsPerLane = 16;
 constexpr uint32_t kVecIters = 4;
 
+// Elements a workgroup takes of a vector or an element segment (group form: on average).
 inline uint64_t tile_elems(const FoldLaunch& L, bool vector) {
+    if (vector && L.waves == kGroupWaves) return uint64_t(kThreads) * kGroupWaves * (kVecBytes / L.elem_size);
     uint64_t per_lane = vector ? uint64_t(L.unroll) * kVecIters * (kVecBytes / L.elem_size) : kElemsPerLane;
     return uint64_t(kThreads) * per_lane;
+}
+
+// Workgroups a segment of `count` elements takes.  Group form: the vector body is cut into groups of
+// kThreads vectors, and workgroups come in blocks of kGroupStride that cover kGroupWaves * kGroupStride groups.
+inline uint64_t segment_tiles(const FoldLaunch& L, bool vector, uint64_t count) {
+    if (vector && L.waves == kGroupWaves) {
+        const uint64_t per_group = uint64_t(kThreads) * (kVecBytes / L.elem_size);
+        const uint64_t groups = (count + per_group - 1) / per_group;
+        const uint64_t span = uint64_t(kGroupWaves) * kGroupStride;
+        return (groups + span - 1) / span * kGroupStride;
+    }
+    const uint64_t per_tile = tile_elems(L, vector);
+    return (count + per_tile - 1) / per_tile;
 }
 
 }  // namespace vrank

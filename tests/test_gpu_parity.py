@@ -75,6 +75,49 @@ def test_all_reduce_group_form(dtype):
                                                  f"order={order} inplace={inplace} rank={r}")
 
 
+@pytest.mark.parametrize("dtype", REDUCE_TYPES)
+def test_segment_group_form(dtype):
+    """The general fold kernel with long vector bodies (4096 groups of 64 vectors and more) runs in its
+    group form: rank counts without a flat kernel (5 and 16: the fold count is read from the launch and
+    the inputs pass through LDS four at a time), buffers that share an offset from a 16-byte boundary,
+    and the ring replay's two-input steps and copies."""
+    size = orc.dtype_size(dtype)
+    rng = np.random.default_rng(277 + dtype)
+    cases = ((5, 0, mr.Schedule.FUSED, orc.SUM, orc.ORDER_UCX), (16, 0, mr.Schedule.FUSED, orc.MAX, orc.ORDER_SHM),
+             (8, max(size, 4), mr.Schedule.FUSED, orc.SUM, orc.ORDER_UCX), (3, 0, mr.Schedule.RING, orc.MIN, orc.ORDER_UCX),
+             (4, 0, mr.Schedule.RING, orc.SUM, orc.ORDER_UCX))
+    for nranks, offset, sched, op, order in cases:
+        if sched == mr.Schedule.RING and dtype == orc.FLOAT16:
+            continue  # the ring replay would round at every hop and is refused for FLOAT16
+        per_chunk = 4300 if sched == mr.Schedule.RING else 0  # ring steps work on one chunk per rank
+        tiles = max(4300, per_chunk * nranks)
+        length = tiles * 1024 // size + 7
+        ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+        d_in = [to_device(x, offset) for x in ins]
+        d_out = [empty_device(length * size, offset) for _ in range(nranks)]
+        runs, _, _ = mr.describe(mr.Collective.ALL_REDUCE, d_in, d_out, length, dtype, order, sched)
+        assert any(r["waves"] == 4 and r["vector"] == 1 for r in runs), "the segment group form is not what runs here"
+        want = orc.fold_all_reduce(ins, dtype, op, order)
+        got = run_all_reduce(ins, dtype, op, order, sched, offsets=[offset] * nranks)
+        for r in range(nranks):
+            assert_same(got[r], want[r], f"segment group form dtype={dtype} N={nranks} offset={offset} sched={sched} "
+                                         f"op={op} rank={r}")
+        if sched == mr.Schedule.FUSED:
+            got = run_all_reduce(ins, dtype, op, order, sched, offsets=[offset] * nranks, inplace=True)
+            for r in range(nranks):
+                assert_same(got[r], want[r], f"in-place segment group form dtype={dtype} N={nranks} rank={r}")
+    # a long copy with a common offset: broadcast through the general kernel's copy
+    nranks, offset = 5, max(size, 4)
+    length = 4200 * 1024 // size + 3
+    src = rand_array(dtype, length, rng)
+    d_src = to_device(src, offset)
+    d_out = [empty_device(length * size, offset) for _ in range(nranks)]
+    mr.broadcast(d_src, d_out, length, dtype, 2)
+    torch.cuda.synchronize()
+    for r in range(nranks):
+        assert_same(to_host(d_out[r], src.dtype), src, f"long unaligned broadcast dtype={dtype} rank={r}")
+
+
 def tree_expectation(ins, dtype, op, root):
     """reduce towards `root`: the oracle's literal replay of the binomial tree; FLOAT16 (which the
     reference cannot reduce) as the same tree in fp32 with one rounding."""
