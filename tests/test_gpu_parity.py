@@ -53,7 +53,7 @@ def test_all_reduce_fused_all_orders(dtype, nranks):
 
 @pytest.mark.parametrize("dtype", REDUCE_TYPES)
 def test_all_reduce_group_form(dtype):
-    """Launches of 4096 tiles and more take the group form of the flat kernel (four wavefronts per
+    """Launches of 512 tiles and more take the group form of the flat kernel (four wavefronts per
     workgroup, four tiles 32 tiles apart): ragged lengths, so that chunk borders fall inside tiles and the
     last group of tiles is incomplete; out of place and in place."""
     size = orc.dtype_size(dtype)
@@ -77,7 +77,7 @@ def test_all_reduce_group_form(dtype):
 
 @pytest.mark.parametrize("dtype", REDUCE_TYPES)
 def test_segment_group_form(dtype):
-    """The general fold kernel with long vector bodies (4096 groups of 64 vectors and more) runs in its
+    """The general fold kernel with long vector bodies (512 groups of 64 vectors and more) runs in its
     group form: rank counts without a flat kernel (5 and 16: the fold count is read from the launch and
     the inputs pass through LDS four at a time), buffers that share an offset from a 16-byte boundary,
     and the ring replay's two-input steps and copies."""
@@ -138,7 +138,7 @@ def tree_expectation(ins, dtype, op, root):
 
 @pytest.mark.parametrize("dtype", REDUCE_TYPES)
 def test_group_form_with_one_output(dtype):
-    """reduce_scatter, reduce towards a root and the two-phase all_reduce at 4096 tiles and more: the
+    """reduce_scatter, reduce towards a root and the two-phase all_reduce on long buffers: the
     group form in which every wavefront stores the tile it folded (shifted outputs, one destination)."""
     size = orc.dtype_size(dtype)
     rng = np.random.default_rng(177 + dtype)
@@ -305,7 +305,7 @@ def test_pack_collectives(dtype):
 
 @pytest.mark.parametrize("dtype", [orc.UINT8, orc.FLOAT16, orc.INT64])
 def test_pack_collectives_group_form(dtype):
-    """Blocks of 1024 tiles and more go through the group form of the pack kernel (four wavefronts, four
+    """Blocks of 128 tiles and more go through the group form of the pack kernel (four wavefronts, four
     tiles per workgroup); the block ends in a partial tile."""
     rng = np.random.default_rng(190 + dtype)
     size = orc.dtype_size(dtype)

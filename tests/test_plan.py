@@ -253,8 +253,8 @@ def test_full_size_plan_shapes():
     assert rs and all(r["waves"] == 4 and r["vector"] == 2 for r in rs)
     tree, _, _ = mr.describe(mr.Collective.REDUCE, sp, rp, 1 << 22, orc.FLOAT32, root=3)
     assert tree and all(r["waves"] == 4 and r["dir"] == 0 for r in tree)
-    for coll, count in ((mr.Collective.ALL_REDUCE, 1 << 19), (mr.Collective.REDUCE_SCATTER, 1 << 16),
-                        (mr.Collective.REDUCE, 1 << 19)):
+    for coll, count in ((mr.Collective.ALL_REDUCE, 1 << 15), (mr.Collective.REDUCE_SCATTER, 1 << 12),
+                        (mr.Collective.REDUCE, 1 << 15)):
         small, _, _ = mr.describe(coll, sp, rp, count, orc.FLOAT32)
         assert small and all(r["waves"] == 1 for r in small)
     # a buffer far beyond one launch's grid is split into several launches, nothing lost
