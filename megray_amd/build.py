@@ -1,6 +1,8 @@
 """Builds libmegray_vrank.so (the gfx950 kernels, the planner, the MegRay C++ API and the C ABI)
 with hipcc, in tree.  Run as ``python -m megray_amd.build``."""
+import json
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -10,6 +12,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(HERE, "libmegray_vrank.so")
+RESOURCES_PATH = os.path.join(HERE, "kernel_resources.json")  # registers, scratch, LDS of every kernel built
 
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 HIPCC = os.environ.get("HIPCC", os.path.join(ROCM, "bin", "hipcc"))
@@ -36,12 +39,30 @@ def _compile(src):
     obj = os.path.join(OBJ_DIR, os.path.basename(src) + ".o")
     cmd = [HIPCC] + COMMON_FLAGS
     if src.endswith(".hip"):
-        cmd += ["-x", "hip"] + DEVICE_FLAGS
+        cmd += ["-x", "hip", "-Rpass-analysis=kernel-resource-usage"] + DEVICE_FLAGS
     else:  # host-only translation units: plain C++ against the HIP runtime API headers
         cmd += ["-x", "c++", "-D__HIP_PLATFORM_AMD__=1", "-pthread", f"-I{ROCM}/include"]
     cmd += ["-c", src, "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     return src, obj, proc
+
+
+def _kernel_resources(stderr):
+    """{kernel symbol: {"vgprs", "agprs", "sgprs", "scratch", "lds", "occupancy"}} from the compiler's
+    kernel-resource-usage remarks."""
+    out, cur = {}, None
+    keys = {"VGPRs": "vgprs", "AGPRs": "agprs", "TotalSGPRs": "sgprs", "ScratchSize [bytes/lane]": "scratch",
+            "LDS Size [bytes/block]": "lds", "Occupancy [waves/SIMD]": "occupancy"}
+    for line in stderr.splitlines():
+        m = re.search(r"remark: (?:\s*)([^:]+): (\S+) \[-Rpass-analysis=kernel-resource-usage\]", line)
+        if not m:
+            continue
+        key, value = m.group(1).strip(), m.group(2)
+        if key == "Function Name":
+            cur = out.setdefault(value, {})
+        elif cur is not None and key in keys:
+            cur[keys[key]] = int(value)
+    return out
 
 
 def build_library(verbose=True):
@@ -51,14 +72,19 @@ def build_library(verbose=True):
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
         results = list(pool.map(_compile, srcs))
     objs = []
+    resources = {}
     for src, obj, proc in results:
         noise = "'-packed-fp32-ops' is not a recognized feature"
-        err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)
+        resources.update(_kernel_resources(proc.stderr))
+        err = "\n".join(l for l in proc.stderr.splitlines()
+                        if noise not in l and "[-Rpass-analysis=kernel-resource-usage]" not in l)
         if proc.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src}:\n{proc.stdout}\n{proc.stderr}")
         if verbose and err.strip():
             print(err, file=sys.stderr)
         objs.append(obj)
+    with open(RESOURCES_PATH, "w") as f:
+        json.dump(resources, f, indent=1, sort_keys=True)
     link = [HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", LIB_PATH] + objs + ["-lpthread"]
     proc = subprocess.run(link, capture_output=True, text=True)
     if proc.returncode != 0:

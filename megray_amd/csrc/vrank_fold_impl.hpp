@@ -661,15 +661,21 @@ __device__ __forceinline__ void flat_tile_by_element(const FlatLaunch& L, uint32
     }
 }
 
-// A tile that lies inside the buffers but straddles run borders, its K input vectors already in
-// registers: folded once per run that touches it (uniform, registers only), and each lane stores
-// the elements that belong to that run.
+// A tile that lies inside the buffers but straddles run borders, its K input vectors staged in LDS
+// as staged[r][lane]: folded once per run that touches it, the inputs fetched from LDS in the run's
+// order (a rolled loop: the fold order is data here, not code, which keeps this rare path small in
+// code and registers); a lane whose vector lies wholly inside the run stores it with one 16-byte
+// store per destination.  The few lanes whose vector is cut by a run border (chunk lengths need not
+// be multiples of a vector) go element by element from global memory.
 template <typename T, int OP, int K, bool TREE>
 __device__ __forceinline__ void flat_tile_across_runs(const FlatLaunch& L, uint32_t tile, uint32_t tid,
-                                                      const u32x4 (&x)[K]) {
+                                                      const u32x4 (*staged)[kThreads]) {
+    using A = typename Wide<T>::type;
     constexpr uint32_t EPV = kVecBytes / sizeof(T);
     constexpr uint32_t TILE = kThreads * EPV;
     const uint64_t e_lo = uint64_t(tile) * TILE, e_hi = e_lo + TILE;
+    const uint64_t lane_lo = e_lo + uint64_t(tid) * EPV;
+    const bool new_wins = L.new_wins_ties != 0;
     for (uint32_t i = 0; i < L.nruns; ++i) {
         // tile_lo = ceil(begin / TILE) and tile_hi >= floor(end / TILE): a run outside this window cannot
         // touch the tile, and the two small tables are already in the scalar cache from the run lookup
@@ -677,27 +683,51 @@ __device__ __forceinline__ void flat_tile_across_runs(const FlatLaunch& L, uint3
         const uint64_t b = L.run[i].begin > e_lo ? L.run[i].begin : e_lo;
         const uint64_t e = L.run[i].end < e_hi ? L.run[i].end : e_hi;
         if (b >= e) continue;
-        VecOf<T> res;
-        if constexpr (TREE) {
-            res.raw = tree_from<T, OP, K>(x, L.run[i].start);
-        } else {
-            res.raw = fold_from<T, OP, K>(x, L.run[i].start, L.run[i].dir, L.new_wins_ties != 0);
-        }
+        const uint32_t start = L.run[i].start;
+        const int dir = L.run[i].dir;
         const uint32_t out_first = L.run[i].out_first;
-        const uint64_t shift = uint64_t(L.run[i].out_shift);
-        // a lane's vector usually lies wholly inside or outside the run: one 16-byte store then
-        const uint64_t lane_lo = e_lo + uint64_t(tid) * EPV;
+        const uint64_t shift = uint64_t(L.run[i].out_shift);  // a whole number of vectors in a flat launch
         const bool inside = lane_lo >= b && lane_lo + EPV <= e;
-        const bool outside = lane_lo + EPV <= b || lane_lo >= e;
-        const bool vector_ok = shift % EPV == 0;  // flat launches shift by whole vectors
-        for (uint32_t m = 0; m < L.nout; ++m) {
-            T* dst = static_cast<T*>(L.out[rotate_rank(out_first, 1, m, K)]);
-            if (inside && vector_ok) {
-                store_vec(reinterpret_cast<char*>(dst + (lane_lo - shift)), res.raw);
-            } else if (!outside) {
+        const bool cut = !inside && lane_lo < e && lane_lo + EPV > b;
+        if (inside) {
+            u32x4 res;
+            if constexpr (TREE) {
+                u32x4 x[K];
 #pragma unroll
-                for (uint32_t k = 0; k < EPV; ++k)
-                    if (lane_lo + k >= b && lane_lo + k < e) dst[lane_lo + k - shift] = res.v[k];
+                for (int r = 0; r < K; ++r) x[r] = staged[r][tid];
+                res = tree_from<T, OP, K>(x, start);
+            } else {
+                AccFor<T, OP> acc;
+                acc.seed(staged[start][tid]);
+#pragma unroll 1
+                for (uint32_t j = 1; j < uint32_t(K); ++j) acc.fold(staged[rotate_rank(start, dir, j, K)][tid], new_wins);
+                res = acc.finish();
+            }
+#pragma unroll 1
+            for (uint32_t m = 0; m < L.nout; ++m) {
+                T* dst = static_cast<T*>(L.out[rotate_rank(out_first, 1, m, K)]);
+                store_vec(reinterpret_cast<char*>(dst + (lane_lo - shift)), res);
+            }
+        } else if (cut) {
+#pragma unroll 1
+            for (uint32_t k = 0; k < EPV; ++k) {
+                const uint64_t el = lane_lo + k;
+                if (el < b || el >= e) continue;
+                T r;
+                if constexpr (TREE) {
+                    r = tree_element<T, OP, K>(L, K, start, el);
+                } else {
+                    A a = static_cast<A>(static_cast<const T*>(L.in[start])[el]);
+#pragma unroll 1
+                    for (uint32_t j = 1; j < uint32_t(K); ++j)
+                        a = combine<OP, A>(
+                                a, static_cast<A>(static_cast<const T*>(L.in[rotate_rank(start, dir, j, K)])[el]),
+                                new_wins);
+                    r = static_cast<T>(a);
+                }
+#pragma unroll 1
+                for (uint32_t m = 0; m < L.nout; ++m)
+                    static_cast<T*>(L.out[rotate_rank(out_first, 1, m, K)])[el - shift] = r;
             }
         }
     }
@@ -752,10 +782,15 @@ __global__ void __launch_bounds__(kThreads) fold_flat_kernel(const FlatLaunch L)
         return;
     }
 
-    if (whole)
-        flat_tile_across_runs<T, OP, K, TREE>(L, tile, tid, x);
-    else
+    if (whole) {
+        // each lane parks its vectors in LDS, where the runs' fold orders can index them
+        __shared__ u32x4 parked[K][kThreads];
+#pragma unroll
+        for (int r = 0; r < K; ++r) parked[r][tid] = x[r];
+        flat_tile_across_runs<T, OP, K, TREE>(L, tile, tid, parked);
+    } else {
         flat_tile_by_element<T, OP, K, TREE>(L, tile, tid);
+    }
 }
 
 // Group form of the flat fold for launches of many tiles.  A workgroup of kGroupWaves wavefronts
@@ -826,10 +861,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
         }
     } else if ((uint64_t(mine) + 1) * TILE <= L.count) {
         // inside the buffers but across run borders: from the staged vectors, stored by this wavefront
-        u32x4 x[K];
-#pragma unroll
-        for (int r = 0; r < K; ++r) x[r] = stage[wave][r][tid];
-        flat_tile_across_runs<T, OP, K, TREE>(L, mine, tid, x);
+        flat_tile_across_runs<T, OP, K, TREE>(L, mine, tid, stage[wave]);
     } else if (mine < L.total_tiles) {
         flat_tile_by_element<T, OP, K, TREE>(L, mine, tid);  // the buffers' last, partial tile
     }

@@ -92,3 +92,22 @@ def test_product_never_imports_the_oracle():
             if name.endswith((".py", ".cpp", ".h", ".hip")):
                 text = open(os.path.join(dirpath, name)).read()
                 assert "import oracle" not in text and "megray_oracle" not in text, name
+
+
+def test_no_kernel_spills_or_hogs_registers():
+    """The build records every kernel's resources.  A kernel that needs scratch memory (register spills,
+    run-time indexed arrays) or more than 128 vector registers halves the wavefronts a CU can hold and
+    has cost a third of the throughput before; the kernels are written so that none does."""
+    import json
+    import os
+
+    from megray_amd import build
+    if not os.path.exists(build.RESOURCES_PATH):
+        pytest.skip("the library was not built in this tree (kernel_resources.json is a build product)")
+    with open(build.RESOURCES_PATH) as f:
+        kernels = json.load(f)
+    assert len(kernels) > 100
+    for name, res in kernels.items():
+        assert res["scratch"] == 0, f"{name} uses {res['scratch']} bytes of scratch per lane"
+        assert res["vgprs"] <= 128, f"{name} uses {res['vgprs']} vector registers"
+        assert res["lds"] <= 40 * 1024, f"{name} uses {res['lds']} bytes of LDS"
