@@ -814,48 +814,53 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
     // wavefront index, made known to be uniform so that it selects pointers in scalar registers
     const uint32_t wave = uint32_t(__builtin_amdgcn_readfirstlane(int(threadIdx.x / kThreads)));
     const uint32_t first = (blockIdx.x / kGroupStride) * (W * kGroupStride) + blockIdx.x % kGroupStride;
-
-    // tile k of the group is first + k * kGroupStride; it is loaded if it lies inside the buffers
-    {
-        u32x4 x[K];
-#pragma unroll
-        for (int r = 0; r < K; ++r) {
-            const uint64_t tile = uint64_t(first) + ((wave + r) % W) * kGroupStride;
-            if ((tile + 1) * TILE <= L.count)
-                x[r] = load_tile_vec(static_cast<const char*>(L.in[r]) + tile * (kThreads * kVecBytes), tid);
-            else
-                x[r] = u32x4{0u, 0u, 0u, 0u};  // never folded: such a tile goes element by element
-        }
-#pragma unroll
-        for (int r = 0; r < K; ++r) stage[(wave + r) % W][r][tid] = x[r];
-    }
-    __syncthreads();
-
     const uint32_t mine = first + wave * kGroupStride;
     const bool exchange = L.exchange != 0;
+
+    // tile k of the group is first + k * kGroupStride; it is loaded if it lies inside the buffers
+    u32x4 x[K];
+#pragma unroll
+    for (int r = 0; r < K; ++r) {
+        const uint64_t tile = uint64_t(first) + ((wave + r) % W) * kGroupStride;
+        if ((tile + 1) * TILE <= L.count)
+            x[r] = load_tile_vec(static_cast<const char*>(L.in[r]) + tile * (kThreads * kVecBytes), tid);
+        else
+            x[r] = u32x4{0u, 0u, 0u, 0u};  // never folded: such a tile goes element by element
+    }
+    // while the loads are in flight: which run does this wavefront's own tile lie in?
     int run = -1;
     for (uint32_t base = 0; base < L.nruns; base += 8) {
 #pragma unroll
         for (uint32_t i = 0; i < 8; ++i)
             if (mine >= L.tile_lo[base + i] && mine < L.tile_hi[base + i]) run = int(base + i);
     }
+    uint32_t start = 0, out_first = 0;
+    int dir = 1;
+    int64_t out_shift = 0;
+    if (run >= 0) {
+        start = L.run[run].start;
+        dir = L.run[run].dir;
+        out_first = L.run[run].out_first;
+        out_shift = L.run[run].out_shift;
+    }
+#pragma unroll
+    for (int r = 0; r < K; ++r) stage[(wave + r) % W][r][tid] = x[r];
+    __syncthreads();
+
     if (run >= 0) {
         // the whole tile shares one fold order (and lies inside the buffers)
-        u32x4 x[K];
 #pragma unroll
         for (int r = 0; r < K; ++r) x[r] = stage[wave][r][tid];
         u32x4 res;
         if constexpr (TREE) {
-            res = tree_from<T, OP, K>(x, L.run[run].start);
+            res = tree_from<T, OP, K>(x, start);
         } else {
-            res = fold_from<T, OP, K>(x, L.run[run].start, L.run[run].dir, L.new_wins_ties != 0);
+            res = fold_from<T, OP, K>(x, start, dir, L.new_wins_ties != 0);
         }
         if (exchange) {
             result[wave][tid] = res;
         } else {
-            const uint64_t out_off =
-                    uint64_t(mine) * (kThreads * kVecBytes) - uint64_t(L.run[run].out_shift) * sizeof(T);
-            const uint32_t out_first = L.run[run].out_first;
+            const uint64_t out_off = uint64_t(mine) * (kThreads * kVecBytes) - uint64_t(out_shift) * sizeof(T);
             for (uint32_t m = 0; m < L.nout; ++m)
                 store_tile_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, K)]) + out_off, tid, res);
         }
