@@ -65,6 +65,24 @@ def _kernel_resources(stderr):
     return out
 
 
+def _diagnostics(stderr, noise):
+    """The compiler's output without the resource-usage remarks (and the source excerpts under them)."""
+    kept, in_remark = [], False
+    for line in stderr.splitlines():
+        if "[-Rpass-analysis=kernel-resource-usage]" in line:
+            in_remark = True
+            continue
+        if in_remark and (re.match(r"^\s*\d*\s*\|", line) or line.startswith("In file included from")):
+            continue
+        in_remark = False
+        if noise in line or re.match(r"^\d+ warnings? generated", line):
+            continue
+        kept.append(line)
+    # "In file included from" headers whose remark followed them
+    return "\n".join(l for i, l in enumerate(kept)
+                     if not (l.startswith("In file included from") and (i + 1 == len(kept) or kept[i + 1].startswith("In file included from") or not kept[i + 1].strip())))
+
+
 def build_library(verbose=True):
     """Compile every source and link the shared library.  Always recompiles."""
     os.makedirs(OBJ_DIR, exist_ok=True)
@@ -76,8 +94,7 @@ def build_library(verbose=True):
     for src, obj, proc in results:
         noise = "'-packed-fp32-ops' is not a recognized feature"
         resources.update(_kernel_resources(proc.stderr))
-        err = "\n".join(l for l in proc.stderr.splitlines()
-                        if noise not in l and "[-Rpass-analysis=kernel-resource-usage]" not in l)
+        err = _diagnostics(proc.stderr, noise)
         if proc.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src}:\n{proc.stdout}\n{proc.stderr}")
         if verbose and err.strip():
