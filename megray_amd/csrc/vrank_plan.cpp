@@ -262,6 +262,29 @@ Status check_elem(uint32_t elem_size) {
     return MEGRAY_OK;
 }
 
+// A length whose byte count, times every rank, still fits 64 bits with room to spare.
+Status check_len(uint64_t len) {
+    if (len > (uint64_t(1) << 48)) return invalid("length beyond 2^48 elements");
+    return MEGRAY_OK;
+}
+
+// Every buffer a launch will touch must be there: a null pointer would fault on the device.
+Status check_present(const void* const* ptrs, uint32_t n, uint64_t bytes, const char* what) {
+    if (!bytes) return MEGRAY_OK;
+    for (uint32_t r = 0; r < n; ++r)
+        if (!ptrs[r]) return invalid(what);
+    return MEGRAY_OK;
+}
+Status check_present(void* const* ptrs, uint32_t n, uint64_t bytes, const char* what) {
+    if (!bytes) return MEGRAY_OK;
+    for (uint32_t r = 0; r < n; ++r)
+        if (!ptrs[r]) return invalid(what);
+    return MEGRAY_OK;
+}
+Status check_present(const void* ptr, uint64_t bytes, const char* what) {
+    return (bytes && !ptr) ? invalid(what) : MEGRAY_OK;
+}
+
 // Buffers of different ranks must not overlap.  A rank's own receive buffer may overlap its send
 // buffer only at the one offset where every element keeps its address (`recv == send + shift`).
 Status check_overlap(const void* const* send, uint64_t send_bytes, void* const* recv, uint64_t recv_bytes,
@@ -350,6 +373,9 @@ Status plan_all_reduce(Plan& plan, const void* const* send, void* const* recv, u
     if (order < 0 || order >= kOrderCount) return invalid("unknown fold order");
     if (sched < 0 || sched >= kSchedCount) return invalid("unknown schedule");
     if (sched == kSchedRing && order != kOrderUcx) return invalid("the ring schedule exists for the ucx order only");
+    PLAN_TRY(check_len(len));
+    PLAN_TRY(check_present(send, nranks, len, "a send buffer is null"));
+    PLAN_TRY(check_present(recv, nranks, len, "a receive buffer is null"));
     PLAN_TRY(check_overlap(send, len * elem_size, recv, len * elem_size, nranks, 0));
     const uint32_t nchunks = order_chunks(order, nranks);
     uint64_t sizes[kMaxChunks], offs[kMaxChunks];
@@ -428,6 +454,9 @@ Status plan_reduce_scatter(Plan& plan, const void* const* send, void* const* rec
     PLAN_TRY(check_elem(elem_size));
     if (order < 0 || order >= kOrderCount) return invalid("unknown fold order");
     if (sched != kSchedFused) return invalid("reduce_scatter has the fused schedule only");
+    PLAN_TRY(check_len(recvlen));
+    PLAN_TRY(check_present(send, nranks, recvlen, "a send buffer is null"));
+    PLAN_TRY(check_present(recv, nranks, recvlen, "a receive buffer is null"));
     const uint64_t total = recvlen * nranks;
     PLAN_TRY(check_overlap(send, total * elem_size, recv, recvlen * elem_size, nranks,
                                int64_t(recvlen * elem_size)));
@@ -462,6 +491,9 @@ Status plan_all_gather(Plan& plan, const void* const* send, void* const* recv, u
                        uint64_t sendlen, uint32_t elem_size) {
     PLAN_TRY(check_ranks(nranks));
     PLAN_TRY(check_elem(elem_size));
+    PLAN_TRY(check_len(sendlen));
+    PLAN_TRY(check_present(send, nranks, sendlen, "a send buffer is null"));
+    PLAN_TRY(check_present(recv, nranks, sendlen, "a receive buffer is null"));
     // in place: rank r's contribution already sits in its slot, send[r] == recv[r] + r * sendlen
     for (uint32_t a = 0; a < nranks; ++a) {
         for (uint32_t b = a + 1; b < nranks; ++b)
@@ -532,6 +564,9 @@ Status plan_all_to_all(Plan& plan, const void* const* send, void* const* recv, u
                        uint64_t len, uint32_t elem_size) {
     PLAN_TRY(check_ranks(nranks));
     PLAN_TRY(check_elem(elem_size));
+    PLAN_TRY(check_len(len));
+    PLAN_TRY(check_present(send, nranks, len, "a send buffer is null"));
+    PLAN_TRY(check_present(recv, nranks, len, "a receive buffer is null"));
     const uint64_t bytes = len * nranks * elem_size;
     for (uint32_t a = 0; a < nranks; ++a) {
         for (uint32_t b = 0; b < nranks; ++b) {
@@ -548,6 +583,9 @@ Status plan_scatter(Plan& plan, const void* send_root, void* const* recv, uint32
     PLAN_TRY(check_elem(elem_size));
     if (root >= nranks) return invalid("root out of range");
     const uint64_t block = recvlen * elem_size;
+    PLAN_TRY(check_len(recvlen));
+    PLAN_TRY(check_present(send_root, recvlen, "the root's send buffer is null"));
+    PLAN_TRY(check_present(recv, nranks, recvlen, "a receive buffer is null"));
     for (uint32_t a = 0; a < nranks; ++a) {
         for (uint32_t b = a + 1; b < nranks; ++b)
             if (overlaps(recv[a], block, recv[b], block)) return invalid("receive buffers of two ranks overlap");
@@ -568,6 +606,9 @@ Status plan_gather(Plan& plan, const void* const* send, void* recv_root, uint32_
     PLAN_TRY(check_elem(elem_size));
     if (root >= nranks) return invalid("root out of range");
     const uint64_t block = sendlen * elem_size;
+    PLAN_TRY(check_len(sendlen));
+    PLAN_TRY(check_present(send, nranks, sendlen, "a send buffer is null"));
+    PLAN_TRY(check_present(recv_root, sendlen, "the root's receive buffer is null"));
     for (uint32_t b = 0; b < nranks; ++b) {
         if (overlaps(recv_root, block * nranks, send[b], block)) {
             const bool in_place = b == root && static_cast<const char*>(send[b]) ==
@@ -586,6 +627,9 @@ Status plan_broadcast(Plan& plan, const void* send_root, void* const* recv, uint
     PLAN_TRY(check_elem(elem_size));
     if (root >= nranks) return invalid("root out of range");
     const uint64_t bytes = len * elem_size;
+    PLAN_TRY(check_len(len));
+    PLAN_TRY(check_present(send_root, len, "the root's send buffer is null"));
+    PLAN_TRY(check_present(recv, nranks, len, "a receive buffer is null"));
     for (uint32_t a = 0; a < nranks; ++a) {
         for (uint32_t b = a + 1; b < nranks; ++b)
             if (overlaps(recv[a], bytes, recv[b], bytes)) return invalid("receive buffers of two ranks overlap");
@@ -616,6 +660,9 @@ Status plan_reduce(Plan& plan, const void* const* send, void* recv_root, uint32_
     if (order < 0 || order >= kOrderCount) return invalid("unknown fold order");
     if (root >= nranks) return invalid("root out of range");
     const uint64_t bytes = len * elem_size;
+    PLAN_TRY(check_len(len));
+    PLAN_TRY(check_present(send, nranks, len, "a send buffer is null"));
+    PLAN_TRY(check_present(recv_root, len, "the root's receive buffer is null"));
     for (uint32_t b = 0; b < nranks; ++b)
         if (overlaps(recv_root, bytes, send[b], bytes) && !(b == root && recv_root == send[b]))
             return invalid("the root's receive buffer overlaps a send buffer out of place");
@@ -660,6 +707,8 @@ Status plan_reduce(Plan& plan, const void* const* send, void* recv_root, uint32_
 
 Status plan_reduce2(Plan& plan, const void* i0, const void* i1, void* o, uint64_t len, uint32_t elem_size) {
     PLAN_TRY(check_elem(elem_size));
+    PLAN_TRY(check_len(len));
+    if (len && (!i0 || !i1 || !o)) return invalid("a buffer is null");
     const uint64_t bytes = len * elem_size;
     if ((overlaps(o, bytes, i0, bytes) && o != i0) || (overlaps(o, bytes, i1, bytes) && o != i1))
         return invalid("the output overlaps an input out of place");

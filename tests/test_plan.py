@@ -279,6 +279,16 @@ def test_planner_rejects_what_it_cannot_honour():
         mr.describe(mr.Collective.ALL_REDUCE, sp, rp, 100, orc.CHAR)
     with pytest.raises(mr.MegRayError, match="root"):
         mr.describe(mr.Collective.SCATTER, sp, rp, 100, orc.FLOAT32, root=4)
+    # a null buffer would fault on the device; a zero-length call touches nothing and may pass them
+    with pytest.raises(mr.MegRayError, match="send buffer is null"):
+        mr.describe(mr.Collective.ALL_REDUCE, [sp[0], 0, sp[2], sp[3]], rp, 100, orc.FLOAT32)
+    with pytest.raises(mr.MegRayError, match="receive buffer is null"):
+        mr.describe(mr.Collective.ALL_GATHER, sp, [rp[0], rp[1], 0, rp[3]], 100, orc.FLOAT32)
+    with pytest.raises(mr.MegRayError, match="root's send buffer is null"):
+        mr.describe(mr.Collective.BROADCAST, [0, 0, 0, 0], rp, 100, orc.FLOAT32, root=2)
+    mr.describe(mr.Collective.ALL_REDUCE, [0] * 4, [0] * 4, 0, orc.FLOAT32)
+    with pytest.raises(mr.MegRayError, match="beyond 2.48 elements"):
+        mr.describe(mr.Collective.ALL_REDUCE, sp, rp, 1 << 50, orc.INT8)
     # in place is fine where every element keeps its address
     mr.describe(mr.Collective.ALL_REDUCE, sp, sp, 100, orc.FLOAT32)
     mr.describe(mr.Collective.REDUCE_SCATTER, sp, [sp[r] + r * 400 for r in range(4)], 100, orc.FLOAT32)
