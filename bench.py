@@ -28,7 +28,7 @@ HBM_PEAK_GBPS = 8000.0
 # FETCH_SIZE / WRITE_SIZE runs scaled by the same counters on a plain copy of known size; the
 # summaries those figures come from are kept as text next to the kernel-trace summaries.
 # FETCH_SIZE counts 2 KiB per unit on this part (scale 1.99990), WRITE_SIZE 1 KiB (scale 1.00000).
-MEASURED_TRAFFIC_BYTES = {"all_reduce_f32_n8_2p28_fused": 17179567119}
+MEASURED_TRAFFIC_BYTES = {"all_reduce_f32_n8_2p28_fused": 17179591511}
 
 
 def parse_args():
