@@ -347,105 +347,63 @@ __device__ __forceinline__ void fold_vector_remainder(const FoldLaunch& L, const
         store_vec(static_cast<char*>(L.out[rotate_rank(sv.out_first, 1, m, nr)]) + out_off, r);
 }
 
+// One wavefront per tile, for short launches.
 // K > 0: fold count known at compile time, all K loads of a lane are issued before the first use.
 // K == 0: fold count read from the launch, loads issued in groups of four.
-template <typename T, int OP, int K, int U>
+template <typename T, int OP, int K>
 __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
     constexpr uint32_t EPV = kVecBytes / sizeof(T);
     const SegmentView sv = find_segment(L, blockIdx.x);
-    const uint64_t in_begin = sv.in_begin, out_begin = sv.out_begin, count = sv.count;
     const uint32_t local_tile = sv.local_tile, start = sv.start, out_first = sv.out_first;
     const int dir = sv.dir;
-    const bool vector = sv.vector;
     const uint32_t nr = L.nranks;
     const uint32_t nfold = K > 0 ? uint32_t(K) : L.nfold;
     const uint32_t nout = L.nout;
     const bool new_wins = L.new_wins_ties != 0;
     const uint32_t tid = threadIdx.x;
 
-    if (vector) {
-        // A tile is kVecIters groups of kThreads * U vectors, taken one after the other: the segment
+    if (sv.vector) {
+        // A tile is kVecIters groups of kThreads vectors, taken one after the other: the segment
         // lookup above is paid once per tile while the registers of one group suffice.
-        const uint64_t nvec = count / EPV;
+        const uint64_t nvec = sv.count / EPV;
         for (uint32_t it = 0; it < kVecIters; ++it) {
-            const uint64_t vbase = (uint64_t(local_tile) * kVecIters + it) * (kThreads * U);
+            const uint64_t vbase = (uint64_t(local_tile) * kVecIters + it) * kThreads;
             if (vbase >= nvec) break;
-            const uint64_t in_off = in_begin * sizeof(T) + vbase * kVecBytes;
-            const uint64_t out_off = out_begin * sizeof(T) + vbase * kVecBytes;
             const uint64_t left = nvec - vbase;  // vectors from this group's start to the segment's end
-            AccFor<T, OP> acc[U];
-            if (left >= uint64_t(kThreads) * U) {
-                // full tile: no predicates
-                if constexpr (K > 0) {
-                    u32x4 x[K][U];
-#pragma unroll
-                    for (int j = 0; j < K; ++j) {
-                        const char* src = static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off;
-#pragma unroll
-                        for (int u = 0; u < U; ++u) x[j][u] = load_tile_vec(src + u * (kThreads * kVecBytes), tid);
-                    }
-#pragma unroll
-                    for (int u = 0; u < U; ++u) {
-                        acc[u].seed(x[0][u]);
-#pragma unroll
-                        for (int j = 1; j < K; ++j) acc[u].fold(x[j][u], new_wins);
-                    }
-                } else {
-                    {
-                        const char* src = static_cast<const char*>(L.in[start]) + in_off;
-#pragma unroll
-                        for (int u = 0; u < U; ++u) acc[u].seed(load_tile_vec(src + u * (kThreads * kVecBytes), tid));
-                    }
-                    uint32_t j = 1;
-                    for (; j + 4 <= nfold; j += 4) {
-                        u32x4 x[4][U];
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) {
-                            const char* src =
-                                    static_cast<const char*>(L.in[rotate_rank(start, dir, j + q, nr)]) + in_off;
-#pragma unroll
-                            for (int u = 0; u < U; ++u) x[q][u] = load_tile_vec(src + u * (kThreads * kVecBytes), tid);
-                        }
-#pragma unroll
-                        for (int q = 0; q < 4; ++q)
-#pragma unroll
-                            for (int u = 0; u < U; ++u) acc[u].fold(x[q][u], new_wins);
-                    }
-                    for (; j < nfold; ++j) {
-                        const char* src = static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off;
-#pragma unroll
-                        for (int u = 0; u < U; ++u)
-                            acc[u].fold(load_tile_vec(src + u * (kThreads * kVecBytes), tid), new_wins);
-                    }
-                }
-                u32x4 res[U];
-#pragma unroll
-                for (int u = 0; u < U; ++u) res[u] = acc[u].finish();
-                for (uint32_t m = 0; m < nout; ++m) {
-                    char* dst = static_cast<char*>(L.out[rotate_rank(out_first, 1, m, nr)]) + out_off;
-#pragma unroll
-                    for (int u = 0; u < U; ++u) store_tile_vec(dst + u * (kThreads * kVecBytes), tid, res[u]);
-                }
-            } else {
-                // last tile of the segment: predicate every vector
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const uint32_t v = u * kThreads + tid;
-                    if (v < left) {
-                        AccFor<T, OP> a;
-                        a.seed(load_vec(static_cast<const char*>(L.in[start]) + in_off + v * kVecBytes));
-                        for (uint32_t j = 1; j < nfold; ++j)
-                            a.fold(load_vec(static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off +
-                                            v * kVecBytes),
-                                   new_wins);
-                        const u32x4 r = a.finish();
-                        for (uint32_t m = 0; m < nout; ++m)
-                            store_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, nr)]) + out_off +
-                                              v * kVecBytes,
-                                      r);
-                    }
-                }
+            if (left < kThreads) {
+                fold_vector_remainder<T, OP>(L, sv, nfold, vbase, left, tid);
+                break;
             }
+            const uint64_t in_off = sv.in_begin * sizeof(T) + vbase * kVecBytes;
+            const uint64_t out_off = sv.out_begin * sizeof(T) + vbase * kVecBytes;
+            AccFor<T, OP> acc;
+            if constexpr (K > 0) {
+                u32x4 x[K];
+#pragma unroll
+                for (int j = 0; j < K; ++j)
+                    x[j] = load_tile_vec(static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off, tid);
+                acc.seed(x[0]);
+#pragma unroll
+                for (int j = 1; j < K; ++j) acc.fold(x[j], new_wins);
+            } else {
+                acc.seed(load_tile_vec(static_cast<const char*>(L.in[start]) + in_off, tid));
+                uint32_t j = 1;
+                for (; j + 4 <= nfold; j += 4) {
+                    u32x4 x[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        x[q] = load_tile_vec(
+                                static_cast<const char*>(L.in[rotate_rank(start, dir, j + q, nr)]) + in_off, tid);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) acc.fold(x[q], new_wins);
+                }
+                for (; j < nfold; ++j)
+                    acc.fold(load_tile_vec(static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off, tid),
+                             new_wins);
+            }
+            const u32x4 res = acc.finish();
+            for (uint32_t m = 0; m < nout; ++m)
+                store_tile_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, nr)]) + out_off, tid, res);
         }
     } else {
         fold_element_tile<T, OP>(L, sv, nfold, local_tile, tid);
@@ -912,11 +870,11 @@ FoldFn pick_fold_group(uint32_t nfold) {
 template <typename T, int OP>
 FoldFn pick_fold(uint32_t nfold) {
     switch (nfold) {
-        case 2: return fold_kernel<T, OP, 2, fold_unroll(2)>;
-        case 3: return fold_kernel<T, OP, 3, fold_unroll(3)>;
-        case 4: return fold_kernel<T, OP, 4, fold_unroll(4)>;
-        case 8: return fold_kernel<T, OP, 8, fold_unroll(8)>;
-        default: return fold_kernel<T, OP, 0, fold_unroll(0)>;
+        case 2: return fold_kernel<T, OP, 2>;
+        case 3: return fold_kernel<T, OP, 3>;
+        case 4: return fold_kernel<T, OP, 4>;
+        case 8: return fold_kernel<T, OP, 8>;
+        default: return fold_kernel<T, OP, 0>;
     }
 }
 

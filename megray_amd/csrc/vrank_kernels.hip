@@ -50,47 +50,31 @@ __device__ __forceinline__ PackEnds pack_ends(const PackLaunch& L, uint32_t copy
     return {copy, 0, 0, copy, n};  // kPackAllGather: read once, write the block into every rank's buffer
 }
 
-template <typename W, int U>
+// One wavefront per tile of kThreads accesses of W bytes: short or narrow block copies.
+template <typename W>
 __global__ void __launch_bounds__(kThreads) pack_kernel(const PackLaunch L) {
     const uint32_t copy = blockIdx.x / L.tiles_per_copy;
     const uint32_t tile = blockIdx.x - copy * L.tiles_per_copy;
     const PackEnds e = pack_ends(L, copy);
-    const uint32_t src_rank = e.src_rank, src_block = e.src_block, dst_rank = e.dst_rank, dst_block = e.dst_block;
-    const uint32_t ndst = e.ndst;
-    const uint64_t base = uint64_t(tile) * (kThreads * U) * sizeof(W);
-    const char* src = static_cast<const char*>(L.in[src_rank]) + src_block * L.block_bytes + base;
-    const uint64_t dst_off = dst_block * L.block_bytes + base;
+    const uint64_t base = uint64_t(tile) * kThreads * sizeof(W);
+    const char* src = static_cast<const char*>(L.in[e.src_rank]) + e.src_block * L.block_bytes + base;
+    const uint64_t dst_off = e.dst_block * L.block_bytes + base;
     const uint64_t left = (L.block_bytes - base) / sizeof(W);
     const uint32_t tid = threadIdx.x;
-    if (left >= uint64_t(kThreads) * U) {
-        W x[U];
+    if (left >= kThreads) {
         if constexpr (sizeof(W) == kVecBytes) {
-#pragma unroll
-            for (int u = 0; u < U; ++u) x[u] = load_tile_vec(src + u * (kThreads * kVecBytes), tid);
-            for (uint32_t m = 0; m < ndst; ++m) {
-                char* dst = static_cast<char*>(L.out[dst_rank + m]) + dst_off;
-#pragma unroll
-                for (int u = 0; u < U; ++u) store_tile_vec(dst + u * (kThreads * kVecBytes), tid, x[u]);
-            }
+            const u32x4 x = load_tile_vec(src, tid);
+            for (uint32_t m = 0; m < e.ndst; ++m)
+                store_tile_vec(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off, tid, x);
         } else {
-#pragma unroll
-            for (int u = 0; u < U; ++u) x[u] = load_w<W>(src + (u * kThreads + tid) * sizeof(W));
-            for (uint32_t m = 0; m < ndst; ++m) {
-                char* dst = static_cast<char*>(L.out[dst_rank + m]) + dst_off;
-#pragma unroll
-                for (int u = 0; u < U; ++u) store_w<W>(dst + (u * kThreads + tid) * sizeof(W), x[u]);
-            }
+            const W x = load_w<W>(src + tid * sizeof(W));
+            for (uint32_t m = 0; m < e.ndst; ++m)
+                store_w<W>(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + tid * sizeof(W), x);
         }
-    } else {
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const uint32_t i = u * kThreads + tid;
-            if (i < left) {
-                const W x = load_w<W>(src + i * sizeof(W));
-                for (uint32_t m = 0; m < ndst; ++m)
-                    store_w<W>(static_cast<char*>(L.out[dst_rank + m]) + dst_off + i * sizeof(W), x);
-            }
-        }
+    } else if (tid < left) {
+        const W x = load_w<W>(src + tid * sizeof(W));
+        for (uint32_t m = 0; m < e.ndst; ++m)
+            store_w<W>(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + tid * sizeof(W), x);
     }
 }
 
@@ -157,10 +141,10 @@ FoldFn pick_copy_group(uint32_t elem_size) {
 
 FoldFn pick_copy(uint32_t elem_size) {
     switch (elem_size) {
-        case 1: return fold_kernel<uint8_t, kCopy, 1, fold_unroll(1)>;
-        case 2: return fold_kernel<uint16_t, kCopy, 1, fold_unroll(1)>;
-        case 4: return fold_kernel<uint32_t, kCopy, 1, fold_unroll(1)>;
-        default: return fold_kernel<uint64_t, kCopy, 1, fold_unroll(1)>;
+        case 1: return fold_kernel<uint8_t, kCopy, 1>;
+        case 2: return fold_kernel<uint16_t, kCopy, 1>;
+        case 4: return fold_kernel<uint32_t, kCopy, 1>;
+        default: return fold_kernel<uint64_t, kCopy, 1>;
     }
 }
 
@@ -210,11 +194,11 @@ const void* pack_kernel_for(const PackLaunch& L) {
     void (*fn)(const PackLaunch) = nullptr;
     if (L.waves == kGroupWaves) return L.width == kVecBytes ? reinterpret_cast<const void*>(&pack_group_kernel) : nullptr;
     switch (L.width) {
-        case 16: fn = pack_kernel<u32x4, pack_unroll()>; break;
-        case 8: fn = pack_kernel<u32x2, pack_unroll()>; break;
-        case 4: fn = pack_kernel<uint32_t, pack_unroll()>; break;
-        case 2: fn = pack_kernel<uint16_t, pack_unroll()>; break;
-        case 1: fn = pack_kernel<uint8_t, pack_unroll()>; break;
+        case 16: fn = pack_kernel<u32x4>; break;
+        case 8: fn = pack_kernel<u32x2>; break;
+        case 4: fn = pack_kernel<uint32_t>; break;
+        case 2: fn = pack_kernel<uint16_t>; break;
+        case 1: fn = pack_kernel<uint8_t>; break;
         default: break;
     }
     return reinterpret_cast<const void*>(fn);

@@ -195,7 +195,6 @@ private:
         m_launch.nfold = m_nfold;
         m_launch.nout = m_nout;
         m_launch.new_wins_ties = m_new_wins ? 1 : 0;
-        m_launch.unroll = fold_unroll(m_nfold);
         m_launch.elem_size = m_elem;
         m_launch.waves = m_waves;
     }
@@ -543,8 +542,7 @@ Status add_pack(Plan& plan, const void* const* in, void* const* out, uint32_t nr
     L.root = root;
     L.ncopies = ncopies;
     L.width = common_width(block_bytes, in, out_c, nranks);
-    L.unroll = pack_unroll();
-    const uint64_t per_tile = uint64_t(kThreads) * L.unroll * L.width;
+    const uint64_t per_tile = uint64_t(kThreads) * L.width;
     const uint64_t tiles = (block_bytes + per_tile - 1) / per_tile;
     if (tiles * ncopies > 0x7fffffffull) return invalid("block too large for one pack launch");
     L.tiles_per_copy = uint32_t(tiles);

@@ -43,7 +43,6 @@ struct FoldLaunch {
     uint32_t nseg;
     uint32_t total_tiles;
     uint32_t new_wins_ties;  // float MAX/MIN: an equal / unordered compare keeps the newcomer
-    uint32_t unroll;         // vectors (or elements) per lane per tile; fixes the tile size
     uint32_t elem_size;
     uint32_t waves;          // wavefronts per workgroup: 1, or 4 for the group form (long vector bodies)
 };
@@ -126,30 +125,20 @@ struct PackLaunch {
     uint32_t ncopies;
     uint32_t tiles_per_copy;
     uint32_t width;   // bytes per lane access: 16, 8, 4, 2 or 1
-    uint32_t unroll;  // accesses per lane per tile
     uint32_t waves;   // wavefronts per workgroup: 1, or kGroupWaves (16-byte accesses, long blocks)
     uint32_t groups_per_copy;  // group form: workgroups per block copy
 };
 
-// Vectors (or elements) each lane moves per tile.  The kernels are instantiated with these values;
-// the planner sizes its tiles with the same function.
-// Measured on MI355X: one vector per lane beats every deeper unroll, for every fold width.
-constexpr uint32_t fold_unroll(uint32_t /*nfold*/) {
-    return 1u;
-}
-constexpr uint32_t pack_unroll() {
-    return 1u;
-}
-
-// Elements each lane handles in an element-wise tile (unaligned buffers, run heads and tails), and
-// vector groups a lane walks through, one after the other, in a vector tile of the general kernel.
+// Tile sizes of the one-wavefront-per-tile kernels.  Measured on MI355X: one 16-byte vector per lane and
+// access beats every deeper unroll, for every fold width; a vector tile is kVecIters such groups
+// taken one after the other, an element tile kElemsPerLane elements per lane.
 constexpr uint32_t kElemsPerLane = 16;
 constexpr uint32_t kVecIters = 4;
 
 // Elements a workgroup takes of a vector or an element segment (group form: on average).
 inline uint64_t tile_elems(const FoldLaunch& L, bool vector) {
     if (vector && L.waves == kGroupWaves) return uint64_t(kThreads) * kGroupWaves * (kVecBytes / L.elem_size);
-    uint64_t per_lane = vector ? uint64_t(L.unroll) * kVecIters * (kVecBytes / L.elem_size) : kElemsPerLane;
+    uint64_t per_lane = vector ? uint64_t(kVecIters) * (kVecBytes / L.elem_size) : kElemsPerLane;
     return uint64_t(kThreads) * per_lane;
 }
 
