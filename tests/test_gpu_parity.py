@@ -470,8 +470,11 @@ def test_planned_collectives_and_graph_replay():
     """mrv_plan_*: a plan launched repeatedly, eagerly and as a HIP graph of kernel nodes, gives the
     eager result on every replay, with other work and host syncs between the replays."""
     rng = np.random.default_rng(11)
-    nranks, length = 8, 40000 + 3
-    for sched in (mr.Schedule.FUSED, mr.Schedule.TWO_PHASE, mr.Schedule.RING):
+    nranks = 8
+    # the second length runs the group kernels (workgroups of 256 threads) also as graph nodes
+    for sched, length in ((mr.Schedule.FUSED, 40000 + 3), (mr.Schedule.TWO_PHASE, 40000 + 3),
+                          (mr.Schedule.RING, 40000 + 3), (mr.Schedule.FUSED, 700 * 256 + 5),
+                          (mr.Schedule.TWO_PHASE, 5000 * 256 + 5)):
         ins = [rand_array(orc.FLOAT32, length, rng) for _ in range(nranks)]
         want = orc.ucx_all_reduce(ins, orc.FLOAT32, orc.SUM)
         d_in = [to_device(x) for x in ins]
