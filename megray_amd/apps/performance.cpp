@@ -38,6 +38,8 @@ struct Arguments {
     int iters = 100;
     std::string func_select = "ALL";
     size_t bufsize = 0, in_bufsize = 0, out_bufsize = 0;
+    hipStream_t shared_stream = nullptr;  // -S: every rank enqueues on this one stream
+    bool share = false;
 };
 
 using Kernel = std::function<void(std::shared_ptr<MegRay::Communicator>, void*, void*, std::shared_ptr<MegRay::Context>)>;
@@ -67,8 +69,8 @@ size_t now_us() {
 // worker() of test/performance.cpp:103-137
 void worker(const Func& func, Arguments args, int dev, int port, double* res) {
     CHECK_HIP(hipSetDevice(0));
-    hipStream_t stream;
-    CHECK_HIP(hipStreamCreate(&stream));
+    hipStream_t stream = args.shared_stream;
+    if (!args.share) CHECK_HIP(hipStreamCreate(&stream));
     auto context = MegRay::HipContext::make(stream);
     auto comm = MegRay::get_communicator(args.n_devs, dev, MegRay::MEGRAY_VRANK);
     if (comm->init(args.master_ip.c_str(), port) != MegRay::MEGRAY_OK) std::exit(1);
@@ -85,7 +87,7 @@ void worker(const Func& func, Arguments args, int dev, int port, double* res) {
     size_t t1 = now_us();
     CHECK_HIP(hipFree(in_ptr));
     CHECK_HIP(hipFree(out_ptr));
-    CHECK_HIP(hipStreamDestroy(stream));
+    if (!args.share) CHECK_HIP(hipStreamDestroy(stream));
     if (dev == 0) *res = double(t1 - t0) / args.iters;
 }
 
@@ -170,6 +172,8 @@ void show_help(const char* argv0) {
                  "      -s[int]     packet size in bytes per rank (default: 8, 1 KiB, 512 KiB, 1 MiB, 10 MiB)\n"
                  "      -w[int]     warm-up iterations (default 100)\n"
                  "      -i[int]     timed iterations (default 100)\n"
+                 "      -S          all ranks enqueue on ONE stream (not in the reference's harness: its ranks\n"
+                 "                  are devices); without it every rank has a stream of its own\n"
                  "      -A -B       send/recv: sending node rank / dev (default 0 / 0)\n"
                  "      -C -D       send/recv: receiving node rank / dev (default 0 / 1)\n\n"
                  "    example: "
@@ -186,9 +190,10 @@ void print(T value) {
 int main(int argc, char* argv[]) {
     Arguments args;
     int ch;
-    while ((ch = getopt(argc, argv, "hd:I:P:n:r:e:f:s:w:i:A:B:C:D:")) != EOF) {
+    while ((ch = getopt(argc, argv, "hSd:I:P:n:r:e:f:s:w:i:A:B:C:D:")) != EOF) {
         switch (ch) {
             case 'h': show_help(argv[0]); return 0;
+            case 'S': args.share = true; break;
             case 'd': args.n_devs = std::atoi(optarg); break;
             case 'I': args.master_ip = optarg; break;
             case 'P': args.port = std::atoi(optarg); break;
@@ -222,6 +227,10 @@ int main(int argc, char* argv[]) {
     if (hipGetDeviceCount(&devices) != hipSuccess || devices < 1) {
         std::cerr << "no GPU\n";
         return 2;
+    }
+    if (args.share) {
+        CHECK_HIP(hipSetDevice(0));
+        CHECK_HIP(hipStreamCreate(&args.shared_stream));
     }
     const std::string want = args.func_select;
     for (const Func& func : all_funcs()) {

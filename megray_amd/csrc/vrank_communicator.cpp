@@ -33,6 +33,7 @@ struct Call {
     void* recv;
     hipStream_t stream;
     int device;
+    bool arrived_recorded = false;  // the rank marked its stream's position itself (see Group::collective)
 };
 
 bool same_collective(const Call& a, const Call& b) {
@@ -85,11 +86,20 @@ public:
 
     // Deposit `call` for `rank` and wait until every rank of the group has done the same; the last
     // to arrive enqueues the collective for all.  Every rank returns the same Status.
-    Status collective(uint32_t rank, const Call& call) {
+    Status collective(uint32_t rank, const Call& in_call) {
+        Call call = in_call;
         // Every rank marks, on its own stream and from its own thread, the point its buffers are
         // ready at; the N records run in parallel instead of one after the other in the leader.
-        if (!m_arrive[rank]) HIP_CHECK(hipEventCreateWithFlags(&m_arrive[rank], hipEventDisableTiming));
-        HIP_CHECK(hipEventRecord(m_arrive[rank], call.stream));
+        // A rank whose stream is the one every rank shared last time skips the record: if all ranks
+        // share a stream again nobody needs it (no cross-stream edge exists), and if not, the leader
+        // records it on the rank's behalf before it waits on it.
+        const bool shared = m_shared_valid.load(std::memory_order_acquire) &&
+                            m_shared_stream.load(std::memory_order_relaxed) == static_cast<void*>(call.stream);
+        if (!shared) {
+            if (!m_arrive[rank]) HIP_CHECK(hipEventCreateWithFlags(&m_arrive[rank], hipEventDisableTiming));
+            HIP_CHECK(hipEventRecord(m_arrive[rank], call.stream));
+            call.arrived_recorded = true;
+        }
 
         std::unique_lock<std::mutex> lock(m_mutex);
         m_slots[rank] = call;
@@ -190,10 +200,20 @@ private:
         }
         // order the leader's stream behind everything already enqueued on the other ranks' streams
         hipStream_t stream = lead.stream;
+        bool one_stream = true;
         for (uint32_t r = 0; r < m_nranks; ++r) {
             if (m_slots[r].stream == stream) continue;
+            one_stream = false;
+            if (!m_slots[r].arrived_recorded) {
+                // the rank expected everyone on its stream; it is parked in collective(), so its stream's
+                // tail is still the point it arrived at
+                if (!m_arrive[r]) HIP_CHECK(hipEventCreateWithFlags(&m_arrive[r], hipEventDisableTiming));
+                HIP_CHECK(hipEventRecord(m_arrive[r], m_slots[r].stream));
+            }
             HIP_CHECK(hipStreamWaitEvent(stream, m_arrive[r], 0));
         }
+        m_shared_stream.store(static_cast<void*>(stream), std::memory_order_relaxed);
+        m_shared_valid.store(one_stream, std::memory_order_release);
         Status st = MEGRAY_OK;
         const uint32_t n = m_nranks;
         switch (lead.kind) {
@@ -224,9 +244,11 @@ private:
                 break;
         }
         if (st == MEGRAY_INVALID_ARGUMENT) MEGRAY_ERROR("collective rejected: %s", plan_error());
-        // the other ranks order their streams behind this point themselves
-        if (!m_done) HIP_CHECK(hipEventCreateWithFlags(&m_done, hipEventDisableTiming));
-        HIP_CHECK(hipEventRecord(m_done, stream));
+        // the other ranks order their streams behind this point themselves (none has to if all share the stream)
+        if (!one_stream) {
+            if (!m_done) HIP_CHECK(hipEventCreateWithFlags(&m_done, hipEventDisableTiming));
+            HIP_CHECK(hipEventRecord(m_done, stream));
+        }
         return st;
     }
 
@@ -260,6 +282,8 @@ private:
     static constexpr int kSpinPolls = 20000;
     Status m_result[2] = {MEGRAY_OK, MEGRAY_OK};
     hipStream_t m_lead_stream[2] = {nullptr, nullptr};
+    std::atomic<void*> m_shared_stream{nullptr};  // the stream of the last collective, ...
+    std::atomic<bool> m_shared_valid{false};      // ... if every rank passed that same one
     std::vector<hipEvent_t> m_arrive;  // per rank: "my buffers are ready", recorded by the rank itself
     hipEvent_t m_done = nullptr;       // recorded by the leader behind the collective
     std::vector<hipEvent_t> m_events;  // point-to-point transfers

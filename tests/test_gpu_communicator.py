@@ -250,6 +250,41 @@ def test_random_data_orders_and_work_queued_on_rank_streams(nranks):
     run_test(nranks, ins, [want[r] if r == nranks - 1 else None for r in range(nranks)], reduce_main)
 
 
+def test_ranks_that_share_a_stream_and_ranks_that_stop_sharing_it():
+    """Ranks on one stream need no cross-stream edges, and a rank skips marking its stream when everyone
+    shared it last time.  Round 1: all four ranks on the default stream.  Round 2: ranks 1 and 3 move to
+    streams of their own, fill their inputs there right before the collective and read the result there
+    right after - the leader has to insert the edges those ranks did not announce.  Round 3: all share
+    again."""
+    nranks, length = 4, 1 << 16
+    rng = np.random.default_rng(99)
+    rounds = [[rand_array(orc.FLOAT32, length, rng) for _ in range(nranks)] for _ in range(3)]
+    wants = [orc.ucx_all_reduce(ins, orc.FLOAT32, orc.SUM) for ins in rounds]
+    shared = torch.cuda.current_stream()
+    gate = threading.Barrier(nranks)
+
+    def main(comm, rank, _inp, _stream):
+        outs = []
+        own = torch.cuda.Stream()
+        for rnd in range(3):
+            stream = own if (rnd == 1 and rank in (1, 3)) else shared
+            staged = torch.from_numpy(rounds[rnd][rank].view(np.uint8).copy()).pin_memory()
+            host_out = torch.empty(length * 4, dtype=torch.uint8).pin_memory()
+            with torch.cuda.stream(stream):
+                src = torch.empty(length * 4, dtype=torch.uint8, device="cuda:0")
+                dst = torch.full((length * 4,), 0x5A, dtype=torch.uint8, device="cuda:0")
+                src.copy_(staged, non_blocking=True)
+                comm.all_reduce(src, dst, length, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream)
+                host_out.copy_(dst, non_blocking=True)
+            stream.synchronize()
+            outs.append(host_out.numpy().view(np.float32).copy())
+            gate.wait(60)  # keep the rounds apart: on the shared stream they would order themselves anyway
+        return np.concatenate(outs)
+
+    expected = [np.concatenate([wants[rnd][r] for rnd in range(3)]) for r in range(nranks)]
+    run_test(nranks, [None] * nranks, expected, main, own_streams=False)
+
+
 def test_contract_violations_throw_on_the_calling_rank():
     nranks = 2
     port = mr.get_free_port()
