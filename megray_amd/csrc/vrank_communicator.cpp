@@ -66,7 +66,7 @@ public:
         for (hipEvent_t ev : m_arrive)
             if (ev) (void)hipEventDestroy(ev);
         if (m_done) (void)hipEventDestroy(m_done);
-        if (m_counters) (void)hipFree(m_counters);
+        for (uint64_t* c : m_counters) (void)hipFree(c);
     }
 
     // Groups are found by the 128-bit id rank 0 drew and the bootstrap broadcast.
@@ -184,24 +184,33 @@ private:
 
     // Cross-stream ordering, "stream B goes on after what stream A holds now", is a mark on A and an
     // await on B.  Where the runtime has stream memory operations, a mark writes a ticket (the
-    // collective's number) into a 64-bit counter in device memory and an await polls it for
+    // collective's number) into a 64-bit counter in signal memory and an await polls it for
     // ">= ticket"; measured on MI355X with 8 threads each doing one mark and one cross-stream await,
     // that costs 27 us a round against 71 us with event record / stream-wait-event, which is the
     // fallback.  Slot r < nranks: rank r has arrived; slot nranks: the collective is enqueued.
     void prepare_edges(hipStream_t probe) {
         std::call_once(m_edges_once, [&] {
-            uint64_t* counters = nullptr;
-            const size_t bytes = sizeof(uint64_t) * kCounterStride * (kMaxRanks + 1);
-            if (hipMalloc(reinterpret_cast<void**>(&counters), bytes) != hipSuccess) {
+            // hipStreamWaitValue64 polls "signal memory" only (an 8-byte allocation of its own kind per
+            // counter), and a device says whether it can
+            int device = 0, can_wait = 0;
+            if (hipGetDevice(&device) != hipSuccess ||
+                hipDeviceGetAttribute(&can_wait, hipDeviceAttributeCanUseStreamWaitValue, device) != hipSuccess ||
+                !can_wait) {
                 (void)hipGetLastError();
                 return;
             }
-            if (hipMemset(counters, 0, bytes) != hipSuccess ||
-                hipStreamWriteValue64(probe, counters + kCounterStride * kMaxRanks, 0, 0) != hipSuccess ||
-                hipStreamWaitValue64(probe, counters + kCounterStride * kMaxRanks, 0, hipStreamWaitValueGte,
-                                     ~uint64_t(0)) != hipSuccess) {
+            std::vector<uint64_t*> counters(m_nranks + 1, nullptr);
+            bool ok = true;
+            for (uint64_t*& c : counters) {
+                ok = ok && hipExtMallocWithFlags(reinterpret_cast<void**>(&c), sizeof(uint64_t), hipMallocSignalMemory) ==
+                                   hipSuccess;
+                ok = ok && hipStreamWriteValue64(probe, c, 0, 0) == hipSuccess;
+            }
+            ok = ok && hipStreamSynchronize(probe) == hipSuccess;
+            if (!ok) {
                 (void)hipGetLastError();
-                (void)hipFree(counters);
+                for (uint64_t* c : counters)
+                    if (c) (void)hipFree(c);
                 return;
             }
             m_counters = counters;
@@ -210,8 +219,8 @@ private:
 
     Status mark(uint32_t slot, hipStream_t stream, uint64_t ticket) {
         prepare_edges(stream);
-        if (m_counters) {
-            HIP_CHECK(hipStreamWriteValue64(stream, m_counters + kCounterStride * slot, ticket, 0));
+        if (!m_counters.empty()) {
+            HIP_CHECK(hipStreamWriteValue64(stream, m_counters[slot], ticket, 0));
             return MEGRAY_OK;
         }
         hipEvent_t& ev = slot < m_nranks ? m_arrive[slot] : m_done;
@@ -221,9 +230,8 @@ private:
     }
 
     Status await(uint32_t slot, hipStream_t stream, uint64_t ticket) {
-        if (m_counters) {
-            HIP_CHECK(hipStreamWaitValue64(stream, m_counters + kCounterStride * slot, ticket, hipStreamWaitValueGte,
-                                           ~uint64_t(0)));
+        if (!m_counters.empty()) {
+            HIP_CHECK(hipStreamWaitValue64(stream, m_counters[slot], ticket, hipStreamWaitValueGte, ~uint64_t(0)));
             return MEGRAY_OK;
         }
         HIP_CHECK(hipStreamWaitEvent(stream, slot < m_nranks ? m_arrive[slot] : m_done, 0));
@@ -327,9 +335,8 @@ private:
     hipStream_t m_lead_stream[2] = {nullptr, nullptr};
     std::atomic<void*> m_shared_stream{nullptr};  // the stream of the last collective, ...
     std::atomic<bool> m_shared_valid{false};      // ... if every rank passed that same one
-    static constexpr size_t kCounterStride = 16;  // counters 128 bytes apart
     std::once_flag m_edges_once;
-    uint64_t* m_counters = nullptr;    // device memory; null: events below are used instead
+    std::vector<uint64_t*> m_counters;  // signal memory, one per slot; empty: the events below are used instead
     std::vector<hipEvent_t> m_arrive;  // per rank: "my buffers are ready", recorded by the rank itself
     hipEvent_t m_done = nullptr;       // recorded by the leader behind the collective
     std::vector<hipEvent_t> m_events;  // point-to-point transfers

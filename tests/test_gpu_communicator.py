@@ -37,7 +37,7 @@ def run_test(nranks, inputs, expected, main_func, own_streams=True, configure=No
         except BaseException as exc:  # noqa: BLE001
             errors.append((rank, repr(exc)))
 
-    threads = [threading.Thread(target=rank_main, args=(r,)) for r in range(nranks)]
+    threads = [threading.Thread(target=rank_main, args=(r,), daemon=True) for r in range(nranks)]
     for t in threads:
         t.start()
     for t in threads:
