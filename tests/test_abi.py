@@ -111,3 +111,23 @@ def test_no_kernel_spills_or_hogs_registers():
         assert res["scratch"] == 0, f"{name} uses {res['scratch']} bytes of scratch per lane"
         assert res["vgprs"] <= 128, f"{name} uses {res['vgprs']} vector registers"
         assert res["lds"] <= 40 * 1024, f"{name} uses {res['lds']} bytes of LDS"
+
+
+def test_device_code_has_no_packed_fp32_instructions(tmp_path):
+    """The fp32 and fp64 folds must be chains of single IEEE operations: the build switches the packed
+    fp32 instructions off, and the generated gfx950 code of the fp32 kernels shows none."""
+    import shutil
+    import subprocess
+
+    from megray_amd import build
+    if not shutil.which(build.HIPCC) and not os.path.exists(build.HIPCC):
+        pytest.skip("no hipcc here")
+    out = tmp_path / "fold_f32.s"
+    cmd = ([build.HIPCC] + build.COMMON_FLAGS + ["-x", "hip"] + build.DEVICE_FLAGS +
+           ["--cuda-device-only", "-S", os.path.join(build.CSRC, "vrank_fold_f32.hip"), "-o", str(out)])
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    text = out.read_text()
+    assert text.count("v_add_f32") > 100, "the fp32 kernels are not in this file"
+    for bad in ("v_pk_add_f32", "v_pk_mul_f32", "v_pk_fma_f32"):
+        assert bad not in text, f"{bad} in the generated code"
