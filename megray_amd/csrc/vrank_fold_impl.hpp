@@ -2,20 +2,28 @@
 // unit per element type (vrank_fold_<type>.hip), each of which instantiates the launchers for its
 // type, so that the types compile in parallel.
 //
-// fold_kernel / fold_flat_kernel / fold_tree_kernel
-//              : every output element is a combination, in a fixed rank order, of the same element
-//                of K input buffers, stored to M output buffers.  They replace the 2-input
-//                reduce_{sum,max,min}_kernel of the reference (src/ucx/kernel.cu:16-38) and the
-//                cpu_reduce_kernel loop (src/shm/utils.cpp:16-37): a whole ring of N-1 two-input
-//                steps on one chunk is one pass here, the ring order surviving as the fold order.
-//                fold_flat_kernel is the fast form for K == rank count on aligned buffers;
-//                fold_kernel takes everything else (any K, unaligned buffers, shifted copies);
-//                fold_tree_kernel is the element-wise binomial tree for arbitrary rank counts.
+// Every output element is a combination, in a fixed rank order, of the same element of K input
+// buffers, stored to M output buffers.  The kernels replace the 2-input reduce_{sum,max,min}_kernel
+// of the reference (src/ucx/kernel.cu:16-38) and the cpu_reduce_kernel loop
+// (src/shm/utils.cpp:16-37): a whole ring of N-1 two-input steps on one chunk is one pass here, the
+// ring order surviving as the fold order.
 //
-// All are pure streaming kernels: HBM-bound, one 128-bit access per lane per buffer, no LDS, no
-// matrix instructions.  A workgroup is ONE 64-wide wavefront whose lanes read consecutive 16-byte
-// vectors, so every load and store instruction covers one contiguous KiB and a tile is 1 KiB per
-// buffer: on MI355X many small tiles sustain more HBM bandwidth than fewer large ones.
+//   flat launches     K == rank count in {2, 3, 4, 8}, buffers 16-byte aligned: tile t is the same
+//                     KiB of every buffer, so loads need nothing but the block index.
+//                     fold_group_kernel (512 tiles and more) / fold_flat_kernel (fewer).
+//   segment launches  any K, buffers that share an offset from a 16-byte boundary or none at all,
+//                     shifted copies: head / vector body / tail segments cut by the planner.
+//                     fold_segment_group_kernel (long vector bodies) / fold_kernel.
+//   fold_tree_kernel  element-wise binomial tree for rank counts without a flat kernel.
+//
+// All are pure streaming kernels: HBM-bound, one 128-bit access per lane per buffer, no matrix
+// instructions.  A wavefront's lanes read consecutive 16-byte vectors, so every load and store
+// instruction covers one contiguous KiB, and a tile is 1 KiB per buffer.  The kernels for short
+// launches run one wavefront per tile.  The group kernels run four wavefronts per workgroup on four
+// tiles that lie 32 tiles apart and pass the tiles between the wavefronts through LDS, so that the
+// accesses one wavefront issues together go to different tiles: on MI355X that sustains 80 - 85 %
+// of the HBM peak where one wavefront per tile reaches 64 - 76 %, depending on where the caller's
+// buffers happen to lie.
 #pragma once
 
 #include <hip/hip_runtime.h>
