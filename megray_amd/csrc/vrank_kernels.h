@@ -16,7 +16,8 @@ const void* flat_kernel_for(const FlatLaunch& launch, DType dtype, ReduceOp op);
 const void* tree_kernel_for(const TreeLaunch& launch, DType dtype, ReduceOp op);
 const void* pack_kernel_for(const PackLaunch& launch);
 
-// Enqueue `kernel` over `grid` one-wavefront workgroups with `*launch` as its only argument.
+// Enqueue `kernel` over `grid` workgroups of `block` threads (one or four wavefronts) with `*launch` as
+// its only argument.
 hipError_t enqueue(const void* kernel, uint32_t grid, uint32_t block, const void* launch, hipStream_t stream);
 
 }  // namespace vrank

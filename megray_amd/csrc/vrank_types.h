@@ -11,7 +11,7 @@ namespace vrank {
 constexpr uint32_t kMaxRanks = 16;            // virtual ranks per group
 constexpr uint32_t kMaxChunks = 2 * kMaxRanks;  // the shm order splits a buffer into 2N chunks
 constexpr uint32_t kMaxSegments = 3 * kMaxChunks;  // head / aligned body / tail per chunk
-constexpr uint32_t kThreads = 64;             // workgroup = one 64-wide wavefront (measured best: 1 KiB per buffer per tile)
+constexpr uint32_t kThreads = 64;             // one 64-wide wavefront per tile (measured best: 1 KiB per buffer per tile)
 constexpr uint32_t kVecBytes = 16;            // one 128-bit global load / store per lane
 
 enum SegmentFlags : uint8_t {
