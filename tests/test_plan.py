@@ -295,3 +295,24 @@ def test_planner_rejects_what_it_cannot_honour():
     mr.describe(mr.Collective.ALL_GATHER, [rp[r] + r * 400 for r in range(4)], rp, 100, orc.FLOAT32)
     with pytest.raises(mr.MegRayError, match="out of place"):
         mr.describe(mr.Collective.REDUCE_SCATTER, sp, sp, 100, orc.FLOAT32)
+
+
+def test_group_form_tile_mapping_covers_every_tile_once():
+    """The group kernels map workgroup b to the tiles first + k * 32 (k = 0..3), first = (b // 32) * 128 + b % 32,
+    over a grid of ceil(tiles / 128) * 32 workgroups (kGroupWaves = 4, kGroupStride = 32 in vrank_types.h).
+    Restated here: every tile below the rounded-up count is owned by exactly one (workgroup, wavefront), so
+    with the kernels' own "tile inside the buffer" checks nothing is skipped and nothing is touched twice."""
+    waves, stride = 4, 32
+    for tiles in (1, 31, 32, 127, 128, 129, 512, 1000, 4097, 65536 + 5):
+        grid = (tiles + waves * stride - 1) // (waves * stride) * stride
+        owned = np.zeros(grid * waves, dtype=np.int32)
+        b = np.arange(grid)
+        first = (b // stride) * (waves * stride) + b % stride
+        for k in range(waves):
+            np.add.at(owned, first + k * stride, 1)
+        assert owned.size >= tiles and owned.size - tiles < waves * stride
+        assert (owned == 1).all(), f"tiles={tiles}"
+    # the planner's grid for a described launch agrees: 2^20 tiles -> 2^18 workgroups of 4 wavefronts
+    sp, rp = fake_ptrs(SEND_BASE, 8, [0] * 8), fake_ptrs(RECV_BASE, 8, [0] * 8)
+    runs, _, _ = mr.describe(mr.Collective.ALL_REDUCE, sp, rp, 1 << 28, orc.FLOAT32)
+    assert sum(r["tiles"] for r in runs) == 1 << 20 and all(r["waves"] == 4 for r in runs)
