@@ -134,8 +134,9 @@ def small_message_sweep(torch, mr):
 def copy_yardstick(torch, mr):
     """What this particular GPU sustains on the simplest streaming job, for context: a 1 GiB device copy
     through this library's copy kernel and through torch (GB/s, read + write)."""
+    from megray_amd import synth
     n = 1 << 30
-    src = torch.empty(n, dtype=torch.uint8, device="cuda:0").zero_()
+    src = synth.fill_torch(torch.uint8, n, 0)  # random bytes: the rate depends on the data (zeros copy faster)
     dst = torch.empty_like(src)
     st = torch.cuda.current_stream()
 
