@@ -243,13 +243,16 @@ def test_float_special_values_and_tie_conventions():
         with np.errstate(over="ignore", under="ignore"):
             vals = base.astype(npdt)
         ins = [rng.choice(vals, size=4096 + 5).astype(npdt) for _ in range(n)]
+        # the same through the group kernels: 600 tiles per buffer
+        long_ins = [rng.choice(vals, size=600 * 1024 // orc.dtype_size(dtype) + 5).astype(npdt) for _ in range(n)]
         for op in OPS:
             for order in ORDERS:
-                want = orc.fold_all_reduce(ins, dtype, op, order)[0]
-                got = run_all_reduce(ins, dtype, op, order, mr.Schedule.FUSED)[0]
-                nan = np.isnan(want)
-                assert np.array_equal(np.isnan(got), nan), f"NaN placement dtype={dtype} op={op} order={order}"
-                assert_same(got[~nan], want[~nan], f"specials dtype={dtype} op={op} order={order}")
+                for data in (ins, long_ins):
+                    want = orc.fold_all_reduce(data, dtype, op, order)[0]
+                    got = run_all_reduce(data, dtype, op, order, mr.Schedule.FUSED)[0]
+                    nan = np.isnan(want)
+                    assert np.array_equal(np.isnan(got), nan), f"NaN placement dtype={dtype} op={op} order={order}"
+                    assert_same(got[~nan], want[~nan], f"specials dtype={dtype} op={op} order={order} len={data[0].size}")
             rs_in = [x[:4096] for x in ins]
             want = orc.fold_reduce_scatter(rs_in, dtype, op, orc.ORDER_UCX)
             d_in = [to_device(x) for x in rs_in]
