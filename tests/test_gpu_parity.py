@@ -511,6 +511,32 @@ def test_planned_collectives_and_graph_replay():
         assert_same(to_host(d_out[2], np.int32), np.stack(ins).max(axis=0), "graph replay on new data")
     with pytest.raises(mr.MegRayError, match="unknown reduce op"):
         mr.CollectivePlan(mr.Collective.ALL_REDUCE, d_in, d_out, 5000, mr.DType.INT32, 9)
+    # the other collectives plan and replay the same way (here: blocks long enough for the group kernels)
+    nranks, block = 4, 200 * 1024 + 16
+    parts = [rand_array(orc.UINT8, block, rng) for _ in range(nranks)]
+    d_parts = [to_device(x) for x in parts]
+    d_all = [empty_device(nranks * block) for _ in range(nranks)]
+    gather_plan = mr.CollectivePlan(mr.Collective.ALL_GATHER, d_parts, d_all, block, mr.DType.UINT8, graph=True)
+    want = orc.ucx_all_gather(parts, orc.UINT8)
+    for _ in range(2):
+        for o in d_all:
+            o.zero_()
+        gather_plan.launch()
+        torch.cuda.synchronize()
+        for r in range(nranks):
+            assert_same(to_host(d_all[r], np.uint8), want[r], "planned all_gather")
+    gather_plan.close()
+    ins = [rand_array(orc.INT32, nranks * 150 * 256, rng) for _ in range(nranks)]
+    d_in = [to_device(x) for x in ins]
+    d_out = [empty_device(150 * 256 * 4) for _ in range(nranks)]
+    rs_plan = mr.CollectivePlan(mr.Collective.REDUCE_SCATTER, d_in, d_out, 150 * 256, mr.DType.INT32, mr.ReduceOp.MIN)
+    want = orc.fold_reduce_scatter(ins, orc.INT32, orc.MIN, orc.ORDER_UCX)
+    for _ in range(2):
+        rs_plan.launch()
+        torch.cuda.synchronize()
+        for r in range(nranks):
+            assert_same(to_host(d_out[r], np.int32), want[r], "planned reduce_scatter")
+    rs_plan.close()
 
 
 def test_sixteen_ranks_many_segments():
