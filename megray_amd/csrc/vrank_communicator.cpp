@@ -1,6 +1,8 @@
 #include "vrank_communicator.h"
 
 #include <atomic>
+#include <cstdlib>
+#include <cstring>
 #include <chrono>
 #include <condition_variable>
 #include <deque>
@@ -190,6 +192,9 @@ private:
     // fallback.  Slot r < nranks: rank r has arrived; slot nranks: the collective is enqueued.
     void prepare_edges(hipStream_t probe) {
         std::call_once(m_edges_once, [&] {
+            // MEGRAY_VRANK_EDGES=events in the environment keeps to events
+            const char* choice = std::getenv("MEGRAY_VRANK_EDGES");
+            if (choice && std::strcmp(choice, "events") == 0) return;
             // hipStreamWaitValue64 polls "signal memory" only (an 8-byte allocation of its own kind per
             // counter), and a device says whether it can
             int device = 0, can_wait = 0;

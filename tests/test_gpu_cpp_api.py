@@ -12,11 +12,17 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 BIN = os.path.join(ROOT, "tests", "cpp", "test_vrank_opr")
 
 
-def test_cpp_api_thread_per_rank():
+@pytest.mark.parametrize("edges", ["default", "events"])
+def test_cpp_api_thread_per_rank(edges):
+    """`edges`: how the ranks' streams are ordered against each other - stream memory operations where the
+    device has them (default), or events (MEGRAY_VRANK_EDGES=events, also the fallback)."""
     if not os.path.exists(BIN):
         from megray_amd import build
         build.build_cpp_test()
-    proc = subprocess.run([BIN], capture_output=True, text=True, timeout=100)
+    env = dict(os.environ)
+    if edges == "events":
+        env["MEGRAY_VRANK_EDGES"] = "events"
+    proc = subprocess.run([BIN], capture_output=True, text=True, timeout=100, env=env)
     print(proc.stdout)
     print(proc.stderr)
     assert proc.returncode == 0, proc.stdout + proc.stderr
