@@ -225,3 +225,30 @@ def test_offsets_beyond_4_gib():
     for r in range(2):
         sl = slice(r * half, (r + 1) * half)
         assert torch.equal(torch.maximum(ins[0][sl], ins[1][sl]), parts[r])
+
+
+def test_long_ragged_launch():
+    """70000 tiles per buffer with a ragged length (the last group of tiles incomplete, the last tile partial,
+    chunk borders inside tiles), three ranks, out of place and in place, checked in full against an on-device
+    recomputation."""
+    nranks = 3
+    n = (70000 * 1024 + 1024 - 32) // 4 - 1  # int32 elements: 70000 tiles and a partial one
+    ins = [gen(n, torch.int32, r) for r in range(nranks)]
+    want = ins[0] + ins[1] + ins[2]  # wraps like the kernel's unsigned sum
+    outs = [torch.empty_like(t) for t in ins]
+    runs, _, _ = mr.describe(mr.Collective.ALL_REDUCE, ins, outs, n, mr.DType.INT32)
+    assert all(r["waves"] == 4 for r in runs) and sum(r["tiles"] for r in runs) >= 65536
+    mr.all_reduce(ins, outs, n, mr.DType.INT32, mr.ReduceOp.SUM)
+    torch.cuda.synchronize()
+    for r in range(nranks):
+        assert torch.equal(want, outs[r]), f"rank {r}"
+    parts = [torch.empty(n // nranks, dtype=torch.int32, device=DEV) for _ in range(nranks)]
+    mr.reduce_scatter(ins, parts, n // nranks, mr.DType.INT32, mr.ReduceOp.MAX)
+    torch.cuda.synchronize()
+    for r in range(nranks):
+        sl = slice(r * (n // nranks), (r + 1) * (n // nranks))
+        assert torch.equal(torch.maximum(torch.maximum(ins[0][sl], ins[1][sl]), ins[2][sl]), parts[r])
+    mr.all_reduce(ins, ins, n, mr.DType.INT32, mr.ReduceOp.SUM)  # in place
+    torch.cuda.synchronize()
+    for r in range(nranks):
+        assert torch.equal(want, ins[r]), f"in place, rank {r}"
