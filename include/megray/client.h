@@ -9,22 +9,20 @@
 namespace MegRay {
 
 // One per rank.  Talks to the server started by create_server(): barrier, broadcast and
-// allgather of small host-side metadata.
+// allgather of small host-side metadata.  All sizes are bytes.
 class Client {
 public:
-    Client(uint32_t nranks, uint32_t rank);
+    Client(uint32_t group_size, uint32_t own_rank);
     ~Client();
 
     Status connect(const char* master_ip, int port);
 
-    // returns when every rank has arrived
+    // Returns when every rank has arrived.
     Status barrier();
-
-    // sendbuff (on root) and recvbuff both hold sendlen bytes
-    Status broadcast(const void* sendbuff, void* recvbuff, size_t sendlen, uint32_t root);
-
-    // sendbuff holds sendlen bytes, recvbuff holds sendlen * nranks bytes
-    Status allgather(const void* sendbuff, void* recvbuff, size_t sendlen);
+    // `bytes` from `src` on `root` into `dst` on every rank.
+    Status broadcast(const void* src, void* dst, size_t bytes, uint32_t root);
+    // `bytes` from every rank's `src`, concatenated by rank into `dst` (bytes * nranks) on every rank.
+    Status allgather(const void* src, void* dst, size_t bytes);
 
 private:
     uint32_t m_nranks;

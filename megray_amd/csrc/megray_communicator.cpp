@@ -11,17 +11,19 @@ Status Communicator::init(const char* master_ip, int port) {
     return do_init();
 }
 
-Status Communicator::init(BcastCallback cb) {
-    return do_init(cb);
+Status Communicator::init(BcastCallback broadcast_fn) {
+    return do_init(broadcast_fn);
 }
 
-Status Communicator::send(const void* sendbuff, size_t len, DType dtype, uint32_t rank,
-                          std::shared_ptr<Context> ctx) {
-    return _send(sendbuff, len * get_dtype_size(dtype), rank, ctx);
+// element counts become byte counts here; the backends' _send / _recv know nothing of types
+Status Communicator::send(const void* src, size_t count, DType dtype, uint32_t peer, ContextPtr ctx) {
+    const size_t bytes = count * get_dtype_size(dtype);
+    return _send(src, bytes, peer, ctx);
 }
 
-Status Communicator::recv(void* recvbuf, size_t len, DType dtype, uint32_t rank, std::shared_ptr<Context> ctx) {
-    return _recv(recvbuf, len * get_dtype_size(dtype), rank, ctx);
+Status Communicator::recv(void* dst, size_t count, DType dtype, uint32_t peer, ContextPtr ctx) {
+    const size_t bytes = count * get_dtype_size(dtype);
+    return _recv(dst, bytes, peer, ctx);
 }
 
 std::shared_ptr<Communicator> get_communicator(uint32_t nranks, uint32_t rank, Backend backend) {
