@@ -28,25 +28,18 @@ public:
     VRankCommunicator(uint32_t nranks, uint32_t rank);
     ~VRankCommunicator();
 
+    // the Communicator interface (buffer sizes as documented there; `src` / `dst` are this rank's)
     Status do_init() override;
-    Status do_init(BcastCallback cb) override;
-
-    Status scatter(const void* sendbuff, void* recvbuff, size_t recvlen, DType dtype, uint32_t root,
-                   std::shared_ptr<Context> ctx) override;
-    Status gather(const void* sendbuff, void* recvbuff, size_t sendlen, DType dtype, uint32_t root,
-                  std::shared_ptr<Context> ctx) override;
-    Status all_to_all(const void* sendbuff, void* recvbuff, size_t len, DType dtype,
-                      std::shared_ptr<Context> ctx) override;
-    Status all_gather(const void* sendbuff, void* recvbuff, size_t sendlen, DType dtype,
-                      std::shared_ptr<Context> ctx) override;
-    Status all_reduce(const void* sendbuff, void* recvbuff, size_t len, DType dtype, ReduceOp op,
-                      std::shared_ptr<Context> ctx) override;
-    Status reduce_scatter(const void* sendbuff, void* recvbuff, size_t recvlen, DType dtype, ReduceOp op,
-                          std::shared_ptr<Context> ctx) override;
-    Status broadcast(const void* sendbuff, void* recvbuff, size_t len, DType dtype, uint32_t root,
-                     std::shared_ptr<Context> ctx) override;
-    Status reduce(const void* sendbuff, void* recvbuff, size_t len, DType dtype, ReduceOp op, uint32_t root,
-                  std::shared_ptr<Context> ctx) override;
+    Status do_init(BcastCallback broadcast_fn) override;
+    Status scatter(const void* src, void* dst, size_t per_rank, DType dtype, uint32_t root, ContextPtr ctx) override;
+    Status gather(const void* src, void* dst, size_t per_rank, DType dtype, uint32_t root, ContextPtr ctx) override;
+    Status all_to_all(const void* src, void* dst, size_t per_pair, DType dtype, ContextPtr ctx) override;
+    Status all_gather(const void* src, void* dst, size_t per_rank, DType dtype, ContextPtr ctx) override;
+    Status all_reduce(const void* src, void* dst, size_t count, DType dtype, ReduceOp op, ContextPtr ctx) override;
+    Status reduce_scatter(const void* src, void* dst, size_t per_rank, DType dtype, ReduceOp op, ContextPtr ctx) override;
+    Status broadcast(const void* src, void* dst, size_t count, DType dtype, uint32_t root, ContextPtr ctx) override;
+    Status reduce(const void* src, void* dst, size_t count, DType dtype, ReduceOp op, uint32_t root,
+                  ContextPtr ctx) override;
     Status group_start() override;
     Status group_end() override;
 
@@ -57,13 +50,12 @@ public:
     void set_schedule(vrank::Schedule sched) { m_sched = sched; }
 
 protected:
-    Status _send(const void* sendbuff, size_t size, uint32_t rank, std::shared_ptr<Context> ctx) override;
-    Status _recv(void* recvbuf, size_t size, uint32_t rank, std::shared_ptr<Context> ctx) override;
+    Status _send(const void* src, size_t bytes, uint32_t peer, ContextPtr ctx) override;
+    Status _recv(void* dst, size_t bytes, uint32_t peer, ContextPtr ctx) override;
 
 private:
     Status join(const uint64_t id[2]);
-    Status p2p(bool is_send, const void* sendbuff, void* recvbuff, size_t size, uint32_t peer,
-               std::shared_ptr<Context> ctx);
+    Status p2p(bool is_send, const void* src, void* dst, size_t bytes, uint32_t peer, ContextPtr ctx);
 
     std::shared_ptr<vrank::Group> m_group;
     vrank::FoldOrder m_order = vrank::kOrderUcx;
