@@ -33,7 +33,7 @@ namespace MegRay {
 // A HIP stream as the per-call context of a collective.
 class HipContext : public Context {
 public:
-    explicit HipContext(hipStream_t s) : m_stream(s) {}
+    HipContext(hipStream_t s) : m_stream(s) {}
     ContextType type() const override { return MEGRAY_CTX_HIP; }
     hipStream_t get_stream() { return m_stream; }
     static std::shared_ptr<HipContext> make(hipStream_t s) { return std::make_shared<HipContext>(s); }

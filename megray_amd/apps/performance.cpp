@@ -9,9 +9,11 @@
 #include <hip/hip_runtime.h>
 #include <unistd.h>
 
+#include <algorithm>
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
+#include <fstream>
 #include <functional>
 #include <iomanip>
 #include <iostream>
@@ -40,6 +42,14 @@ struct Arguments {
     size_t bufsize = 0, in_bufsize = 0, out_bufsize = 0;
     hipStream_t shared_stream = nullptr;  // -S: every rank enqueues on this one stream
     bool share = false;
+    std::string json_path;  // -J: per-size results as JSON lines, with the spread of the per-call times
+};
+
+// What rank 0's thread measured for one buffer size.
+struct Timing {
+    double avg_us = 0;     // wall time of all iterations including the final stream sync, per iteration
+    double median_us = 0;  // of the time from one call's return to the next call's return
+    double p99_us = 0;
 };
 
 using Kernel = std::function<void(std::shared_ptr<MegRay::Communicator>, void*, void*, std::shared_ptr<MegRay::Context>)>;
@@ -60,14 +70,12 @@ struct Func {
         }                                                                                  \
     } while (0)
 
-size_t now_us() {
-    return size_t(std::chrono::duration_cast<std::chrono::microseconds>(
-                          std::chrono::steady_clock::now().time_since_epoch())
-                          .count());
+double now_us() {
+    return std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now().time_since_epoch()).count();
 }
 
 // worker() of test/performance.cpp:103-137
-void worker(const Func& func, Arguments args, int dev, int port, double* res) {
+void worker(const Func& func, Arguments args, int dev, int port, Timing* res) {
     CHECK_HIP(hipSetDevice(0));
     hipStream_t stream = args.shared_stream;
     if (!args.share) CHECK_HIP(hipStreamCreate(&stream));
@@ -81,18 +89,31 @@ void worker(const Func& func, Arguments args, int dev, int port, double* res) {
     Kernel kernel = func.make(args, dev);
     for (int i = 0; i < args.warmup_iters; i++) kernel(comm, in_ptr, out_ptr, context);
     CHECK_HIP(hipStreamSynchronize(stream));
-    size_t t0 = now_us();
-    for (int i = 0; i < args.iters; i++) kernel(comm, in_ptr, out_ptr, context);
+    std::vector<double> stamps;
+    if (dev == 0) stamps.reserve(size_t(args.iters) + 1);
+    const double t0 = now_us();
+    if (dev == 0) stamps.push_back(t0);
+    for (int i = 0; i < args.iters; i++) {
+        kernel(comm, in_ptr, out_ptr, context);
+        if (dev == 0) stamps.push_back(now_us());
+    }
     CHECK_HIP(hipStreamSynchronize(stream));
-    size_t t1 = now_us();
+    const double t1 = now_us();
     CHECK_HIP(hipFree(in_ptr));
     CHECK_HIP(hipFree(out_ptr));
     if (!args.share) CHECK_HIP(hipStreamDestroy(stream));
-    if (dev == 0) *res = double(t1 - t0) / args.iters;
+    if (dev == 0) {
+        std::vector<double> gaps;
+        for (size_t i = 1; i < stamps.size(); ++i) gaps.push_back(stamps[i] - stamps[i - 1]);
+        std::sort(gaps.begin(), gaps.end());
+        res->avg_us = (t1 - t0) / args.iters;
+        res->median_us = gaps[gaps.size() / 2];
+        res->p99_us = gaps[std::min(gaps.size() - 1, size_t(double(gaps.size()) * 0.99))];
+    }
 }
 
-double run_test(const Func& func, const Arguments& args) {
-    double res = 0;
+Timing run_test(const Func& func, const Arguments& args) {
+    Timing res;
     int port = MegRay::get_free_port();
     if (MegRay::create_server(args.n_devs, port) != MegRay::MEGRAY_OK) std::exit(1);
     std::vector<std::thread> threads;
@@ -169,9 +190,11 @@ void show_help(const char* argv0) {
                  "      -e[string]  backend: ALL or VRANK\n"
                  "      -f[string]  function: ALL, all_reduce, send_recv, scatter, gather, all_to_all,\n"
                  "                  all_gather, reduce_scatter, broadcast, reduce\n"
-                 "      -s[int]     packet size in bytes per rank (default: 8, 1 KiB, 512 KiB, 1 MiB, 10 MiB)\n"
+                 "      -s[int,..]  packet size(s) in bytes per rank (default: 8, 1 KiB, 512 KiB, 1 MiB, 10 MiB)\n"
                  "      -w[int]     warm-up iterations (default 100)\n"
                  "      -i[int]     timed iterations (default 100)\n"
+                 "      -J[path]    also append one JSON line per size to this file: avg, median and 99th percentile\n"
+                 "                  of the per-call time on rank 0 (not in the reference's harness)\n"
                  "      -S          all ranks enqueue on ONE stream (not in the reference's harness: its ranks\n"
                  "                  are devices); without it every rank has a stream of its own\n"
                  "      -A -B       send/recv: sending node rank / dev (default 0 / 0)\n"
@@ -190,10 +213,11 @@ void print(T value) {
 int main(int argc, char* argv[]) {
     Arguments args;
     int ch;
-    while ((ch = getopt(argc, argv, "hSd:I:P:n:r:e:f:s:w:i:A:B:C:D:")) != EOF) {
+    while ((ch = getopt(argc, argv, "hSd:I:P:n:r:e:f:s:w:i:A:B:C:D:J:")) != EOF) {
         switch (ch) {
             case 'h': show_help(argv[0]); return 0;
             case 'S': args.share = true; break;
+            case 'J': args.json_path = optarg; break;
             case 'd': args.n_devs = std::atoi(optarg); break;
             case 'I': args.master_ip = optarg; break;
             case 'P': args.port = std::atoi(optarg); break;
@@ -201,7 +225,16 @@ int main(int argc, char* argv[]) {
             case 'r': args.node_rank = std::atoi(optarg); break;
             case 'e': args.backends = optarg; break;
             case 'f': args.func_select = optarg; break;
-            case 's': args.sizes = std::vector<size_t>(1, size_t(std::atoll(optarg))); break;
+            case 's': {  // one size, or several separated by commas
+                args.sizes.clear();
+                for (const char* p = optarg; *p;) {
+                    char* end = nullptr;
+                    args.sizes.push_back(size_t(std::strtoull(p, &end, 10)));
+                    if (end == p) { std::cerr << "Error arguments\n"; return 1; }
+                    p = *end == ',' ? end + 1 : end;
+                }
+                break;
+            }
             case 'w': args.warmup_iters = std::atoi(optarg); break;
             case 'i': args.iters = std::atoi(optarg); break;
             case 'A': break;  // node ranks of the send/recv pair: one node only
@@ -232,6 +265,14 @@ int main(int argc, char* argv[]) {
         CHECK_HIP(hipSetDevice(0));
         CHECK_HIP(hipStreamCreate(&args.shared_stream));
     }
+    std::ofstream json;
+    if (!args.json_path.empty()) {
+        json.open(args.json_path, std::ios::app);
+        if (!json) {
+            std::cerr << "cannot write " << args.json_path << "\n";
+            return 1;
+        }
+    }
     const std::string want = args.func_select;
     for (const Func& func : all_funcs()) {
         if (want != "ALL" && func.name.rfind(want, 0) != 0) continue;
@@ -249,7 +290,14 @@ int main(int argc, char* argv[]) {
             run.bufsize = size / 4 * 4;
             run.in_bufsize = func.in_bytes(run.bufsize, args.n_devs);
             run.out_bufsize = func.out_bytes(run.bufsize, args.n_devs);
-            double avg_us = run_test(func, run);
+            const Timing timing = run_test(func, run);
+            const double avg_us = timing.avg_us;
+            if (json.is_open()) {
+                json << "{\"func\": \"" << func.name << "\", \"ranks\": " << args.n_devs << ", \"bufsize\": " << size
+                     << ", \"streams\": \"" << (args.share ? "shared" : "own") << "\", \"iters\": " << args.iters
+                     << ", \"avg_us\": " << timing.avg_us << ", \"median_us\": " << timing.median_us
+                     << ", \"p99_us\": " << timing.p99_us << "}" << std::endl;
+            }
             double hbm = func.hbm_bytes(run.bufsize, args.n_devs) / avg_us / 1000.0;
             print(size);
             print(avg_us);

@@ -39,14 +39,17 @@ void set_error(const char* text) {
 template <typename F>
 int guarded(F&& body) {
     try {
+        set_plan_error("");
         Status st = body();
-        if (st == MEGRAY_INVALID_ARGUMENT) {
+        if (st == MEGRAY_OK) return int(st);
+        // the planner and the rank rendezvous leave their reason in plan_error(), the same text on every rank
+        if (plan_error()[0]) {
             set_error(plan_error());
         } else if (st == MEGRAY_HIP_ERR) {
             set_error("hip error (see the log line on stderr)");
         } else if (st == MEGRAY_INVALID_USAGE) {
             set_error("invalid usage (see the log line on stderr)");
-        } else if (st != MEGRAY_OK) {
+        } else {
             set_error("error");
         }
         return int(st);
@@ -213,43 +216,7 @@ namespace {
 // Plans `collective` the way the device entry points do.  Throws for contract violations.
 Status build_plan(Plan& plan, int collective, const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks,
                   size_t count, DType dt, int order, int schedule, uint32_t root) {
-    switch (collective) {
-        case MRV_ALL_REDUCE:
-            if (as_schedule(schedule) == kSchedRing && dt == MEGRAY_FLOAT16)
-                MEGRAY_THROW("the ring schedule is not offered for FLOAT16 (it would round at every hop)");
-            return plan_all_reduce(plan, sendbuffs, recvbuffs, nranks, count, reduce_elem_size(dt), as_order(order),
-                                   as_schedule(schedule));
-        case MRV_REDUCE_SCATTER:
-            return plan_reduce_scatter(plan, sendbuffs, recvbuffs, nranks, count, reduce_elem_size(dt),
-                                       as_order(order), as_schedule(schedule));
-        case MRV_ALL_GATHER:
-            return plan_all_gather(plan, sendbuffs, recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)));
-        case MRV_ALL_TO_ALL:
-            return plan_all_to_all(plan, sendbuffs, recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)));
-        case MRV_SCATTER:
-            if (root >= nranks) MEGRAY_THROW("root out of range");
-            return plan_scatter(plan, sendbuffs[root], recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)), root);
-        case MRV_GATHER:
-            if (root >= nranks) MEGRAY_THROW("root out of range");
-            return plan_gather(plan, sendbuffs, recvbuffs[root], nranks, count, uint32_t(get_dtype_size(dt)), root);
-        case MRV_BROADCAST:
-            if (root >= nranks) MEGRAY_THROW("root out of range");
-            return plan_broadcast(plan, sendbuffs[root], recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)),
-                                  root);
-        case MRV_REDUCE:
-            if (root >= nranks) MEGRAY_THROW("root out of range");
-            return plan_reduce(plan, sendbuffs, recvbuffs[root], nranks, count, reduce_elem_size(dt), as_order(order),
-                               root);
-        case MRV_REDUCE2:
-            return plan_reduce2(plan, sendbuffs[0], sendbuffs[1], recvbuffs[0], count, reduce_elem_size(dt));
-        default:
-            MEGRAY_THROW("unknown collective");
-    }
-}
-
-bool is_reduction(int collective) {
-    return collective == MRV_ALL_REDUCE || collective == MRV_REDUCE_SCATTER || collective == MRV_REDUCE ||
-           collective == MRV_REDUCE2;
+    return plan_collective(plan, collective, sendbuffs, recvbuffs, nranks, count, dt, order, schedule, root);
 }
 
 }  // namespace
@@ -261,6 +228,13 @@ struct mrv_plan {
     std::vector<KernelCall> calls;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+    mrv_plan() = default;
+    mrv_plan(const mrv_plan&) = delete;
+    mrv_plan& operator=(const mrv_plan&) = delete;
+    ~mrv_plan() {
+        if (exec) (void)hipGraphExecDestroy(exec);
+        if (graph) (void)hipGraphDestroy(graph);
+    }
 };
 
 extern "C" {
@@ -323,10 +297,7 @@ size_t mrv_plan_launch_count(const mrv_plan* plan) {
 }
 
 void mrv_plan_destroy(mrv_plan* plan) {
-    if (!plan) return;
-    if (plan->exec) (void)hipGraphExecDestroy(plan->exec);
-    if (plan->graph) (void)hipGraphDestroy(plan->graph);
-    delete plan;
+    delete plan;  // destroys the graph, if any
 }
 
 int mrv_describe(int collective, const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks,

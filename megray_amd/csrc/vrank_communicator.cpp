@@ -7,24 +7,25 @@
 #include <condition_variable>
 #include <deque>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <random>
 
 #include <unistd.h>
 
 #include "megray/hip_context.h"
+#include "vrank_edges.h"
 #include "vrank_engine.h"
+#include "vrank_kernels.h"
 
 namespace MegRay {
 namespace vrank {
 
 namespace {
 
-enum class Kind : int { kScatter, kGather, kAllToAll, kAllGather, kAllReduce, kReduceScatter, kBroadcast, kReduce };
-
 // What one rank brings to a collective.
 struct Call {
-    Kind kind;
+    int kind;  // CollectiveKind
     size_t len;
     DType dtype;
     ReduceOp op;
@@ -35,12 +36,31 @@ struct Call {
     void* recv;
     hipStream_t stream;
     int device;
-    bool arrived_recorded = false;  // the rank marked its stream's position itself (see Group::collective)
+    bool marked = false;    // the rank put a mark on its stream: everything enqueued before the call precedes it
+    bool poisoned = false;  // the rank's own arguments were rejected; it does not take part
 };
 
 bool same_collective(const Call& a, const Call& b) {
     return a.kind == b.kind && a.len == b.len && a.dtype == b.dtype && a.op == b.op && a.root == b.root &&
            a.order == b.order && a.sched == b.sched && a.device == b.device;
+}
+
+// A planned collective kept for the next call with the same arguments and buffers: training loops
+// and benchmarks repeat their collectives, and planning costs more than the launch itself.
+struct CachedPlan {
+    Call key;
+    const void* send[kMaxRanks];
+    void* recv[kMaxRanks];
+    Plan plan;
+    std::vector<KernelCall> calls;  // point into `plan`
+};
+
+uint64_t env_u64(const char* name, uint64_t fallback) {
+    const char* text = std::getenv(name);
+    if (!text || !*text) return fallback;
+    char* end = nullptr;
+    const unsigned long long v = std::strtoull(text, &end, 10);
+    return end == text ? fallback : uint64_t(v);
 }
 
 }  // namespace
@@ -61,14 +81,16 @@ struct PendingP2P {
 class Group {
 public:
     explicit Group(uint32_t nranks)
-            : m_nranks(nranks), m_slots(nranks), m_arrive(nranks, nullptr), m_mail(size_t(nranks) * nranks) {}
+            : m_nranks(nranks), m_slots(nranks), m_entered(nranks, 0), m_arrive(nranks, nullptr),
+              m_mail(size_t(nranks) * nranks) {}
 
     ~Group() {
         for (hipEvent_t ev : m_events) (void)hipEventDestroy(ev);
         for (hipEvent_t ev : m_arrive)
             if (ev) (void)hipEventDestroy(ev);
         if (m_done) (void)hipEventDestroy(m_done);
-        for (uint64_t* c : m_counters) (void)hipFree(c);
+        if (m_words) (void)hipFree(m_words);
+        if (m_status) (void)hipHostFree(m_status);
     }
 
     // Groups are found by the 128-bit id rank 0 drew and the bootstrap broadcast.
@@ -88,59 +110,36 @@ public:
     }
 
     // Deposit `call` for `rank` and wait until every rank of the group has done the same; the last
-    // to arrive enqueues the collective for all.  Every rank returns the same Status.
+    // to arrive enqueues the collective for all.  Every rank returns the same Status (and finds the
+    // same text in plan_error()).
     Status collective(uint32_t rank, const Call& in_call) {
         Call call = in_call;
+        await_release(rank);
         // Every rank marks, on its own stream and from its own thread, the point its buffers are
-        // ready at; the N records run in parallel instead of one after the other in the leader.
-        // A rank whose stream is the one every rank shared last time skips the record: if all ranks
-        // share a stream again nobody needs it (no cross-stream edge exists), and if not, the leader
-        // records it on the rank's behalf before it waits on it.
+        // ready at; the marks are enqueued in parallel instead of one after the other by the leader.
+        // No mark is needed from a rank whose stream is the one every rank shared last time (if all
+        // share a stream again no cross-stream edge exists; if not, the leader marks it on the rank's
+        // behalf, the rank being parked here) or from the rank that sees all others arrived already (it
+        // is going to launch on its own stream).  (Asking the runtime whether a stream is idle, to
+        // skip the mark, costs as much as the mark itself when the stream is busy.)
         const bool shared = m_shared_valid.load(std::memory_order_acquire) &&
                             m_shared_stream.load(std::memory_order_relaxed) == static_cast<void*>(call.stream);
-        const uint64_t ticket = m_generation.load(std::memory_order_acquire) + 1;  // stable until this rank arrives
-        if (!shared) {
-            MEGRAY_CHECK(mark(rank, call.stream, ticket));
-            call.arrived_recorded = true;
+        const bool last = m_arrived.load(std::memory_order_acquire) == m_nranks - 1;
+        if (!shared && !last) {
+            const Status st = mark(rank, call.stream);
+            if (st != MEGRAY_OK) return withdraw(rank, "a stream mark could not be enqueued", st);
+            call.marked = true;
         }
+        return arrive(rank, call, true);
+    }
 
-        std::unique_lock<std::mutex> lock(m_mutex);
-        m_slots[rank] = call;
-        const uint64_t gen = m_generation.load(std::memory_order_relaxed);
-        if (++m_arrived == m_nranks) {
-            Status st;
-            try {
-                st = launch(rank);
-            } catch (const MegRay::Exception& e) {
-                MEGRAY_ERROR("collective failed: %s", e.what());
-                st = MEGRAY_INVALID_ARGUMENT;
-            }
-            m_result[gen & 1] = st;
-            m_lead_stream[gen & 1] = call.stream;
-            m_arrived = 0;
-            m_generation.store(gen + 1, std::memory_order_release);
-            lock.unlock();
-            m_cv.notify_all();
-            return st;
-        }
-        lock.unlock();
-        // The other ranks are usually a few microseconds away: poll the generation for a while before
-        // going to sleep on the condition variable (a sleeping thread costs tens of microseconds to wake).
-        bool released = false;
-        for (int spin = 0; spin < kSpinPolls && !released; ++spin) {
-            released = m_generation.load(std::memory_order_acquire) != gen;
-            if (!released) __builtin_ia32_pause();
-        }
-        if (!released) {
-            lock.lock();
-            m_cv.wait(lock, [&] { return m_generation.load(std::memory_order_acquire) != gen; });
-            lock.unlock();
-        }
-        // ... and orders its own stream behind the result.  The done mark is not set again before
-        // every rank has passed this point: the next collective needs all of them to arrive first.
-        const Status st = m_result[gen & 1];
-        if (st == MEGRAY_OK && call.stream != m_lead_stream[gen & 1]) MEGRAY_CHECK(await(m_nranks, call.stream, gen + 1));
-        return st;
+    // A rank whose own arguments were rejected tells the group and leaves at once (its caller gets
+    // the exception); the other ranks' calls come back with MEGRAY_INVALID_USAGE instead of waiting
+    // for a rank that will never arrive.
+    void poison(uint32_t rank, const char* why) {
+        // still counted as withdrawn from a collective the other ranks have not finished: nothing to add
+        if (m_generation.load(std::memory_order_acquire) < m_entered[rank]) return;
+        (void)withdraw(rank, why, MEGRAY_INVALID_USAGE);
     }
 
     // Post one side of a point-to-point transfer; the side that finds its counterpart already
@@ -184,128 +183,240 @@ private:
         return m_events[index];
     }
 
-    // Cross-stream ordering, "stream B goes on after what stream A holds now", is a mark on A and an
-    // await on B.  Where the runtime has stream memory operations, a mark writes a ticket (the
-    // collective's number) into a 64-bit counter in signal memory and an await polls it for
-    // ">= ticket"; measured on MI355X with 8 threads each doing one mark and one cross-stream await,
-    // that costs 27 us a round against 71 us with event record / stream-wait-event, which is the
-    // fallback.  Slot r < nranks: rank r has arrived; slot nranks: the collective is enqueued.
-    void prepare_edges(hipStream_t probe) {
+    // A rank that left a collective early (poison) comes back only when that collective is over.
+    void await_release(uint32_t rank) {
+        const uint64_t need = m_entered[rank];
+        if (m_generation.load(std::memory_order_acquire) >= need) return;
+        sleep_until_past(need);
+    }
+
+    Status withdraw(uint32_t rank, const char* why, Status st) {
+        Call call{};
+        call.poisoned = true;
+        char text[200];
+        std::snprintf(text, sizeof(text), "rank %u left the collective: %s", rank, why ? why : "");
+        {
+            std::lock_guard<std::mutex> lock(m_poison_mutex);
+            if (!m_poison_text[0]) std::snprintf(m_poison_text, sizeof(m_poison_text), "%s", text);
+        }
+        (void)arrive(rank, call, false);
+        return st;
+    }
+
+    // Deposit and, for the last rank, launch; `park`: wait for the release and order the own stream
+    // behind the result.  Arrival is one atomic increment (eight threads meeting at a mutex spend
+    // more time in its wait queue than the launch takes); the rank whose increment completes the
+    // count reads every slot and launches, the others poll the generation.
+    Status arrive(uint32_t rank, const Call& call, bool park) {
+        m_slots[rank].call = call;
+        if (call.marked) m_marks.fetch_add(1, std::memory_order_relaxed);
+        const uint64_t gen = m_generation.load(std::memory_order_relaxed);  // cannot move on before this rank arrives
+        m_entered[rank] = gen + 1;
+        if (m_arrived.fetch_add(1, std::memory_order_acq_rel) + 1 == m_nranks) {
+            Status st;
+            try {
+                st = launch(rank);
+            } catch (const MegRay::Exception& e) {
+                set_plan_error(e.what());
+                st = MEGRAY_INVALID_ARGUMENT;
+            } catch (const std::exception& e) {
+                set_plan_error(e.what());
+                st = MEGRAY_UNEXPECTED_ERR;
+            } catch (...) {
+                set_plan_error("unknown failure while launching the collective");
+                st = MEGRAY_UNEXPECTED_ERR;
+            }
+            if (st != MEGRAY_OK) {
+                MEGRAY_ERROR("collective failed: %s", plan_error());
+                std::snprintf(m_error[gen & 1], sizeof(m_error[0]), "%s", plan_error());
+            }
+            m_result[gen & 1] = st;
+            m_lead_stream[gen & 1] = call.stream;
+            {
+                std::lock_guard<std::mutex> lock(m_poison_mutex);
+                m_poison_text[0] = 0;
+            }
+            m_arrived.store(0, std::memory_order_relaxed);
+            m_generation.store(gen + 1, std::memory_order_seq_cst);
+            if (m_sleepers.load(std::memory_order_seq_cst)) {
+                { std::lock_guard<std::mutex> lock(m_mutex); }  // a sleeper is either waiting or has not yet checked
+                m_cv.notify_all();
+            }
+            return st;
+        }
+        if (!park) return MEGRAY_OK;
+        // The other ranks are usually a few microseconds away: poll the generation for a while before
+        // going to sleep on the condition variable (a sleeping thread costs tens of microseconds to wake).
+        bool released = false;
+        for (int spin = 0; spin < kSpinPolls && !released; ++spin) {
+            released = m_generation.load(std::memory_order_acquire) != gen;
+            if (!released) __builtin_ia32_pause();
+        }
+        if (!released) sleep_until_past(gen + 1);
+        // ... and orders its own stream behind the result.  The done mark is not set again before
+        // every rank has passed this point: the next collective needs all of them to arrive first.
+        const Status st = m_result[gen & 1];
+        if (st != MEGRAY_OK) {
+            set_plan_error(m_error[gen & 1]);
+            return st;
+        }
+        if (call.stream != m_lead_stream[gen & 1]) MEGRAY_CHECK(await_done(call.stream, gen + 1));
+        return st;
+    }
+
+    void sleep_until_past(uint64_t need) {
+        std::unique_lock<std::mutex> lock(m_mutex);
+        m_sleepers.fetch_add(1, std::memory_order_seq_cst);
+        m_cv.wait(lock, [&] { return m_generation.load(std::memory_order_seq_cst) >= need; });
+        m_sleepers.fetch_sub(1, std::memory_order_seq_cst);
+    }
+
+    // Cross-stream ordering, "stream B goes on after what stream A holds now", is a mark on A and a
+    // wait on B.  Default: the one-wavefront kernels of vrank_edges.h on counters in device memory
+    // (kernel launches from several threads run in parallel in the runtime; its stream memory
+    // operations and event calls are serialised across threads and cost 3 - 5 times as much on
+    // MI355X).  MEGRAY_VRANK_EDGES=events in the environment keeps to event record / stream-wait-event,
+    // which is also the fallback when the counters cannot be allocated.
+    void prepare_edges() {
         std::call_once(m_edges_once, [&] {
-            // MEGRAY_VRANK_EDGES=events in the environment keeps to events
             const char* choice = std::getenv("MEGRAY_VRANK_EDGES");
             if (choice && std::strcmp(choice, "events") == 0) return;
-            // hipStreamWaitValue64 polls "signal memory" only (an 8-byte allocation of its own kind per
-            // counter), and a device says whether it can
-            int device = 0, can_wait = 0;
-            if (hipGetDevice(&device) != hipSuccess ||
-                hipDeviceGetAttribute(&can_wait, hipDeviceAttributeCanUseStreamWaitValue, device) != hipSuccess ||
-                !can_wait) {
-                (void)hipGetLastError();
-                return;
-            }
-            std::vector<uint64_t*> counters(m_nranks + 1, nullptr);
-            bool ok = true;
-            for (uint64_t*& c : counters) {
-                ok = ok && hipExtMallocWithFlags(reinterpret_cast<void**>(&c), sizeof(uint64_t), hipMallocSignalMemory) ==
-                                   hipSuccess;
-                ok = ok && hipStreamWriteValue64(probe, c, 0, 0) == hipSuccess;
-            }
-            ok = ok && hipStreamSynchronize(probe) == hipSuccess;
+            int device = 0, khz = 0;
+            EdgeWords* words = nullptr;
+            uint64_t* status = nullptr;
+            bool ok = hipGetDevice(&device) == hipSuccess &&
+                      hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, device) == hipSuccess && khz > 0;
+            ok = ok && hipMalloc(reinterpret_cast<void**>(&words), sizeof(EdgeWords)) == hipSuccess;
+            ok = ok && hipMemset(words, 0, sizeof(EdgeWords)) == hipSuccess;
+            ok = ok && hipHostMalloc(reinterpret_cast<void**>(&status), sizeof(uint64_t), hipHostMallocDefault) == hipSuccess;
             if (!ok) {
                 (void)hipGetLastError();
-                for (uint64_t* c : counters)
-                    if (c) (void)hipFree(c);
+                if (words) (void)hipFree(words);
+                if (status) (void)hipHostFree(status);
                 return;
             }
-            m_counters = counters;
+            *status = 0;
+            // a wait gives up after this long (wall-clock ticks): long enough for any stream to drain,
+            // short enough that a lost mark does not hold a wavefront for ever
+            const uint64_t limit_ms = env_u64("MEGRAY_VRANK_WAIT_LIMIT_MS", 10000);
+            m_limit_ticks = limit_ms * uint64_t(khz);
+            m_status = status;
+            m_words = words;
         });
     }
 
-    Status mark(uint32_t slot, hipStream_t stream, uint64_t ticket) {
-        prepare_edges(stream);
-        if (!m_counters.empty()) {
-            HIP_CHECK(hipStreamWriteValue64(stream, m_counters[slot], ticket, 0));
+    Status mark(uint32_t rank, hipStream_t stream) {
+        prepare_edges();
+        if (m_words) {
+            HIP_CHECK(edge_arrive(m_words, stream));
             return MEGRAY_OK;
         }
-        hipEvent_t& ev = slot < m_nranks ? m_arrive[slot] : m_done;
+        hipEvent_t& ev = m_arrive[rank];
         if (!ev) HIP_CHECK(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
         HIP_CHECK(hipEventRecord(ev, stream));
         return MEGRAY_OK;
     }
 
-    Status await(uint32_t slot, hipStream_t stream, uint64_t ticket) {
-        if (!m_counters.empty()) {
-            HIP_CHECK(hipStreamWaitValue64(stream, m_counters[slot], ticket, hipStreamWaitValueGte, ~uint64_t(0)));
+    Status await_done(hipStream_t stream, uint64_t ticket) {
+        if (m_words) {
+            HIP_CHECK(edge_wait_done(m_words, ticket, m_limit_ticks, m_status, stream));
             return MEGRAY_OK;
         }
-        HIP_CHECK(hipStreamWaitEvent(stream, slot < m_nranks ? m_arrive[slot] : m_done, 0));
+        HIP_CHECK(hipStreamWaitEvent(stream, m_done, 0));
         return MEGRAY_OK;
     }
 
-    // Called with the mutex held by the last rank to arrive.
+    CachedPlan* lookup(const Call& lead, const void* const* send, void* const* recv) {
+        for (auto& cp : m_plans) {
+            if (same_collective(cp->key, lead) && std::memcmp(cp->send, send, sizeof(cp->send)) == 0 &&
+                std::memcmp(cp->recv, recv, sizeof(cp->recv)) == 0)
+                return cp.get();
+        }
+        return nullptr;
+    }
+
+    // Called by the last rank to arrive; every other rank is parked or has withdrawn.
     Status launch(uint32_t leader) {
-        const Call& lead = m_slots[leader];
-        for (uint32_t r = 0; r < m_nranks; ++r) {
-            if (!same_collective(lead, m_slots[r])) {
-                MEGRAY_ERROR("rank %u and rank %u called different collectives (or with different arguments)",
-                             leader, r);
+        {
+            std::lock_guard<std::mutex> lock(m_poison_mutex);
+            if (m_poison_text[0]) {
+                set_plan_error(m_poison_text);
                 return MEGRAY_INVALID_USAGE;
             }
+        }
+        const Call& lead = m_slots[leader].call;
+        for (uint32_t r = 0; r < m_nranks; ++r) {
+            if (!same_collective(lead, m_slots[r].call)) {
+                char text[160];
+                std::snprintf(text, sizeof(text),
+                              "rank %u and rank %u called different collectives (or with different arguments)", leader, r);
+                set_plan_error(text);
+                return MEGRAY_INVALID_USAGE;
+            }
+        }
+        if (m_status && *m_status != m_status_seen) {
+            m_status_seen = *m_status;
+            set_plan_error("a stream wait of an earlier collective gave up: a rank's stream did not get there in time");
+            return MEGRAY_UNEXPECTED_ERR;
         }
         const void* send[kMaxRanks] = {};
         void* recv[kMaxRanks] = {};
         for (uint32_t r = 0; r < m_nranks; ++r) {
-            send[r] = m_slots[r].send;
-            recv[r] = m_slots[r].recv;
+            send[r] = m_slots[r].call.send;
+            recv[r] = m_slots[r].call.recv;
+        }
+        // plan first: a rejected call must not leave marks or waits behind
+        CachedPlan* cp = lookup(lead, send, recv);
+        if (!cp) {
+            auto fresh = std::make_unique<CachedPlan>();
+            fresh->key = lead;
+            std::memcpy(fresh->send, send, sizeof(send));
+            std::memcpy(fresh->recv, recv, sizeof(recv));
+            Status st = plan_collective(fresh->plan, lead.kind, send, recv, m_nranks, lead.len, lead.dtype, lead.order,
+                                        lead.sched, lead.root);
+            if (st == MEGRAY_OK) st = resolve(fresh->plan, lead.dtype, is_reduction(lead.kind) ? lead.op : MEGRAY_SUM, fresh->calls);
+            if (st != MEGRAY_OK) return st;
+            if (m_plans.size() < kPlanSlots) {
+                m_plans.push_back(std::move(fresh));
+                cp = m_plans.back().get();
+            } else {
+                m_plans[m_plan_next] = std::move(fresh);
+                cp = m_plans[m_plan_next].get();
+                m_plan_next = (m_plan_next + 1) % kPlanSlots;
+            }
         }
         // order the leader's stream behind everything already enqueued on the other ranks' streams
         hipStream_t stream = lead.stream;
-        bool one_stream = true;
+        bool one_stream = true, wait_needed = false;
         for (uint32_t r = 0; r < m_nranks; ++r) {
-            if (m_slots[r].stream == stream) continue;
+            const Call& other = m_slots[r].call;
+            if (other.stream == stream) continue;
             one_stream = false;
-            const uint64_t ticket = m_generation.load(std::memory_order_relaxed) + 1;
-            // a rank that expected everyone on its stream did not mark it; it is parked in collective(),
+            // a rank that expected everyone on its stream did not mark it; it is parked in arrive(),
             // so its stream's tail is still the point it arrived at
-            if (!m_slots[r].arrived_recorded) MEGRAY_CHECK(mark(r, m_slots[r].stream, ticket));
-            MEGRAY_CHECK(await(r, stream, ticket));
+            if (!other.marked) {
+                MEGRAY_CHECK(mark(r, other.stream));
+                m_marks.fetch_add(1, std::memory_order_relaxed);
+            }
+            wait_needed = true;
+            if (!m_words) HIP_CHECK(hipStreamWaitEvent(stream, m_arrive[r], 0));
         }
+        if (wait_needed && m_words)
+            HIP_CHECK(edge_wait_arrived(m_words, m_marks.load(std::memory_order_relaxed), m_limit_ticks, m_status, stream));
         m_shared_stream.store(static_cast<void*>(stream), std::memory_order_relaxed);
         m_shared_valid.store(one_stream, std::memory_order_release);
-        Status st = MEGRAY_OK;
-        const uint32_t n = m_nranks;
-        switch (lead.kind) {
-            case Kind::kAllReduce:
-                st = all_reduce(send, recv, n, lead.len, lead.dtype, lead.op, lead.order, lead.sched, stream);
-                break;
-            case Kind::kReduceScatter:
-                st = reduce_scatter(send, recv, n, lead.len, lead.dtype, lead.op, lead.order, stream);
-                break;
-            case Kind::kAllGather:
-                st = all_gather(send, recv, n, lead.len, lead.dtype, stream);
-                break;
-            case Kind::kAllToAll:
-                st = all_to_all(send, recv, n, lead.len, lead.dtype, stream);
-                break;
-            case Kind::kScatter:
-                st = scatter(send[lead.root], recv, n, lead.len, lead.dtype, lead.root, stream);
-                break;
-            case Kind::kGather:
-                st = gather(send, recv[lead.root], n, lead.len, lead.dtype, lead.root, stream);
-                break;
-            case Kind::kBroadcast:
-                st = broadcast(send[lead.root], recv, n, lead.len, lead.dtype, lead.root, stream);
-                break;
-            case Kind::kReduce:
-                st = reduce_to_root(send, recv[lead.root], n, lead.len, lead.dtype, lead.op, lead.order, lead.root,
-                                    stream);
-                break;
-        }
-        if (st == MEGRAY_INVALID_ARGUMENT) MEGRAY_ERROR("collective rejected: %s", plan_error());
+        for (const KernelCall& call : cp->calls) HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, stream));
         // the other ranks order their streams behind this point themselves (none has to if all share the stream)
-        if (!one_stream) MEGRAY_CHECK(mark(m_nranks, stream, m_generation.load(std::memory_order_relaxed) + 1));
-        return st;
+        if (!one_stream) {
+            const uint64_t ticket = m_generation.load(std::memory_order_relaxed) + 1;
+            if (m_words) {
+                HIP_CHECK(edge_notify(m_words, ticket, stream));
+            } else {
+                if (!m_done) HIP_CHECK(hipEventCreateWithFlags(&m_done, hipEventDisableTiming));
+                HIP_CHECK(hipEventRecord(m_done, stream));
+            }
+        }
+        return MEGRAY_OK;
     }
 
     // Enqueue the copy of a matched send / receive pair: on the receiver's stream, after the
@@ -329,23 +440,39 @@ private:
         return MEGRAY_OK;
     }
 
+    struct alignas(64) Slot {  // one cache line (or more) per rank: ranks deposit at the same time
+        Call call;
+    };
     const uint32_t m_nranks;
-    std::mutex m_mutex;
+    std::mutex m_mutex;  // point-to-point mailboxes; sleeping waiters
     std::condition_variable m_cv;
-    std::vector<Call> m_slots;
-    uint32_t m_arrived = 0;
-    std::atomic<uint64_t> m_generation{0};
+    std::mutex m_poison_mutex;
+    std::vector<Slot> m_slots;
+    std::vector<uint64_t> m_entered;  // per rank: the generation count that ends the collective it last entered
     static constexpr int kSpinPolls = 20000;
+    static constexpr size_t kPlanSlots = 8;
     Status m_result[2] = {MEGRAY_OK, MEGRAY_OK};
+    char m_error[2][256] = {"", ""};  // text that goes with m_result
+    char m_poison_text[200] = "";
     hipStream_t m_lead_stream[2] = {nullptr, nullptr};
     std::atomic<void*> m_shared_stream{nullptr};  // the stream of the last collective, ...
     std::atomic<bool> m_shared_valid{false};      // ... if every rank passed that same one
     std::once_flag m_edges_once;
-    std::vector<uint64_t*> m_counters;  // signal memory, one per slot; empty: the events below are used instead
+    EdgeWords* m_words = nullptr;    // device counters of the edge kernels; null: the events below are used instead
+    uint64_t* m_status = nullptr;    // host memory: waits that gave up
+    uint64_t m_status_seen = 0;
+    uint64_t m_limit_ticks = 0;
+    std::atomic<uint64_t> m_marks{0};  // arrive kernels enqueued so far = value `arrived` reaches when all have run
+    std::atomic<uint32_t> m_sleepers{0};
+    alignas(64) std::atomic<uint32_t> m_arrived{0};     // ranks that have deposited their call
+    alignas(64) std::atomic<uint64_t> m_generation{0};  // collectives released so far; parked ranks poll it
+    alignas(64) char m_pad = 0;
     std::vector<hipEvent_t> m_arrive;  // per rank: "my buffers are ready", recorded by the rank itself
     hipEvent_t m_done = nullptr;       // recorded by the leader behind the collective
     std::vector<hipEvent_t> m_events;  // point-to-point transfers
     std::vector<Mailbox> m_mail;
+    std::vector<std::unique_ptr<CachedPlan>> m_plans;
+    size_t m_plan_next = 0;
 };
 
 }  // namespace vrank
@@ -361,9 +488,14 @@ hipStream_t stream_of(const std::shared_ptr<Context>& ctx) {
     return static_cast<HipContext*>(ctx.get())->get_stream();
 }
 
+// The device the calling thread works on; -1 without one (the group then fails at its first launch,
+// on every rank alike, instead of on this rank alone).
 int current_device() {
     int device = 0;
-    HIP_ASSERT(hipGetDevice(&device));
+    if (hipGetDevice(&device) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
+    }
     return device;
 }
 
@@ -418,68 +550,67 @@ Status VRankCommunicator::do_init(BcastCallback cb) {
     return join(id);
 }
 
-#define VRANK_COLLECTIVE(KIND, LEN, DTYPE, OP, ROOT)                                        \
-    do {                                                                                    \
-        MEGRAY_ASSERT(m_group != nullptr, "communicator used before init()");               \
-        Call call{KIND, LEN, DTYPE, OP, ROOT, m_order, m_sched, sendbuff, recvbuff, stream_of(ctx), \
-                  current_device()};                                                        \
-        return m_group->collective(m_rank, call);                                           \
+// Argument checks run on the calling rank's own thread and throw there, like the reference's; the
+// group is told, so that the other ranks' calls come back instead of waiting for this one.
+#define VRANK_COLLECTIVE(KIND, LEN, DTYPE, OP, ROOT, CHECKS)                                    \
+    do {                                                                                        \
+        MEGRAY_ASSERT(m_group != nullptr, "communicator used before init()");                   \
+        hipStream_t stream = nullptr;                                                           \
+        try {                                                                                   \
+            CHECKS;                                                                             \
+            stream = stream_of(ctx);                                                            \
+        } catch (const MegRay::Exception& e) {                                                  \
+            m_group->poison(m_rank, e.what());                                                  \
+            throw;                                                                              \
+        }                                                                                       \
+        Call call{KIND, LEN, DTYPE, OP, ROOT, m_order, m_sched, sendbuff, recvbuff, stream,     \
+                  current_device()};                                                            \
+        return m_group->collective(m_rank, call);                                               \
     } while (0)
+
+#define VRANK_ROOT_IN_RANGE MEGRAY_ASSERT(root < m_nranks, "root %u out of range", root)
 
 Status VRankCommunicator::scatter(const void* sendbuff, void* recvbuff, size_t recvlen, DType dtype, uint32_t root,
                                   std::shared_ptr<Context> ctx) {
-    get_dtype_size(dtype);  // throws "unknown dtype" on this rank's own thread
-    MEGRAY_ASSERT(root < m_nranks, "root %u out of range", root);
-    VRANK_COLLECTIVE(Kind::kScatter, recvlen, dtype, MEGRAY_SUM, root);
+    // get_dtype_size throws "unknown dtype" (src/core/common.cpp:35-36)
+    VRANK_COLLECTIVE(kCollScatter, recvlen, dtype, MEGRAY_SUM, root, get_dtype_size(dtype); VRANK_ROOT_IN_RANGE);
 }
 
 Status VRankCommunicator::gather(const void* sendbuff, void* recvbuff, size_t sendlen, DType dtype, uint32_t root,
                                  std::shared_ptr<Context> ctx) {
-    get_dtype_size(dtype);
-    MEGRAY_ASSERT(root < m_nranks, "root %u out of range", root);
-    VRANK_COLLECTIVE(Kind::kGather, sendlen, dtype, MEGRAY_SUM, root);
+    VRANK_COLLECTIVE(kCollGather, sendlen, dtype, MEGRAY_SUM, root, get_dtype_size(dtype); VRANK_ROOT_IN_RANGE);
 }
 
 Status VRankCommunicator::all_to_all(const void* sendbuff, void* recvbuff, size_t len, DType dtype,
                                      std::shared_ptr<Context> ctx) {
-    get_dtype_size(dtype);
-    VRANK_COLLECTIVE(Kind::kAllToAll, len, dtype, MEGRAY_SUM, 0);
+    VRANK_COLLECTIVE(kCollAllToAll, len, dtype, MEGRAY_SUM, 0, get_dtype_size(dtype));
 }
 
 Status VRankCommunicator::all_gather(const void* sendbuff, void* recvbuff, size_t sendlen, DType dtype,
                                      std::shared_ptr<Context> ctx) {
-    get_dtype_size(dtype);
-    VRANK_COLLECTIVE(Kind::kAllGather, sendlen, dtype, MEGRAY_SUM, 0);
+    VRANK_COLLECTIVE(kCollAllGather, sendlen, dtype, MEGRAY_SUM, 0, get_dtype_size(dtype));
 }
 
 Status VRankCommunicator::all_reduce(const void* sendbuff, void* recvbuff, size_t len, DType dtype, ReduceOp op,
                                      std::shared_ptr<Context> ctx) {
-    reduce_elem_size(dtype);  // "unknown dtype", src/ucx/kernel.cu:95-96
-    check_reduce_op(op);      // "unknown reduce op", src/ucx/kernel.cu:55-56
-    VRANK_COLLECTIVE(Kind::kAllReduce, len, dtype, op, 0);
+    // "unknown dtype" and "unknown reduce op", src/ucx/kernel.cu:95-96 and :55-56
+    VRANK_COLLECTIVE(kCollAllReduce, len, dtype, op, 0, reduce_elem_size(dtype); check_reduce_op(op));
 }
 
 Status VRankCommunicator::reduce_scatter(const void* sendbuff, void* recvbuff, size_t recvlen, DType dtype,
                                          ReduceOp op, std::shared_ptr<Context> ctx) {
-    reduce_elem_size(dtype);
-    check_reduce_op(op);
-    VRANK_COLLECTIVE(Kind::kReduceScatter, recvlen, dtype, op, 0);
+    VRANK_COLLECTIVE(kCollReduceScatter, recvlen, dtype, op, 0, reduce_elem_size(dtype); check_reduce_op(op));
 }
 
 Status VRankCommunicator::broadcast(const void* sendbuff, void* recvbuff, size_t len, DType dtype, uint32_t root,
                                     std::shared_ptr<Context> ctx) {
-    get_dtype_size(dtype);
-    MEGRAY_ASSERT(root < m_nranks, "root %u out of range", root);
-    VRANK_COLLECTIVE(Kind::kBroadcast, len, dtype, MEGRAY_SUM, root);
+    VRANK_COLLECTIVE(kCollBroadcast, len, dtype, MEGRAY_SUM, root, get_dtype_size(dtype); VRANK_ROOT_IN_RANGE);
 }
 
 Status VRankCommunicator::reduce(const void* sendbuff, void* recvbuff, size_t len, DType dtype, ReduceOp op,
                                  uint32_t root, std::shared_ptr<Context> ctx) {
-    reduce_elem_size(dtype);
-    check_reduce_op(op);
-    MEGRAY_ASSERT(root < m_nranks, "root %u out of range", root);
     if (m_rank != root) recvbuff = nullptr;  // only the root's pointer means anything (test/test_opr.cpp:501-505)
-    VRANK_COLLECTIVE(Kind::kReduce, len, dtype, op, root);
+    VRANK_COLLECTIVE(kCollReduce, len, dtype, op, root, reduce_elem_size(dtype); check_reduce_op(op); VRANK_ROOT_IN_RANGE);
 }
 
 // Between group_start() and group_end() sends and receives are only collected; group_end() posts

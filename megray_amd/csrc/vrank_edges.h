@@ -1,0 +1,43 @@
+// Cross-stream ordering for the thread-per-rank API: small kernels that let the stream a collective
+// runs on wait for the other ranks' streams, and those wait for the collective.
+//
+// The reference orders its ranks with host-side synchronisation (cudaStreamSynchronize per ring
+// step, src/ucx/all_reduce.cpp:30,77) and with flags in shared memory that stream callbacks set and
+// a thread polls (src/shm/utils.cpp:71-95).  Here the flags live in device memory and the polling
+// is done by a one-wavefront kernel on the waiting stream, so the host never blocks:
+//
+//   arrive   (a rank's stream)     arrived += 1 once everything enqueued before it has finished
+//   wait     (the launch stream)   returns when arrived >= target: the inputs are ready
+//   notify   (the launch stream)   done = ticket, after the collective's launches
+//   wait     (a rank's stream)     returns when done >= ticket: the outputs are ready
+//
+// Every wait is enqueued after the kernel that satisfies it, so streams that share a hardware queue
+// cannot block each other; and every wait gives up after a time limit (counted in `timeouts`, which
+// the host reads back through `status`), so no wavefront spins for ever.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdint>
+
+namespace MegRay {
+namespace vrank {
+
+// Device-side words of one communicator group.
+struct EdgeWords {
+    uint64_t arrived;   // arrive kernels that have run since the group was formed
+    uint64_t done;      // ticket of the last collective whose launches have finished
+    uint64_t timeouts;  // waits that gave up
+    uint64_t reserved[5];
+};
+
+hipError_t edge_arrive(EdgeWords* words, hipStream_t stream);
+hipError_t edge_notify(EdgeWords* words, uint64_t ticket, hipStream_t stream);
+// `status` is host-visible memory: a wait that gives up adds 1 to it as well.
+hipError_t edge_wait_arrived(EdgeWords* words, uint64_t target, uint64_t limit_ticks, uint64_t* status,
+                             hipStream_t stream);
+hipError_t edge_wait_done(EdgeWords* words, uint64_t ticket, uint64_t limit_ticks, uint64_t* status,
+                          hipStream_t stream);
+
+}  // namespace vrank
+}  // namespace MegRay

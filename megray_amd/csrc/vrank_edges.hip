@@ -1,0 +1,61 @@
+#include "vrank_edges.h"
+
+#include <hip/hip_runtime.h>
+
+namespace MegRay {
+namespace vrank {
+
+namespace {
+
+__global__ void __launch_bounds__(64) edge_arrive_kernel(uint64_t* arrived) {
+    if (threadIdx.x == 0) __hip_atomic_fetch_add(arrived, uint64_t(1), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__global__ void __launch_bounds__(64) edge_notify_kernel(uint64_t* done, uint64_t ticket) {
+    if (threadIdx.x == 0) __hip_atomic_store(done, ticket, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// One lane polls `word` until it reaches `target` or `limit_ticks` of the constant-rate wall clock
+// have passed; the wavefront sleeps between polls.
+__global__ void __launch_bounds__(64) edge_wait_kernel(const uint64_t* word, uint64_t target, uint64_t limit_ticks,
+                                                       uint64_t* timeouts, uint64_t* status) {
+    if (threadIdx.x != 0) return;
+    const uint64_t begin = wall_clock64();
+    while (__hip_atomic_load(word, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < target) {
+        if (wall_clock64() - begin > limit_ticks) {
+            __hip_atomic_fetch_add(timeouts, uint64_t(1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_fetch_add(status, uint64_t(1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            return;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
+
+}  // namespace
+
+hipError_t edge_arrive(EdgeWords* words, hipStream_t stream) {
+    hipLaunchKernelGGL(edge_arrive_kernel, dim3(1), dim3(64), 0, stream, &words->arrived);
+    return hipGetLastError();
+}
+
+hipError_t edge_notify(EdgeWords* words, uint64_t ticket, hipStream_t stream) {
+    hipLaunchKernelGGL(edge_notify_kernel, dim3(1), dim3(64), 0, stream, &words->done, ticket);
+    return hipGetLastError();
+}
+
+hipError_t edge_wait_arrived(EdgeWords* words, uint64_t target, uint64_t limit_ticks, uint64_t* status,
+                             hipStream_t stream) {
+    hipLaunchKernelGGL(edge_wait_kernel, dim3(1), dim3(64), 0, stream, &words->arrived, target, limit_ticks,
+                       &words->timeouts, status);
+    return hipGetLastError();
+}
+
+hipError_t edge_wait_done(EdgeWords* words, uint64_t ticket, uint64_t limit_ticks, uint64_t* status,
+                          hipStream_t stream) {
+    hipLaunchKernelGGL(edge_wait_kernel, dim3(1), dim3(64), 0, stream, &words->done, ticket, limit_ticks,
+                       &words->timeouts, status);
+    return hipGetLastError();
+}
+
+}  // namespace vrank
+}  // namespace MegRay

@@ -30,6 +30,54 @@ void check_reduce_op(ReduceOp op) {
     if (op != MEGRAY_SUM && op != MEGRAY_MAX && op != MEGRAY_MIN) MEGRAY_THROW("unknown reduce op");
 }
 
+namespace {
+FoldOrder as_order(int order) {
+    if (order < 0 || order >= kOrderCount) MEGRAY_THROW("unknown fold order");
+    return static_cast<FoldOrder>(order);
+}
+Schedule as_schedule(int schedule) {
+    if (schedule < 0 || schedule >= kSchedCount) MEGRAY_THROW("unknown schedule");
+    return static_cast<Schedule>(schedule);
+}
+}  // namespace
+
+Status plan_collective(Plan& plan, int kind, const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks,
+                       size_t count, DType dt, int order, int schedule, uint32_t root) {
+    switch (kind) {
+        case kCollAllReduce:
+            // a ring hop stores its partial result in the element type: FLOAT16 would round N-1 times
+            if (as_schedule(schedule) == kSchedRing && dt == MEGRAY_FLOAT16)
+                MEGRAY_THROW("the ring schedule is not offered for FLOAT16 (it would round at every hop)");
+            return plan_all_reduce(plan, sendbuffs, recvbuffs, nranks, count, reduce_elem_size(dt), as_order(order),
+                                   as_schedule(schedule));
+        case kCollReduceScatter:
+            return plan_reduce_scatter(plan, sendbuffs, recvbuffs, nranks, count, reduce_elem_size(dt),
+                                       as_order(order), as_schedule(schedule));
+        case kCollAllGather:
+            return plan_all_gather(plan, sendbuffs, recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)));
+        case kCollAllToAll:
+            return plan_all_to_all(plan, sendbuffs, recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)));
+        case kCollScatter:
+            if (root >= nranks) MEGRAY_THROW("root out of range");
+            return plan_scatter(plan, sendbuffs[root], recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)), root);
+        case kCollGather:
+            if (root >= nranks) MEGRAY_THROW("root out of range");
+            return plan_gather(plan, sendbuffs, recvbuffs[root], nranks, count, uint32_t(get_dtype_size(dt)), root);
+        case kCollBroadcast:
+            if (root >= nranks) MEGRAY_THROW("root out of range");
+            return plan_broadcast(plan, sendbuffs[root], recvbuffs, nranks, count, uint32_t(get_dtype_size(dt)),
+                                  root);
+        case kCollReduce:
+            if (root >= nranks) MEGRAY_THROW("root out of range");
+            return plan_reduce(plan, sendbuffs, recvbuffs[root], nranks, count, reduce_elem_size(dt), as_order(order),
+                               root);
+        case kCollReduce2:
+            return plan_reduce2(plan, sendbuffs[0], sendbuffs[1], recvbuffs[0], count, reduce_elem_size(dt));
+        default:
+            MEGRAY_THROW("unknown collective");
+    }
+}
+
 Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCall>& calls) {
     calls.clear();
     calls.reserve(plan.steps.size());

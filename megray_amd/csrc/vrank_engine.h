@@ -31,6 +31,29 @@ struct KernelCall {
     const void* launch;
 };
 
+// Which collective a plan is for (the values of the C ABI's MRV_* selectors).
+enum CollectiveKind : int {
+    kCollAllReduce = 0,
+    kCollReduceScatter = 1,
+    kCollAllGather = 2,
+    kCollAllToAll = 3,
+    kCollScatter = 4,
+    kCollGather = 5,
+    kCollBroadcast = 6,
+    kCollReduce2 = 7,
+    kCollReduce = 8,
+};
+
+inline bool is_reduction(int kind) {
+    return kind == kCollAllReduce || kind == kCollReduceScatter || kind == kCollReduce || kind == kCollReduce2;
+}
+
+// Plans collective `kind` over the N rank buffers.  Contract violations (unknown dtype / op / order /
+// schedule / collective, root out of range) throw MegRay::Exception like the reference; shapes a
+// single pass cannot honour come back as MEGRAY_INVALID_ARGUMENT with plan_error() set.
+Status plan_collective(Plan& plan, int kind, const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks,
+                       size_t count, DType dtype, int order, int schedule, uint32_t root);
+
 // Enqueue every launch of `plan` on `stream`.
 Status execute(const Plan& plan, DType dtype, ReduceOp op, hipStream_t stream);
 // The same launches, resolved but not enqueued.

@@ -309,6 +309,10 @@ const char* plan_error() {
     return g_plan_error;
 }
 
+void set_plan_error(const char* text) {
+    std::snprintf(g_plan_error, sizeof(g_plan_error), "%s", text ? text : "");
+}
+
 void chunk_partition(uint64_t len, uint32_t nchunks, uint64_t* sizes, uint64_t* offsets) {
     const uint64_t quotient = len / nchunks, remainder = len % nchunks;
     uint64_t offset = 0;

@@ -89,6 +89,7 @@ Status plan_reduce(Plan& plan, const void* const* send, void* recv_root, uint32_
 Status plan_reduce2(Plan& plan, const void* i0, const void* i1, void* o, uint64_t len, uint32_t elem_size);
 
 const char* plan_error();  // text for the last MEGRAY_INVALID_ARGUMENT of this thread
+void set_plan_error(const char* text);  // lets a thread pass the text on to the threads it planned for
 
 }  // namespace vrank
 }  // namespace MegRay
