@@ -346,8 +346,10 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                 }
             } else if (step.kind == Step::kFlat) {
                 const FlatLaunch& L = step.flat;
+                const uint64_t tile = uint64_t(kThreads) * (kVecBytes / L.elem_size);  // elements per tile
                 for (uint32_t s = 0; s < L.nruns; ++s) {
-                    const FlatRun& fr = L.run[s];
+                    const uint64_t begin = s ? L.end[s - 1] : 0, end = L.end[s];
+                    const uint32_t start = L.meta[s] & 0xffu, out_first = (L.meta[s] >> 16) & 0xffu;
                     mrv_plan_run run;
                     std::memset(&run, 0, sizeof(run));
                     run.step = uint32_t(i);
@@ -357,17 +359,18 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.new_wins_ties = L.new_wins_ties;
                     run.vector = 2;
                     run.waves = L.waves;
-                    run.start = fr.start;
-                    run.dir = L.tree ? 0 : fr.dir;
-                    run.out_first = fr.out_first;
-                    run.tiles = L.tile_hi[s] - L.tile_lo[s];
-                    run.reads_recv = (collective == MRV_ALL_REDUCE && fr.start < nranks &&
-                                      L.in[fr.start] == recvbuffs[fr.start] && L.in[fr.start] != sendbuffs[fr.start])
+                    run.start = start;
+                    run.dir = L.tree ? 0 : int(int8_t((L.meta[s] >> 8) & 0xffu));
+                    run.out_first = out_first;
+                    const uint64_t lo = (begin + tile - 1) / tile, hi = end / tile;  // tiles wholly inside the run
+                    run.tiles = uint32_t(hi > lo ? hi - lo : 0);
+                    run.reads_recv = (collective == MRV_ALL_REDUCE && start < nranks && L.in[start] == recvbuffs[start] &&
+                                      L.in[start] != sendbuffs[start])
                                              ? 1
                                              : 0;
-                    run.in_begin = fr.begin;
-                    run.out_begin = fr.begin - uint64_t(fr.out_shift);
-                    run.count = fr.end - fr.begin;
+                    run.in_begin = begin;
+                    run.out_begin = begin - L.shift[s];
+                    run.count = end - begin;
                     emit(run);
                 }
             } else if (step.kind == Step::kTree) {

@@ -401,14 +401,27 @@ private:
             wait_needed = true;
             if (!m_words) HIP_CHECK(hipStreamWaitEvent(stream, m_arrive[r], 0));
         }
-        if (wait_needed && m_words)
-            HIP_CHECK(edge_wait_arrived(m_words, m_marks.load(std::memory_order_relaxed), m_limit_ticks, m_status, stream));
         m_shared_stream.store(static_cast<void*>(stream), std::memory_order_relaxed);
         m_shared_valid.store(one_stream, std::memory_order_release);
+        const uint64_t ticket = m_generation.load(std::memory_order_relaxed) + 1;
+        // A short flat launch waits for the marks and publishes its completion itself: two launches
+        // less on this thread, on which every rank is waiting.
+        FlatLaunch* hooked = nullptr;
+        if (m_words && !one_stream && cp->plan.steps.size() == 1 && cp->plan.steps[0].kind == Step::kFlat &&
+            cp->plan.steps[0].flat.waves == 1)
+            hooked = &cp->plan.steps[0].flat;
+        if (hooked) {
+            hooked->hooks = EdgeHooks{reinterpret_cast<uint64_t*>(m_words), m_status, m_limit_ticks};
+            hooked->hook_target = wait_needed ? m_marks.load(std::memory_order_relaxed) : 0;
+            hooked->hook_ticket = ticket;
+        } else if (wait_needed && m_words) {
+            HIP_CHECK(edge_wait_arrived(m_words, m_marks.load(std::memory_order_relaxed), m_limit_ticks, m_status, stream));
+        }
         for (const KernelCall& call : cp->calls) HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, stream));
         // the other ranks order their streams behind this point themselves (none has to if all share the stream)
-        if (!one_stream) {
-            const uint64_t ticket = m_generation.load(std::memory_order_relaxed) + 1;
+        if (hooked) {
+            hooked->hook_target = hooked->hook_ticket = 0;
+        } else if (!one_stream) {
             if (m_words) {
                 HIP_CHECK(edge_notify(m_words, ticket, stream));
             } else {
@@ -466,7 +479,7 @@ private:
     std::atomic<uint32_t> m_sleepers{0};
     alignas(64) std::atomic<uint32_t> m_arrived{0};     // ranks that have deposited their call
     alignas(64) std::atomic<uint64_t> m_generation{0};  // collectives released so far; parked ranks poll it
-    alignas(64) char m_pad = 0;
+    [[maybe_unused]] alignas(64) char m_pad[64] = {};  // keeps what follows off the polled line
     std::vector<hipEvent_t> m_arrive;  // per rank: "my buffers are ready", recorded by the rank itself
     hipEvent_t m_done = nullptr;       // recorded by the leader behind the collective
     std::vector<hipEvent_t> m_events;  // point-to-point transfers

@@ -28,7 +28,8 @@ struct EdgeWords {
     uint64_t arrived;   // arrive kernels that have run since the group was formed
     uint64_t done;      // ticket of the last collective whose launches have finished
     uint64_t timeouts;  // waits that gave up
-    uint64_t reserved[5];
+    uint64_t finished;  // workgroups of a launch that publishes `done` itself (EdgeHooks) that have stored
+    uint64_t reserved[4];
 };
 
 hipError_t edge_arrive(EdgeWords* words, hipStream_t stream);

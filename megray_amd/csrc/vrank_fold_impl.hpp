@@ -585,6 +585,51 @@ __global__ void __launch_bounds__(kThreads) fold_tree_kernel(const TreeLaunch L)
     if (el < L.count) static_cast<T*>(L.out)[el] = tree_element<T, OP, 0>(L, L.nranks, L.root, el);
 }
 
+// The run tables of a flat launch are kernel arguments read through scalar loads.  Written naively
+// (short-circuit conditions, one field at a time) every entry becomes a load of its own that the next
+// compare waits for, sixteen and more in a row; the helpers below fetch eight runs with a few wide
+// loads that are all in flight together, and only the tables the launch needs.
+struct RunBatch {
+    uint64_t begin0;    // where the first run of the batch begins
+    uint64_t end[8];
+    uint32_t meta[8];
+    uint64_t shift[8];
+    __device__ __forceinline__ uint64_t begin(uint32_t i) const { return i ? end[i - 1] : begin0; }
+};
+
+__device__ __forceinline__ RunBatch load_batch(const FlatLaunch& L, uint32_t base) {
+    RunBatch b;
+    b.begin0 = base ? L.end[base - 1] : 0;
+    __builtin_memcpy(b.end, &L.end[base], sizeof(b.end));
+    __builtin_memcpy(b.meta, &L.meta[base], sizeof(b.meta));
+    if (L.unshifted) {
+#pragma unroll
+        for (uint32_t i = 0; i < 8; ++i) b.shift[i] = 0;
+    } else {
+        __builtin_memcpy(b.shift, &L.shift[base], sizeof(b.shift));
+    }
+    return b;
+}
+__device__ __forceinline__ uint32_t meta_start(uint32_t meta) { return meta & 0xffu; }
+__device__ __forceinline__ int meta_dir(uint32_t meta) { return int(int8_t((meta >> 8) & 0xffu)); }
+__device__ __forceinline__ uint32_t meta_out_first(uint32_t meta) { return (meta >> 16) & 0xffu; }
+
+// The run that holds all of a tile, if there is one (everything here is uniform: scalar registers).
+struct TileRun {
+    bool covered = false;
+    uint32_t meta = 1u << 8;
+    uint64_t shift = 0;
+};
+__device__ __forceinline__ void uniform_scan(const RunBatch& b, uint64_t e_lo, uint64_t e_hi, TileRun& tr) {
+#pragma unroll
+    for (uint32_t i = 0; i < 8; ++i) {
+        const bool covers = (b.begin(i) <= e_lo) & (e_hi <= b.end[i]);  // unused entries end at 0
+        tr.covered = tr.covered | covers;
+        tr.meta = covers ? b.meta[i] : tr.meta;
+        tr.shift = covers ? b.shift[i] : tr.shift;
+    }
+}
+
 // One tile of a flat launch element by element: a tile that straddles a run border or the end of
 // the buffers.  One run at a time, so that ranks and destinations stay uniform.
 template <typename T, int OP, int K, bool TREE>
@@ -597,16 +642,14 @@ __device__ __forceinline__ void flat_tile_by_element(const FlatLaunch& L, uint32
     const uint64_t e_lo = uint64_t(tile) * TILE;
     const uint64_t e_hi = e_lo + TILE < L.count ? e_lo + TILE : L.count;
     for (uint32_t i = 0; i < L.nruns; ++i) {
-        // tile_lo = ceil(begin / TILE) and tile_hi >= floor(end / TILE): a run outside this window cannot
-        // touch the tile, and the two small tables are already in the scalar cache from the run lookup
-        if (L.tile_lo[i] > tile + 1 || L.tile_hi[i] < tile) continue;
-        const uint64_t b = L.run[i].begin > e_lo ? L.run[i].begin : e_lo;
-        const uint64_t e = L.run[i].end < e_hi ? L.run[i].end : e_hi;
+        const uint64_t run_begin = i ? L.end[i - 1] : 0, run_end = L.end[i];
+        const uint64_t b = run_begin > e_lo ? run_begin : e_lo;
+        const uint64_t e = run_end < e_hi ? run_end : e_hi;
         if (b >= e) continue;
-        const uint32_t start = L.run[i].start;
-        const int dir = L.run[i].dir;
-        const uint32_t out_first = L.run[i].out_first;
-        const uint64_t shift = uint64_t(L.run[i].out_shift);
+        const uint32_t start = meta_start(L.meta[i]);
+        const int dir = meta_dir(L.meta[i]);
+        const uint32_t out_first = meta_out_first(L.meta[i]);
+        const uint64_t shift = L.shift[i];
         for (uint32_t k = 0; k < EPV; ++k) {
             const uint64_t el = e_lo + uint64_t(tid) * EPV + k;
             if (el < b || el >= e) continue;
@@ -627,86 +670,149 @@ __device__ __forceinline__ void flat_tile_by_element(const FlatLaunch& L, uint32
     }
 }
 
+// What a lane knows about the run its own 16-byte vector lies in.
+struct LaneRun {
+    bool inside = false;  // the vector lies wholly inside one run (whose order and destinations follow)
+    bool cut = false;     // the vector is cut by a run border
+    uint32_t meta = 1u << 8;
+    uint32_t shift_lo = 0, shift_hi = 0;  // the run's out_shift: a whole number of vectors in a flat launch
+};
+
+// Eight runs against the lanes of tile `tile`, without branches (unused entries end at 0 and match
+// nothing).  A run's borders are clamped to the tile on the scalar side, so the per-lane part is 32-bit.
+template <typename T>
+__device__ __forceinline__ void lane_scan(const RunBatch& w, uint32_t tile, uint32_t tid, LaneRun& lr) {
+    constexpr uint32_t EPV = kVecBytes / sizeof(T);
+    constexpr uint32_t TILE = kThreads * EPV;
+    const uint64_t e_lo = uint64_t(tile) * TILE;
+    const uint32_t lane_off = tid * EPV;  // the lane's vector, in elements from the tile's start
+#pragma unroll
+    for (uint32_t i = 0; i < 8; ++i) {
+        const uint64_t b64 = w.begin(i) > e_lo ? w.begin(i) - e_lo : 0;
+        const uint64_t e64 = w.end[i] > e_lo ? w.end[i] - e_lo : 0;
+        const uint32_t b = uint32_t(b64 < TILE ? b64 : TILE), e = uint32_t(e64 < TILE ? e64 : TILE);
+        const bool holds = (lane_off >= b) & (lane_off + EPV <= e);
+        lr.cut = lr.cut | (!holds & (lane_off < e) & (lane_off + EPV > b));
+        lr.inside = lr.inside | holds;
+        lr.meta = holds ? w.meta[i] : lr.meta;
+        lr.shift_lo = holds ? uint32_t(w.shift[i]) : lr.shift_lo;
+        lr.shift_hi = holds ? uint32_t(w.shift[i] >> 32) : lr.shift_hi;
+    }
+}
+
 // A tile that lies inside the buffers but straddles run borders, its K input vectors staged in LDS
-// as staged[r][lane]: folded once per run that touches it, the inputs fetched from LDS in the run's
-// order (a rolled loop: the fold order is data here, not code, which keeps this rare path small in
-// code and registers); a lane whose vector lies wholly inside the run stores it with one 16-byte
-// store per destination.  The few lanes whose vector is cut by a run border (chunk lengths need not
-// be multiples of a vector) go element by element from global memory.
+// as staged[r][lane].  Every lane has looked up the run its own vector lies in (LaneRun) and folds
+// its vector in that run's order, fetching the inputs from LDS by rank: one straight pass whatever
+// the number of runs in the tile, which is what the smallest messages consist of (8 ranks x 4 KiB:
+// every tile holds two chunks).  The few lanes whose vector is cut by a run border (chunk lengths
+// need not be multiples of a vector) then go element by element from global memory, run by run.
 template <typename T, int OP, int K, bool TREE>
 __device__ __forceinline__ void flat_tile_across_runs(const FlatLaunch& L, uint32_t tile, uint32_t tid,
-                                                      const u32x4 (*staged)[kThreads]) {
+                                                      const u32x4 (*staged)[kThreads], const LaneRun& lr) {
     using A = typename Wide<T>::type;
     constexpr uint32_t EPV = kVecBytes / sizeof(T);
     constexpr uint32_t TILE = kThreads * EPV;
     const uint64_t e_lo = uint64_t(tile) * TILE, e_hi = e_lo + TILE;
     const uint64_t lane_lo = e_lo + uint64_t(tid) * EPV;
     const bool new_wins = L.new_wins_ties != 0;
-    for (uint32_t i = 0; i < L.nruns; ++i) {
-        // tile_lo = ceil(begin / TILE) and tile_hi >= floor(end / TILE): a run outside this window cannot
-        // touch the tile, and the two small tables are already in the scalar cache from the run lookup
-        if (L.tile_lo[i] > tile + 1 || L.tile_hi[i] < tile) continue;
-        const uint64_t b = L.run[i].begin > e_lo ? L.run[i].begin : e_lo;
-        const uint64_t e = L.run[i].end < e_hi ? L.run[i].end : e_hi;
-        if (b >= e) continue;
-        const uint32_t start = L.run[i].start;
-        const int dir = L.run[i].dir;
-        const uint32_t out_first = L.run[i].out_first;
-        const uint64_t shift = uint64_t(L.run[i].out_shift);  // a whole number of vectors in a flat launch
-        const bool inside = lane_lo >= b && lane_lo + EPV <= e;
-        const bool cut = !inside && lane_lo < e && lane_lo + EPV > b;
-        if (inside) {
-            u32x4 res;
-            if constexpr (TREE) {
-                u32x4 x[K];
+    const uint32_t nout = L.nout;
+    const uint32_t start = meta_start(lr.meta), out_first = meta_out_first(lr.meta);
+    const int dir = meta_dir(lr.meta);
+    const uint64_t shift = uint64_t(lr.shift_lo) | (uint64_t(lr.shift_hi) << 32);
+    if (lr.inside) {
+        u32x4 res;
+        if constexpr (TREE) {
+            u32x4 x[K];
 #pragma unroll
-                for (int r = 0; r < K; ++r) x[r] = staged[r][tid];
-                res = tree_from<T, OP, K>(x, start);
+            for (int r = 0; r < K; ++r) x[r] = staged[r][tid];
+            res = tree_from<T, OP, K>(x, start);
+        } else {
+            AccFor<T, OP> acc;
+            acc.seed(staged[start][tid]);
+#pragma unroll
+            for (uint32_t j = 1; j < uint32_t(K); ++j) acc.fold(staged[rotate_rank(start, dir, j, K)][tid], new_wins);
+            res = acc.finish();
+        }
+        const uint64_t out_el = lane_lo - shift;
+        if (nout == uint32_t(K) && L.unshifted) {
+            // all_reduce: every rank's copy of the tile, at the inputs' offset, with the stores of the main path
+            const uint64_t tile_off = e_lo * sizeof(T);
+#pragma unroll
+            for (int m = 0; m < K; ++m) store_tile_vec(static_cast<char*>(L.out[m]) + tile_off, tid, res);
+        } else {
+#pragma unroll 1
+            for (uint32_t m = 0; m < nout; ++m)
+                store_vec(reinterpret_cast<char*>(static_cast<T*>(L.out[rotate_rank(out_first, 1, m, K)]) + out_el), res);
+        }
+    }
+    if (!__builtin_amdgcn_ballot_w64(lr.cut)) return;
+    for (uint32_t i = 0; i < L.nruns; ++i) {
+        const uint64_t run_begin = i ? L.end[i - 1] : 0, run_end = L.end[i];
+        const uint64_t b = run_begin > e_lo ? run_begin : e_lo;
+        const uint64_t e = run_end < e_hi ? run_end : e_hi;
+        if (b >= e) continue;
+        const bool whole = lane_lo >= b && lane_lo + EPV <= e;
+        if (whole || lane_lo >= e || lane_lo + EPV <= b) continue;
+        const uint32_t rstart = meta_start(L.meta[i]);
+        const int rdir = meta_dir(L.meta[i]);
+        const uint32_t rout = meta_out_first(L.meta[i]);
+        const uint64_t rshift = L.shift[i];
+#pragma unroll 1
+        for (uint32_t k = 0; k < EPV; ++k) {
+            const uint64_t el = lane_lo + k;
+            if (el < b || el >= e) continue;
+            T r;
+            if constexpr (TREE) {
+                r = tree_element<T, OP, K>(L, K, rstart, el);
             } else {
-                AccFor<T, OP> acc;
-                acc.seed(staged[start][tid]);
+                A a = static_cast<A>(static_cast<const T*>(L.in[rstart])[el]);
 #pragma unroll 1
-                for (uint32_t j = 1; j < uint32_t(K); ++j) acc.fold(staged[rotate_rank(start, dir, j, K)][tid], new_wins);
-                res = acc.finish();
+                for (uint32_t j = 1; j < uint32_t(K); ++j)
+                    a = combine<OP, A>(
+                            a, static_cast<A>(static_cast<const T*>(L.in[rotate_rank(rstart, rdir, j, K)])[el]),
+                            new_wins);
+                r = static_cast<T>(a);
             }
 #pragma unroll 1
-            for (uint32_t m = 0; m < L.nout; ++m) {
-                T* dst = static_cast<T*>(L.out[rotate_rank(out_first, 1, m, K)]);
-                store_vec(reinterpret_cast<char*>(dst + (lane_lo - shift)), res);
-            }
-        } else if (cut) {
-#pragma unroll 1
-            for (uint32_t k = 0; k < EPV; ++k) {
-                const uint64_t el = lane_lo + k;
-                if (el < b || el >= e) continue;
-                T r;
-                if constexpr (TREE) {
-                    r = tree_element<T, OP, K>(L, K, start, el);
-                } else {
-                    A a = static_cast<A>(static_cast<const T*>(L.in[start])[el]);
-#pragma unroll 1
-                    for (uint32_t j = 1; j < uint32_t(K); ++j)
-                        a = combine<OP, A>(
-                                a, static_cast<A>(static_cast<const T*>(L.in[rotate_rank(start, dir, j, K)])[el]),
-                                new_wins);
-                    r = static_cast<T>(a);
-                }
-#pragma unroll 1
-                for (uint32_t m = 0; m < L.nout; ++m)
-                    static_cast<T*>(L.out[rotate_rank(out_first, 1, m, K)])[el - shift] = r;
-            }
+            for (uint32_t m = 0; m < nout; ++m)
+                static_cast<T*>(L.out[rotate_rank(rout, 1, m, K)])[el - rshift] = r;
         }
     }
 }
 
-// TREE selects the binomial-tree combination; it is a template parameter, not a run-time branch,
-// so that the tree's K live accumulators do not cost the left fold any registers.
+// Every lane polls the same word (one request per wavefront) until it reaches `target` or the time
+// limit passes; each lane's acquire keeps its own loads behind the wait.
+__device__ __forceinline__ void hook_wait(const EdgeHooks& h, uint64_t target) {
+    const uint64_t begin = wall_clock64();
+    while (__hip_atomic_load(h.words, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < target) {
+        if (wall_clock64() - begin > h.limit_ticks) {
+            if (threadIdx.x == 0) {
+                __hip_atomic_fetch_add(h.words + 2, uint64_t(1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_fetch_add(h.status, uint64_t(1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+            return;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
+
+// After a one-wavefront workgroup's stores: count it, and let the last one publish the ticket.
+__device__ __forceinline__ void hook_publish(const EdgeHooks& h, uint64_t ticket) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // this wavefront's stores before its count
+    if (threadIdx.x == 0) {
+        const uint64_t before = __hip_atomic_fetch_add(h.words + 3, uint64_t(1), __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        if (before + 1 == gridDim.x) {
+            __hip_atomic_store(h.words + 3, uint64_t(0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(h.words + 1, ticket, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+// One tile of a flat launch by one wavefront.
 template <typename T, int OP, int K, bool TREE>
-__global__ void __launch_bounds__(kThreads) fold_flat_kernel(const FlatLaunch L) {
+__device__ __forceinline__ void flat_tile(const FlatLaunch& L, uint32_t tile, uint32_t tid) {
     constexpr uint32_t EPV = kVecBytes / sizeof(T);
     constexpr uint32_t TILE = kThreads * EPV;  // elements per tile
-    const uint32_t tile = blockIdx.x;
-    const uint32_t tid = threadIdx.x;
     const uint64_t tile_off = uint64_t(tile) * (kThreads * kVecBytes);  // byte offset of the tile
     const bool whole = (uint64_t(tile) + 1) * TILE <= L.count;  // tile lies inside the buffer
 
@@ -716,22 +822,25 @@ __global__ void __launch_bounds__(kThreads) fold_flat_kernel(const FlatLaunch L)
         for (int r = 0; r < K; ++r) x[r] = load_tile_vec(static_cast<const char*>(L.in[r]) + tile_off, tid);
     }
 
-    // run lookup, eight runs per pair of scalar loads
-    int run = -1;
-    for (uint32_t base = 0; base < L.nruns; base += 8) {
-#pragma unroll
-        for (uint32_t i = 0; i < 8; ++i)
-            if (tile >= L.tile_lo[base + i] && tile < L.tile_hi[base + i]) run = int(base + i);
-    }
+    // Which run holds this tile?  Eight runs per round of scalar loads (one round for up to eight
+    // runs, which is every all_reduce of up to eight ranks in the ring order).
+    const uint64_t e_lo = uint64_t(tile) * TILE, e_hi = e_lo + TILE;
+    const RunBatch first = load_batch(L, 0);
+    TileRun tr;
+    uniform_scan(first, e_lo, e_hi, tr);
+    for (uint32_t base = 8; base < L.nruns && !tr.covered; base += 8) uniform_scan(load_batch(L, base), e_lo, e_hi, tr);
+    const bool covered = tr.covered;
+    const uint32_t meta = tr.meta;
+    const uint64_t shift = tr.shift;
     const bool new_wins = L.new_wins_ties != 0;
     const uint32_t nout = L.nout;
 
-    if (run >= 0) {
+    if (covered && whole) {
         // the whole tile shares one fold order (and lies inside the buffer)
-        const uint32_t start = L.run[run].start;
-        const int dir = L.run[run].dir;
-        const uint32_t out_first = L.run[run].out_first;
-        const uint64_t out_off = tile_off - uint64_t(L.run[run].out_shift) * sizeof(T);
+        const uint32_t start = meta_start(meta);
+        const int dir = meta_dir(meta);
+        const uint32_t out_first = meta_out_first(meta);
+        const uint64_t out_off = tile_off - shift * sizeof(T);
         u32x4 res;
         if constexpr (TREE) {
             res = tree_from<T, OP, K>(x, start);
@@ -749,14 +858,26 @@ __global__ void __launch_bounds__(kThreads) fold_flat_kernel(const FlatLaunch L)
     }
 
     if (whole) {
-        // each lane parks its vectors in LDS, where the runs' fold orders can index them
+        // each lane parks its vectors in LDS, where its own run's fold order can index them
         __shared__ u32x4 parked[K][kThreads];
 #pragma unroll
         for (int r = 0; r < K; ++r) parked[r][tid] = x[r];
-        flat_tile_across_runs<T, OP, K, TREE>(L, tile, tid, parked);
+        LaneRun lr;
+        lane_scan<T>(first, tile, tid, lr);
+        for (uint32_t base = 8; base < L.nruns; base += 8) lane_scan<T>(load_batch(L, base), tile, tid, lr);
+        flat_tile_across_runs<T, OP, K, TREE>(L, tile, tid, parked, lr);
     } else {
         flat_tile_by_element<T, OP, K, TREE>(L, tile, tid);
     }
+}
+
+// TREE selects the binomial-tree combination; it is a template parameter, not a run-time branch,
+// so that the tree's K live accumulators do not cost the left fold any registers.
+template <typename T, int OP, int K, bool TREE>
+__global__ void __launch_bounds__(kThreads) fold_flat_kernel(const FlatLaunch L) {
+    if (L.hook_target) hook_wait(L.hooks, L.hook_target);
+    flat_tile<T, OP, K, TREE>(L, blockIdx.x, threadIdx.x);
+    if (L.hook_ticket) hook_publish(L.hooks, L.hook_ticket);
 }
 
 // Group form of the flat fold for launches of many tiles.  A workgroup of kGroupWaves wavefronts
@@ -794,21 +915,15 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
             x[r] = u32x4{0u, 0u, 0u, 0u};  // never folded: such a tile goes element by element
     }
     // while the loads are in flight: which run does this wavefront's own tile lie in?
-    int run = -1;
-    for (uint32_t base = 0; base < L.nruns; base += 8) {
-#pragma unroll
-        for (uint32_t i = 0; i < 8; ++i)
-            if (mine >= L.tile_lo[base + i] && mine < L.tile_hi[base + i]) run = int(base + i);
+    TileRun tr;
+    {
+        const uint64_t e_lo = uint64_t(mine) * TILE;
+        for (uint32_t base = 0; base < L.nruns && !tr.covered; base += 8) uniform_scan(load_batch(L, base), e_lo, e_lo + TILE, tr);
     }
-    uint32_t start = 0, out_first = 0;
-    int dir = 1;
-    int64_t out_shift = 0;
-    if (run >= 0) {
-        start = L.run[run].start;
-        dir = L.run[run].dir;
-        out_first = L.run[run].out_first;
-        out_shift = L.run[run].out_shift;
-    }
+    const int run = tr.covered ? 0 : -1;
+    const uint32_t start = meta_start(tr.meta), out_first = meta_out_first(tr.meta);
+    const int dir = meta_dir(tr.meta);
+    const uint64_t out_shift = tr.shift;
 #pragma unroll
     for (int r = 0; r < K; ++r) stage[(wave + r) % W][r][tid] = x[r];
     __syncthreads();
@@ -826,13 +941,15 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
         if (exchange) {
             result[wave][tid] = res;
         } else {
-            const uint64_t out_off = uint64_t(mine) * (kThreads * kVecBytes) - uint64_t(out_shift) * sizeof(T);
+            const uint64_t out_off = uint64_t(mine) * (kThreads * kVecBytes) - out_shift * sizeof(T);
             for (uint32_t m = 0; m < L.nout; ++m)
                 store_tile_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, K)]) + out_off, tid, res);
         }
     } else if ((uint64_t(mine) + 1) * TILE <= L.count) {
         // inside the buffers but across run borders: from the staged vectors, stored by this wavefront
-        flat_tile_across_runs<T, OP, K, TREE>(L, mine, tid, stage[wave]);
+        LaneRun lr;
+        for (uint32_t base = 0; base < L.nruns; base += 8) lane_scan<T>(load_batch(L, base), mine, tid, lr);
+        flat_tile_across_runs<T, OP, K, TREE>(L, mine, tid, stage[wave], lr);
     } else if (mine < L.total_tiles) {
         flat_tile_by_element<T, OP, K, TREE>(L, mine, tid);  // the buffers' last, partial tile
     }

@@ -122,16 +122,9 @@ private:
         }
         for (size_t i = 0; i < m_runs.size(); ++i) {
             const Run& r = m_runs[i];
-            FlatRun& fr = L.run[i];
-            fr.begin = r.in_begin;
-            fr.end = r.in_begin + r.count;
-            fr.out_shift = int64_t(r.in_begin - r.out_begin);
-            fr.start = r.start;
-            fr.dir = r.dir;
-            fr.out_first = r.out_first;
-            const uint64_t lo = (fr.begin + tile - 1) / tile, hi = fr.end / tile;
-            L.tile_lo[i] = uint32_t(lo);
-            L.tile_hi[i] = uint32_t(hi > lo ? hi : lo);
+            L.end[i] = r.in_begin + r.count;
+            L.meta[i] = flat_meta(r.start, r.dir, r.out_first);
+            L.shift[i] = r.in_begin - r.out_begin;
         }
         L.count = expect;
         L.nranks = m_nranks;
@@ -147,6 +140,7 @@ private:
         for (const Run& r : m_runs) unshifted = unshifted && r.in_begin == r.out_begin;
         L.waves = total >= kGroupMinTiles ? kGroupWaves : 1;
         L.exchange = (L.waves == kGroupWaves && !m_tree && m_nout == m_nranks && unshifted) ? 1 : 0;
+        L.unshifted = unshifted ? 1 : 0;
         m_plan.steps.push_back(step);
         return true;
     }

@@ -47,40 +47,57 @@ struct FoldLaunch {
     uint32_t waves;          // wavefronts per workgroup: 1, or 4 for the group form (long vector bodies)
 };
 
+// Cross-stream ordering carried by a launch itself (thread-per-rank API, short launches): before it
+// reads, every workgroup waits until `arrived` has reached FlatLaunch::hook_target (the other ranks'
+// streams have got to the collective); after its stores, the last workgroup to finish publishes
+// FlatLaunch::hook_ticket in `done`.  The four words are the group's counters in device memory.
+struct EdgeHooks {
+    uint64_t* words;       // [0] arrived  [1] done  [2] timeouts  [3] workgroups finished
+    uint64_t* status;      // host-visible count of waits that gave up
+    uint64_t limit_ticks;  // a wait gives up after this many wall-clock ticks
+};
+
 constexpr uint32_t kMaxFlatRuns = 48;  // 2N chunks cut again at N-1 rank borders
 
-// One run of a flat launch: elements [begin, end) of the buffer, one fold order, one destination
-// set, outputs shifted by a whole number of 16-byte vectors.
-struct FlatRun {
-    uint64_t begin;
-    uint64_t end;
-    int64_t out_shift;  // output index = element index - out_shift
-    uint8_t start;
-    int8_t dir;
-    uint8_t out_first;
-    uint8_t pad[5];
-};
+// A flat run's fold order and destinations in one word: start | (dir & 0xff) << 8 | out_first << 16
+// (start: the rank whose buffer seeds the accumulator; dir +1 / -1; destinations are ranks
+// out_first .. out_first + nout - 1 mod nranks).
+constexpr uint32_t flat_meta(uint32_t start, int dir, uint32_t out_first) {
+    return (start & 0xffu) | ((uint32_t(dir) & 0xffu) << 8) | ((out_first & 0xffu) << 16);
+}
 
 // One launch of the flat fold kernel.  Tile t always covers bytes [1024 t, 1024 t + 1024) of every
 // input buffer, so a wavefront can issue its loads before it knows which run it is in; the run (and
 // with it the fold order) is looked up while the loads are in flight.  Needs nfold == nranks, all
-// buffers 16-byte aligned and every out_shift a multiple of a vector.
+// buffers 16-byte aligned, runs that tile [0, count) in order, and every shift a multiple of a vector.
+//
+// The layout serves the short launches, whose time is the latency of a few reads of this very
+// structure: a kernel-argument cache line that a wavefront touches for the first time costs about
+// 0.2 us on MI355X, so what every wavefront needs sits in as few 64-byte lines as possible (eight
+// input pointers, eight output pointers, the scalars, eight run ends, eight run words: five lines for
+// an all_reduce of eight ranks) and tables a launch does not need (shifts) are never read.
 struct FlatLaunch {
     const void* in[kMaxRanks];
     void* out[kMaxRanks];
-    uint32_t tile_lo[kMaxFlatRuns];  // tiles [tile_lo, tile_hi) lie wholly inside the run;
-    uint32_t tile_hi[kMaxFlatRuns];  // unused entries are 0, 0
-    FlatRun run[kMaxFlatRuns];
+    // one line of scalars
     uint64_t count;          // elements per input buffer
+    uint64_t hook_target;    // 0: do not wait (see EdgeHooks)
+    uint64_t hook_ticket;    // 0: do not publish
     uint32_t nranks;         // == fold width
     uint32_t nout;
     uint32_t nruns;
     uint32_t total_tiles;    // ceil(count * elem_size / 1024)
     uint32_t new_wins_ties;
     uint32_t elem_size;
-    uint32_t tree;  // 1: combine in binomial-tree order towards rank run.start instead of a left fold
+    uint32_t tree;  // 1: combine in binomial-tree order towards rank `start` instead of a left fold
     uint32_t waves;     // wavefronts per workgroup: 1, or kGroupWaves for the group form (launches of many tiles)
     uint32_t exchange;  // group form: 1 = every rank is an output at the inputs' offsets, results are exchanged too
+    uint32_t unshifted; // 1 = every run's outputs sit at the inputs' offsets (shift == 0 throughout)
+    // run i covers elements [end[i - 1], end[i]) (from 0 for the first); unused entries are 0
+    uint64_t end[kMaxFlatRuns];
+    uint32_t meta[kMaxFlatRuns];   // flat_meta() of the run
+    uint64_t shift[kMaxFlatRuns];  // output index = element index - shift
+    EdgeHooks hooks;               // one wavefront per tile only
 };
 
 // Group form of the flat fold: a workgroup of kGroupWaves wavefronts owns kGroupWaves tiles that lie
