@@ -244,6 +244,24 @@ MRV_API int mrv_comm_all_gather(mrv_comm* comm, const void* sendbuff, void* recv
                                 int dtype, void* stream);
 MRV_API int mrv_comm_all_reduce(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t len, int dtype,
                                 int op, void* stream);
+/*
+ * mrv_comm_all_reduce for callers that cannot allocate device memory (harnesses that forbid
+ * hipMalloc, tight serving loops).  No counterpart in the reference.  Same arguments, same result
+ * bit for bit.  mrv_comm_all_reduce orders the ranks' streams through counters it allocates at the
+ * group's first collective (hipMalloc + hipHostMalloc), or through events; this entry point keeps
+ * the counters in a 2 KiB array that is part of the library's device code (every GPU the library
+ * runs on holds its copy until the process ends), cut into 32 blocks of 64 bytes, one per
+ * communicator group.  It calls no hipMalloc / hipFree / hipHostMalloc / hipEventCreate.
+ *   - at most 32 groups per process can use it at the same time; the 33rd gets
+ *     MEGRAY_INVALID_USAGE ("every counter block of the static array is in use") on every rank;
+ *   - a group's first call clears its block (one synchronous 64-byte hipMemset): a block keeps what
+ *     the last group that held it left there;
+ *   - every rank of a group must make this same call (mixing it with mrv_comm_all_reduce in one
+ *     collective is rejected like any other mismatch); a group's collectives follow one another, so
+ *     its block is never used by two calls at once, and groups do not share blocks.
+ */
+MRV_API int mrv_comm_all_reduce_no_alloc(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t len,
+                                         int dtype, int op, void* stream);
 MRV_API int mrv_comm_reduce_scatter(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t recvlen,
                                     int dtype, int op, void* stream);
 MRV_API int mrv_comm_broadcast(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t len, int dtype,

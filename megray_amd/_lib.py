@@ -79,6 +79,7 @@ def load():
     L.mrv_comm_all_to_all.argtypes = [vp, vp, vp, sz, i32, vp]
     L.mrv_comm_all_gather.argtypes = [vp, vp, vp, sz, i32, vp]
     L.mrv_comm_all_reduce.argtypes = [vp, vp, vp, sz, i32, i32, vp]
+    L.mrv_comm_all_reduce_no_alloc.argtypes = [vp, vp, vp, sz, i32, i32, vp]
     L.mrv_comm_reduce_scatter.argtypes = [vp, vp, vp, sz, i32, i32, vp]
     L.mrv_comm_broadcast.argtypes = [vp, vp, vp, sz, i32, u32, vp]
     L.mrv_comm_reduce.argtypes = [vp, vp, vp, sz, i32, i32, u32, vp]
@@ -94,6 +95,7 @@ def load():
     for name in ("mrv_reduce_to_root", "mrv_get_free_port", "mrv_create_server", "mrv_comm_create",
                  "mrv_comm_init", "mrv_comm_configure", "mrv_comm_send", "mrv_comm_recv", "mrv_comm_scatter",
                  "mrv_comm_gather", "mrv_comm_all_to_all", "mrv_comm_all_gather", "mrv_comm_all_reduce",
+                 "mrv_comm_all_reduce_no_alloc",
                  "mrv_comm_reduce_scatter", "mrv_comm_broadcast", "mrv_comm_reduce", "mrv_comm_group_start",
                  "mrv_comm_group_end", "mrv_client_create", "mrv_client_connect", "mrv_client_barrier",
                  "mrv_client_broadcast", "mrv_client_allgather"):

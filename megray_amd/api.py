@@ -340,6 +340,12 @@ class Communicator:
         _check(_lib.load().mrv_comm_all_reduce(self._h, _ptr(sendbuff), _ptr(recvbuff), length, int(dtype),
                                                int(op), _stream(stream)))
 
+    def all_reduce_no_alloc(self, sendbuff, recvbuff, length, dtype, op, stream=None):
+        """all_reduce for callers that may not allocate device memory: the counters that order the ranks'
+        streams are a block of the library's static device array (mrv_comm_all_reduce_no_alloc)."""
+        _check(_lib.load().mrv_comm_all_reduce_no_alloc(self._h, _ptr(sendbuff), _ptr(recvbuff), length, int(dtype),
+                                                        int(op), _stream(stream)))
+
     def reduce_scatter(self, sendbuff, recvbuff, recvlen, dtype, op, stream=None):
         _check(_lib.load().mrv_comm_reduce_scatter(self._h, _ptr(sendbuff), _ptr(recvbuff), recvlen, int(dtype),
                                                    int(op), _stream(stream)))

@@ -534,6 +534,18 @@ int mrv_comm_all_reduce(mrv_comm* comm, const void* sendbuff, void* recvbuff, si
     COMM_CALL(all_reduce(sendbuff, recvbuff, len, static_cast<DType>(dtype), static_cast<ReduceOp>(op), ctx));
 }
 
+int mrv_comm_all_reduce_no_alloc(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t len, int dtype, int op,
+                                 void* stream) {
+    return guarded([&] {
+        need(comm, "comm is null");
+        auto* vr = dynamic_cast<VRankCommunicator*>(comm->comm.get());
+        if (!vr) MEGRAY_THROW("not a vrank communicator");
+        auto ctx = HipContext::make(as_stream(stream));
+        return vr->all_reduce_no_alloc(sendbuff, recvbuff, len, static_cast<DType>(dtype), static_cast<ReduceOp>(op),
+                                       ctx);
+    });
+}
+
 int mrv_comm_reduce_scatter(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t recvlen, int dtype, int op,
                             void* stream) {
     COMM_CALL(reduce_scatter(sendbuff, recvbuff, recvlen, static_cast<DType>(dtype), static_cast<ReduceOp>(op), ctx));

@@ -38,11 +38,32 @@ struct Call {
     int device;
     bool marked = false;    // the rank put a mark on its stream: everything enqueued before the call precedes it
     bool poisoned = false;  // the rank's own arguments were rejected; it does not take part
+    bool fixed = false;     // allocation-free call: the edge counters are a block of the library's static device array
 };
 
 bool same_collective(const Call& a, const Call& b) {
     return a.kind == b.kind && a.len == b.len && a.dtype == b.dtype && a.op == b.op && a.root == b.root &&
-           a.order == b.order && a.sched == b.sched && a.device == b.device;
+           a.order == b.order && a.sched == b.sched && a.device == b.device && a.fixed == b.fixed;
+}
+
+// Slots of the static counter array, handed out process-wide (a group keeps its slot while it lives).
+std::mutex g_slot_mutex;
+bool g_slot_taken[kStaticEdgeSlots] = {};
+
+int take_static_slot() {
+    std::lock_guard<std::mutex> lock(g_slot_mutex);
+    for (uint32_t i = 0; i < kStaticEdgeSlots; ++i) {
+        if (!g_slot_taken[i]) {
+            g_slot_taken[i] = true;
+            return int(i);
+        }
+    }
+    return -1;
+}
+
+void give_back_static_slot(int slot) {
+    std::lock_guard<std::mutex> lock(g_slot_mutex);
+    if (slot >= 0) g_slot_taken[slot] = false;
 }
 
 // A planned collective kept for the next call with the same arguments and buffers: training loops
@@ -89,8 +110,9 @@ public:
         for (hipEvent_t ev : m_arrive)
             if (ev) (void)hipEventDestroy(ev);
         if (m_done) (void)hipEventDestroy(m_done);
-        if (m_words) (void)hipFree(m_words);
-        if (m_status) (void)hipHostFree(m_status);
+        if (m_edges[0].words) (void)hipFree(m_edges[0].words);
+        if (m_edges[0].status) (void)hipHostFree(m_edges[0].status);
+        give_back_static_slot(m_fixed_slot);
     }
 
     // Groups are found by the 128-bit id rank 0 drew and the bootstrap broadcast.
@@ -126,8 +148,9 @@ public:
                             m_shared_stream.load(std::memory_order_relaxed) == static_cast<void*>(call.stream);
         const bool last = m_arrived.load(std::memory_order_acquire) == m_nranks - 1;
         if (!shared && !last) {
-            const Status st = mark(rank, call.stream);
-            if (st != MEGRAY_OK) return withdraw(rank, "a stream mark could not be enqueued", st);
+            const Status st = mark(rank, call.stream, call.fixed);
+            if (st != MEGRAY_OK)
+                return withdraw(rank, call.fixed && !m_edges[1].words ? m_fixed_error : "a stream mark could not be enqueued", st);
             call.marked = true;
         }
         return arrive(rank, call, true);
@@ -200,6 +223,7 @@ private:
             if (!m_poison_text[0]) std::snprintf(m_poison_text, sizeof(m_poison_text), "%s", text);
         }
         (void)arrive(rank, call, false);
+        set_plan_error(text);
         return st;
     }
 
@@ -209,7 +233,7 @@ private:
     // count reads every slot and launches, the others poll the generation.
     Status arrive(uint32_t rank, const Call& call, bool park) {
         m_slots[rank].call = call;
-        if (call.marked) m_marks.fetch_add(1, std::memory_order_relaxed);
+        if (call.marked) m_edges[call.fixed].marks.fetch_add(1, std::memory_order_relaxed);
         const uint64_t gen = m_generation.load(std::memory_order_relaxed);  // cannot move on before this rank arrives
         m_entered[rank] = gen + 1;
         if (m_arrived.fetch_add(1, std::memory_order_acq_rel) + 1 == m_nranks) {
@@ -260,7 +284,7 @@ private:
             set_plan_error(m_error[gen & 1]);
             return st;
         }
-        if (call.stream != m_lead_stream[gen & 1]) MEGRAY_CHECK(await_done(call.stream, gen + 1));
+        if (call.stream != m_lead_stream[gen & 1]) MEGRAY_CHECK(await_done(call.stream, gen + 1, call.fixed));
         return st;
     }
 
@@ -277,15 +301,26 @@ private:
     // operations and event calls are serialised across threads and cost 3 - 5 times as much on
     // MI355X).  MEGRAY_VRANK_EDGES=events in the environment keeps to event record / stream-wait-event,
     // which is also the fallback when the counters cannot be allocated.
+    bool wait_limit() {
+        int device = 0, khz = 0;
+        if (hipGetDevice(&device) != hipSuccess ||
+            hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, device) != hipSuccess || khz <= 0) {
+            (void)hipGetLastError();
+            return false;
+        }
+        // a wait gives up after this long (wall-clock ticks): long enough for any stream to drain,
+        // short enough that a lost mark does not hold a wavefront for ever
+        m_limit_ticks = env_u64("MEGRAY_VRANK_WAIT_LIMIT_MS", 10000) * uint64_t(khz);
+        return true;
+    }
+
     void prepare_edges() {
         std::call_once(m_edges_once, [&] {
             const char* choice = std::getenv("MEGRAY_VRANK_EDGES");
             if (choice && std::strcmp(choice, "events") == 0) return;
-            int device = 0, khz = 0;
             EdgeWords* words = nullptr;
             uint64_t* status = nullptr;
-            bool ok = hipGetDevice(&device) == hipSuccess &&
-                      hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, device) == hipSuccess && khz > 0;
+            bool ok = wait_limit();
             ok = ok && hipMalloc(reinterpret_cast<void**>(&words), sizeof(EdgeWords)) == hipSuccess;
             ok = ok && hipMemset(words, 0, sizeof(EdgeWords)) == hipSuccess;
             ok = ok && hipHostMalloc(reinterpret_cast<void**>(&status), sizeof(uint64_t), hipHostMallocDefault) == hipSuccess;
@@ -296,19 +331,47 @@ private:
                 return;
             }
             *status = 0;
-            // a wait gives up after this long (wall-clock ticks): long enough for any stream to drain,
-            // short enough that a lost mark does not hold a wavefront for ever
-            const uint64_t limit_ms = env_u64("MEGRAY_VRANK_WAIT_LIMIT_MS", 10000);
-            m_limit_ticks = limit_ms * uint64_t(khz);
-            m_status = status;
-            m_words = words;
+            m_edges[0].status = status;
+            m_edges[0].words = words;
         });
     }
 
-    Status mark(uint32_t rank, hipStream_t stream) {
-        prepare_edges();
-        if (m_words) {
-            HIP_CHECK(edge_arrive(m_words, stream));
+    // The counters of the allocation-free entry point: a block of the library's static device array,
+    // cleared once when the group takes it (a block keeps what its last user left).  Nothing is allocated.
+    void prepare_fixed_edges() {
+        std::call_once(m_fixed_once, [&] {
+            if (!wait_limit()) {
+                m_fixed_error = "the device's wall clock rate is unknown";
+                return;
+            }
+            m_fixed_slot = take_static_slot();
+            if (m_fixed_slot < 0) {
+                m_fixed_error = "every counter block of the static array is in use (32 communicator groups at a time)";
+                return;
+            }
+            EdgeWords* words = nullptr;
+            if (edge_static_words(uint32_t(m_fixed_slot), &words) != hipSuccess ||
+                hipMemset(words, 0, sizeof(EdgeWords)) != hipSuccess) {
+                (void)hipGetLastError();
+                m_fixed_error = "the static counter array could not be reached on this device";
+                return;
+            }
+            m_edges[1].words = words;
+        });
+    }
+
+    Status mark(uint32_t rank, hipStream_t stream, bool fixed) {
+        if (fixed) {
+            prepare_fixed_edges();
+            if (!m_edges[1].words) {
+                MEGRAY_ERROR("allocation-free collective: %s", m_fixed_error);
+                return MEGRAY_INVALID_USAGE;
+            }
+        } else {
+            prepare_edges();
+        }
+        if (m_edges[fixed].words) {
+            HIP_CHECK(edge_arrive(m_edges[fixed].words, stream));
             return MEGRAY_OK;
         }
         hipEvent_t& ev = m_arrive[rank];
@@ -317,9 +380,10 @@ private:
         return MEGRAY_OK;
     }
 
-    Status await_done(hipStream_t stream, uint64_t ticket) {
-        if (m_words) {
-            HIP_CHECK(edge_wait_done(m_words, ticket, m_limit_ticks, m_status, stream));
+    Status await_done(hipStream_t stream, uint64_t ticket, bool fixed) {
+        const EdgeSet& set = m_edges[fixed];
+        if (set.words) {
+            HIP_CHECK(edge_wait_done(set.words, ticket, m_limit_ticks, set.status, stream));
             return MEGRAY_OK;
         }
         HIP_CHECK(hipStreamWaitEvent(stream, m_done, 0));
@@ -354,8 +418,9 @@ private:
                 return MEGRAY_INVALID_USAGE;
             }
         }
-        if (m_status && *m_status != m_status_seen) {
-            m_status_seen = *m_status;
+        EdgeSet& set = m_edges[lead.fixed];
+        if (set.status && *set.status != set.status_seen) {
+            set.status_seen = *set.status;
             set_plan_error("a stream wait of an earlier collective gave up: a rank's stream did not get there in time");
             return MEGRAY_UNEXPECTED_ERR;
         }
@@ -395,11 +460,11 @@ private:
             // a rank that expected everyone on its stream did not mark it; it is parked in arrive(),
             // so its stream's tail is still the point it arrived at
             if (!other.marked) {
-                MEGRAY_CHECK(mark(r, other.stream));
-                m_marks.fetch_add(1, std::memory_order_relaxed);
+                MEGRAY_CHECK(mark(r, other.stream, lead.fixed));
+                set.marks.fetch_add(1, std::memory_order_relaxed);
             }
             wait_needed = true;
-            if (!m_words) HIP_CHECK(hipStreamWaitEvent(stream, m_arrive[r], 0));
+            if (!set.words) HIP_CHECK(hipStreamWaitEvent(stream, m_arrive[r], 0));
         }
         m_shared_stream.store(static_cast<void*>(stream), std::memory_order_relaxed);
         m_shared_valid.store(one_stream, std::memory_order_release);
@@ -407,23 +472,23 @@ private:
         // A short flat launch waits for the marks and publishes its completion itself: two launches
         // less on this thread, on which every rank is waiting.
         FlatLaunch* hooked = nullptr;
-        if (m_words && !one_stream && cp->plan.steps.size() == 1 && cp->plan.steps[0].kind == Step::kFlat &&
+        if (set.words && !one_stream && cp->plan.steps.size() == 1 && cp->plan.steps[0].kind == Step::kFlat &&
             cp->plan.steps[0].flat.waves == 1)
             hooked = &cp->plan.steps[0].flat;
         if (hooked) {
-            hooked->hooks = EdgeHooks{reinterpret_cast<uint64_t*>(m_words), m_status, m_limit_ticks};
-            hooked->hook_target = wait_needed ? m_marks.load(std::memory_order_relaxed) : 0;
+            hooked->hooks = EdgeHooks{reinterpret_cast<uint64_t*>(set.words), set.status, m_limit_ticks};
+            hooked->hook_target = wait_needed ? set.marks.load(std::memory_order_relaxed) : 0;
             hooked->hook_ticket = ticket;
-        } else if (wait_needed && m_words) {
-            HIP_CHECK(edge_wait_arrived(m_words, m_marks.load(std::memory_order_relaxed), m_limit_ticks, m_status, stream));
+        } else if (wait_needed && set.words) {
+            HIP_CHECK(edge_wait_arrived(set.words, set.marks.load(std::memory_order_relaxed), m_limit_ticks, set.status, stream));
         }
         for (const KernelCall& call : cp->calls) HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, stream));
         // the other ranks order their streams behind this point themselves (none has to if all share the stream)
         if (hooked) {
             hooked->hook_target = hooked->hook_ticket = 0;
         } else if (!one_stream) {
-            if (m_words) {
-                HIP_CHECK(edge_notify(m_words, ticket, stream));
+            if (set.words) {
+                HIP_CHECK(edge_notify(set.words, ticket, stream));
             } else {
                 if (!m_done) HIP_CHECK(hipEventCreateWithFlags(&m_done, hipEventDisableTiming));
                 HIP_CHECK(hipEventRecord(m_done, stream));
@@ -471,11 +536,19 @@ private:
     std::atomic<void*> m_shared_stream{nullptr};  // the stream of the last collective, ...
     std::atomic<bool> m_shared_valid{false};      // ... if every rank passed that same one
     std::once_flag m_edges_once;
-    EdgeWords* m_words = nullptr;    // device counters of the edge kernels; null: the events below are used instead
-    uint64_t* m_status = nullptr;    // host memory: waits that gave up
-    uint64_t m_status_seen = 0;
-    uint64_t m_limit_ticks = 0;
-    std::atomic<uint64_t> m_marks{0};  // arrive kernels enqueued so far = value `arrived` reaches when all have run
+    // Counters of the edge kernels.  [0]: allocated at the first collective (null: the events below are
+    // used instead).  [1]: a block of the library's static device array, for the allocation-free entry point.
+    struct EdgeSet {
+        EdgeWords* words = nullptr;
+        uint64_t* status = nullptr;  // host memory: waits that gave up
+        uint64_t status_seen = 0;
+        std::atomic<uint64_t> marks{0};  // arrive kernels enqueued so far = value `arrived` reaches when all have run
+    };
+    EdgeSet m_edges[2];
+    std::once_flag m_fixed_once;
+    int m_fixed_slot = -1;
+    const char* m_fixed_error = "";
+    std::atomic<uint64_t> m_limit_ticks{0};
     std::atomic<uint32_t> m_sleepers{0};
     alignas(64) std::atomic<uint32_t> m_arrived{0};     // ranks that have deposited their call
     alignas(64) std::atomic<uint64_t> m_generation{0};  // collectives released so far; parked ranks poll it
@@ -565,7 +638,8 @@ Status VRankCommunicator::do_init(BcastCallback cb) {
 
 // Argument checks run on the calling rank's own thread and throw there, like the reference's; the
 // group is told, so that the other ranks' calls come back instead of waiting for this one.
-#define VRANK_COLLECTIVE(KIND, LEN, DTYPE, OP, ROOT, CHECKS)                                    \
+#define VRANK_COLLECTIVE(KIND, LEN, DTYPE, OP, ROOT, CHECKS) VRANK_COLLECTIVE_ON(false, KIND, LEN, DTYPE, OP, ROOT, CHECKS)
+#define VRANK_COLLECTIVE_ON(FIXED, KIND, LEN, DTYPE, OP, ROOT, CHECKS)                          \
     do {                                                                                        \
         MEGRAY_ASSERT(m_group != nullptr, "communicator used before init()");                   \
         hipStream_t stream = nullptr;                                                           \
@@ -578,6 +652,7 @@ Status VRankCommunicator::do_init(BcastCallback cb) {
         }                                                                                       \
         Call call{KIND, LEN, DTYPE, OP, ROOT, m_order, m_sched, sendbuff, recvbuff, stream,     \
                   current_device()};                                                            \
+        call.fixed = FIXED;                                                                     \
         return m_group->collective(m_rank, call);                                               \
     } while (0)
 
@@ -608,6 +683,11 @@ Status VRankCommunicator::all_reduce(const void* sendbuff, void* recvbuff, size_
                                      std::shared_ptr<Context> ctx) {
     // "unknown dtype" and "unknown reduce op", src/ucx/kernel.cu:95-96 and :55-56
     VRANK_COLLECTIVE(kCollAllReduce, len, dtype, op, 0, reduce_elem_size(dtype); check_reduce_op(op));
+}
+
+Status VRankCommunicator::all_reduce_no_alloc(const void* sendbuff, void* recvbuff, size_t len, DType dtype,
+                                              ReduceOp op, std::shared_ptr<Context> ctx) {
+    VRANK_COLLECTIVE_ON(true, kCollAllReduce, len, dtype, op, 0, reduce_elem_size(dtype); check_reduce_op(op));
 }
 
 Status VRankCommunicator::reduce_scatter(const void* sendbuff, void* recvbuff, size_t recvlen, DType dtype,

@@ -43,6 +43,14 @@ public:
     Status group_start() override;
     Status group_end() override;
 
+    // Not part of the reference API: all_reduce for callers that may not allocate device memory
+    // (harnesses that forbid it, tight serving loops).  Same result as all_reduce(); the counters that
+    // order the ranks' streams are a block of the library's static device array instead of an
+    // allocation made at the group's first collective, and there is no fallback to events.  At most
+    // vrank::kStaticEdgeSlots groups per process can use it at a time; every rank of a group must make
+    // the same call.
+    Status all_reduce_no_alloc(const void* src, void* dst, size_t count, DType dtype, ReduceOp op, ContextPtr ctx);
+
     // Not part of the reference API: which reference loop's combination order all_reduce /
     // reduce_scatter / reduce reproduce (default: the ucx ring), and how all_reduce is laid out in
     // launches (default: fused).  Every rank of a group must choose the same.

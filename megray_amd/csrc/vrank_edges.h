@@ -32,9 +32,17 @@ struct EdgeWords {
     uint64_t reserved[4];
 };
 
+// Counters for callers that may not allocate: the library keeps a small array in device memory
+// (a file-scope variable of the code object, so every GPU the library runs on holds its own copy
+// until the process ends), cut into kStaticEdgeSlots counter blocks.  `edge_static_words` returns
+// block `slot` of the current device's copy; the address is looked up once per device and no memory
+// is allocated.  A block keeps what its last user left in it: whoever takes a slot clears it.
+constexpr uint32_t kStaticEdgeSlots = 32;
+hipError_t edge_static_words(uint32_t slot, EdgeWords** words);
+
 hipError_t edge_arrive(EdgeWords* words, hipStream_t stream);
 hipError_t edge_notify(EdgeWords* words, uint64_t ticket, hipStream_t stream);
-// `status` is host-visible memory: a wait that gives up adds 1 to it as well.
+// `status` is host-visible memory: a wait that gives up adds 1 to it as well (null: it does not).
 hipError_t edge_wait_arrived(EdgeWords* words, uint64_t target, uint64_t limit_ticks, uint64_t* status,
                              hipStream_t stream);
 hipError_t edge_wait_done(EdgeWords* words, uint64_t ticket, uint64_t limit_ticks, uint64_t* status,

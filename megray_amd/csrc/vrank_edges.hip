@@ -2,10 +2,21 @@
 
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 namespace MegRay {
 namespace vrank {
 
+// The counter blocks of groups that must not allocate.  In host code this name stands for the
+// variable, it is not a device address: the address of the current device's copy comes from
+// hipGetSymbolAddress (edge_static_words below) and is what kernels, clears and copies are given.
+static __device__ __align__(256) uint64_t scratch[kStaticEdgeSlots * (sizeof(EdgeWords) / sizeof(uint64_t))];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+uint64_t* g_scratch_base[kMaxDevices] = {};  // per device: where its copy of `scratch` lies
 
 __global__ void __launch_bounds__(64) edge_arrive_kernel(uint64_t* arrived) {
     if (threadIdx.x == 0) __hip_atomic_fetch_add(arrived, uint64_t(1), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
@@ -24,7 +35,7 @@ __global__ void __launch_bounds__(64) edge_wait_kernel(const uint64_t* word, uin
     while (__hip_atomic_load(word, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < target) {
         if (wall_clock64() - begin > limit_ticks) {
             __hip_atomic_fetch_add(timeouts, uint64_t(1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_fetch_add(status, uint64_t(1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            if (status) __hip_atomic_fetch_add(status, uint64_t(1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
             return;
         }
         __builtin_amdgcn_s_sleep(1);
@@ -32,6 +43,24 @@ __global__ void __launch_bounds__(64) edge_wait_kernel(const uint64_t* word, uin
 }
 
 }  // namespace
+
+hipError_t edge_static_words(uint32_t slot, EdgeWords** words) {
+    if (!words || slot >= kStaticEdgeSlots) return hipErrorInvalidValue;
+    *words = nullptr;
+    int device = 0;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return err;
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_base[device]) {
+        void* base = nullptr;
+        err = hipGetSymbolAddress(&base, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) return err;
+        g_scratch_base[device] = static_cast<uint64_t*>(base);
+    }
+    *words = reinterpret_cast<EdgeWords*>(g_scratch_base[device]) + slot;
+    return hipSuccess;
+}
 
 hipError_t edge_arrive(EdgeWords* words, hipStream_t stream) {
     hipLaunchKernelGGL(edge_arrive_kernel, dim3(1), dim3(64), 0, stream, &words->arrived);

@@ -788,7 +788,7 @@ __device__ __forceinline__ void hook_wait(const EdgeHooks& h, uint64_t target) {
         if (wall_clock64() - begin > h.limit_ticks) {
             if (threadIdx.x == 0) {
                 __hip_atomic_fetch_add(h.words + 2, uint64_t(1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_fetch_add(h.status, uint64_t(1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                if (h.status) __hip_atomic_fetch_add(h.status, uint64_t(1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
             }
             return;
         }
