@@ -9,13 +9,23 @@ with all buffers already resident in HBM.  Prints ONE JSON line:
   roofline   the fold kernel against the 8 TB/s HBM peak, timed with HIP events on the launch stream
   cpu_baseline  the reference tests' expected-value loop (test/test_opr.cpp:321-330) re-stated in the
              CPU oracle, timed on this host on a bounded sample of the same workload
+  comm_api_us   the same all_reduce at 4 KiB .. 1 MiB per rank through MegRay::Communicator::all_reduce,
+             one thread per rank (the reference's test/performance.cpp:103-137 harness shape), every
+             rank on a stream of its own and all ranks on one stream: microseconds per collective
+  small_msg_us  the same sizes through the flat C ABI (one caller, one stream)
+  other_configs the other benchmark configurations (reduce_scatter / all_gather fp16, MAX int32,
+             MIN int64, all_to_all uint8, SUM int8), each timed with HIP events
 
-Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--log2n 28] [--no-cpu] [--no-small]
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--log2n 28] [--no-cpu] [--no-small] [--no-comm]
+                       [--no-others]
 """
 import argparse
+import hashlib
 import json
 import os
+import subprocess
 import sys
+import tempfile
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -24,11 +34,34 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per launch of the fold kernel on the headline workload, from rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE runs scaled by the same counters on a plain copy of known size; the
-# summaries those figures come from are kept as text next to the kernel-trace summaries.
-# FETCH_SIZE counts 2 KiB per unit on this part (scale 1.99990), WRITE_SIZE 1 KiB (scale 1.00000).
-MEASURED_TRAFFIC_BYTES = {"all_reduce_f32_n8_2p28_fused": 17179591511}
+# HBM bytes per launch measured offline (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the same
+# counters on a plain copy of known size) are kept in a tracked file together with a hash of the kernel
+# sources they were measured on; a figure whose hash is not that of the sources in this tree is stale
+# and is not reported.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+KERNEL_SOURCES = ("vrank_fold_impl.hpp", "vrank_types.h", "vrank_kernels.hip")
+
+
+def kernel_source_hash():
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "megray_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(key):
+    """HBM bytes per launch of workload `key` from the tracked profile summary, or None if there is no
+    figure for the kernels as they are now."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        return None
+    entry = table.get("workloads", {}).get(key)
+    if not entry or table.get("kernel_source_hash") != kernel_source_hash():
+        return None
+    return entry.get("hbm_bytes_per_launch")
 
 
 def parse_args():
@@ -47,6 +80,8 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-small", action="store_true", help="skip the small-message sweep")
     ap.add_argument("--no-check", action="store_true", help="skip the correctness checks")
+    ap.add_argument("--no-comm", action="store_true", help="skip the thread-per-rank Communicator API leg")
+    ap.add_argument("--no-others", action="store_true", help="skip the other benchmark configurations")
     return ap.parse_args()
 
 
@@ -131,6 +166,33 @@ def small_message_sweep(torch, mr):
     return out
 
 
+def comm_api_sweep():
+    """all_reduce SUM fp32, 8 ranks, 4 KiB .. 1 MiB per rank through MegRay::Communicator::all_reduce, driven like
+    the reference's benchmark (test/performance.cpp:103-137): one thread per rank, 200 warm-up and 2000 timed
+    calls back to back, one stream sync at the end.  Runs the performance CLI as a child process (its threads
+    are C++ threads; this process has not touched the GPU yet).
+
+    avg_us     wall time of the 2000 calls including the final sync, per call (the reference's "time(us)")
+    median_us / p99_us   of the time from one call's return to the next call's return on rank 0
+    """
+    exe = os.path.join(ROOT, "megray_amd", "apps", "megray_performance")
+    if not os.path.exists(exe):
+        raise SystemExit("bench: megray_amd/apps/megray_performance is not built (python -m megray_amd.build)")
+    sizes = "4096,16384,65536,262144,1048576"
+    out = {}
+    for mode, flag in (("own_streams", []), ("shared_stream", ["-S"])):
+        with tempfile.NamedTemporaryFile("r", suffix=".jsonl") as tmp:
+            cmd = [exe, "-d", "8", "-f", "all_reduce", "-s", sizes, "-w", "200", "-i", "2000", "-J", tmp.name] + flag
+            proc = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+            if proc.returncode != 0:
+                raise SystemExit(f"bench: {' '.join(cmd)} failed:\n{proc.stdout}\n{proc.stderr}")
+            rows = [json.loads(line) for line in tmp.read().splitlines() if line.strip()]
+        out[mode] = {str(r["bufsize"]): {"avg_us": round(r["avg_us"], 2), "median_us": round(r["median_us"], 2),
+                                          "p99_us": round(r["p99_us"], 2)} for r in rows}
+    out["harness"] = "megray_performance -d 8 -f all_reduce -w 200 -i 2000 (thread per rank, MegRay::Communicator API)"
+    return out
+
+
 def copy_yardstick(torch, mr):
     """What this particular GPU sustains on the simplest streaming job, for context: a 1 GiB device copy
     through this library's copy kernel and through torch (GB/s, read + write)."""
@@ -197,12 +259,12 @@ def cpu_baseline(orc, np, nranks):
     }
 
 
-def run_other_workload(args, torch, mr):
-    """The non-headline workloads: same timing, one JSON line, no CPU / small-message legs."""
+def time_workload(w, torch, mr, steps, warmup):
+    """One of the non-headline workloads: builds its inputs in HBM, times `steps` collectives with HIP
+    events on the launch stream and returns the figures."""
     dev = "cuda:0"
     st = torch.cuda.current_stream()
     n8 = 8
-    w = args.workload
 
     def rnd(n, dtype, rank):
         from megray_amd import synth
@@ -244,42 +306,67 @@ def run_other_workload(args, torch, mr):
         step = lambda: mr.all_to_all(src, dst, blk, mr.DType.UINT8, stream=st)  # noqa: E731
         desc = (mr.Collective.ALL_TO_ALL, src, dst, blk, mr.DType.UINT8)
         text, dt = "all_to_all uint8, 8 ranks x 8 blocks of 16 MiB", "u8"
-    else:
+    elif w == "c5_sum_int8":
         n = 1 << 27
         src = [rnd(n, torch.int8, r) for r in range(n8)]
         dst = [torch.empty(n, dtype=torch.int8, device=dev) for _ in range(n8)]
         step = lambda: mr.all_reduce(src, dst, n, mr.DType.INT8, mr.ReduceOp.SUM, stream=st)  # noqa: E731
         desc = (mr.Collective.ALL_REDUCE, src, dst, n, mr.DType.INT8)
         text, dt = "all_reduce SUM int8 (wrap-around), 8 ranks x 2^27 elements", "i8"
+    else:
+        raise SystemExit(f"bench: unknown workload {w}")
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record(st)
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     e1.record(st)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     runs, bytes_read, bytes_written = mr.describe(desc[0], desc[1], desc[2], desc[3], desc[4])
     launches = max(1, len({r["step"] for r in runs}))
-    executed = bytes_read + bytes_written
-    kernel_ms = e0.elapsed_time(e1) / args.steps / launches
+    executed = bytes_read + bytes_written  # these workloads run in one pass: executed bytes = B_min
+    kernel_ms = e0.elapsed_time(e1) / steps / launches
     achieved = executed / launches / (kernel_ms * 1e-3) / 1e9
-    value = executed / (wall / args.steps) / 1e9
+    del src, dst
+    torch.cuda.empty_cache()
+    return {"workload": text, "dtype": dt, "launches": launches, "bytes": executed, "wall_s": wall,
+            "kernel_ms": kernel_ms, "achieved": achieved, "traffic": measured_traffic(w)}
+
+
+def run_other_workload(args, torch, mr):
+    """A non-headline workload on its own: same timing, one JSON line, no CPU / small-message legs."""
+    r = time_workload(args.workload, torch, mr, args.steps, args.warmup)
+    value = r["bytes"] / (r["wall_s"] / args.steps) / 1e9
     print(json.dumps({
         "metric": "achieved HBM GB/s (% of peak)", "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt, "data": "synthetic",
-        "config": {"workload": text, "launches_per_step": launches},
-        "pct_of_peak": round(100.0 * value / HBM_PEAK_GBPS, 2), "bytes_executed": executed,
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel_ms": round(kernel_ms, 4), "algorithmic_bytes_per_launch": executed // launches},
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(r["wall_s"] * 1e3 / args.steps, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": r["dtype"], "data": "synthetic",
+        "config": {"workload": r["workload"], "launches_per_step": r["launches"]},
+        "pct_of_peak": round(100.0 * value / HBM_PEAK_GBPS, 2), "bytes_executed": r["bytes"],
+        "roofline": {"bound": "hbm", "achieved": round(r["achieved"], 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(r["achieved"] / HBM_PEAK_GBPS, 4), "traffic": r["traffic"],
+                     "kernel_ms": round(r["kernel_ms"], 4),
+                     "algorithmic_bytes_per_launch": r["bytes"] // r["launches"]},
     }))
     return 0
+
+
+def other_configs(torch, mr):
+    """The other benchmark configurations, ten timed steps each: milliseconds per collective (HIP events),
+    GB/s on the collective's minimum bytes (which is what each of them executes) and that as a fraction of
+    the HBM peak."""
+    out = {}
+    for w in ("c2_reduce_scatter", "c2_all_gather", "c3_max_int32", "c3_min_int64", "c5_all_to_all", "c5_sum_int8"):
+        r = time_workload(w, torch, mr, 10, 2)
+        out[w] = {"workload": r["workload"], "ms": round(r["kernel_ms"] * r["launches"], 4),
+                  "gbps": round(r["achieved"], 1), "frac": round(r["achieved"] / HBM_PEAK_GBPS, 4),
+                  "bytes_min": r["bytes"], "traffic": r["traffic"]}
+    return out
 
 
 def main():
@@ -288,6 +375,10 @@ def main():
         print("bench.py: this build runs on ONE GPU; the N ranks are virtual ranks inside it "
               "(use --gpus 1, rank count is --ranks)", file=sys.stderr)
         return 2
+    headline = args.workload == "all_reduce"
+    # the thread-per-rank leg runs in a child process, before this process touches the GPU
+    comm_api = comm_api_sweep() if headline and not args.no_comm else None
+
     import numpy as np
     import torch
 
@@ -343,7 +434,7 @@ def main():
     achieved = (executed / launches) / (kernel_ms * 1e-3) / 1e9
     key = f"all_reduce_f32_n{nranks}_2p{args.log2n}_{args.schedule}"
     result = {
-        "metric": "achieved HBM GB/s (% of peak) for 8-rank fp32 SUM all_reduce; small-msg µs",
+        "metric": f"achieved HBM GB/s (% of peak) for {nranks}-rank fp32 SUM all_reduce; small-msg µs",
         "value": round(value, 1),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -366,7 +457,7 @@ def main():
         "bytes_executed": executed,
         "roofline": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(key),
+            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(key),
             "kernel": "fold_group_kernel<float, SUM, K=8>" if args.schedule == "fused" else "fold kernels (several)",
             "kernel_ms": round(kernel_ms, 4), "algorithmic_bytes_per_launch": executed // launches,
         },
@@ -379,6 +470,10 @@ def main():
     result["copy_yardstick"] = copy_yardstick(torch, mr)
     if not args.no_small:
         result["small_msg_us"] = small_message_sweep(torch, mr)
+    if comm_api is not None:
+        result["comm_api_us"] = comm_api
+    if not args.no_others:
+        result["other_configs"] = other_configs(torch, mr)
     if not args.no_cpu:
         import oracle as orc
         result["cpu_baseline"] = cpu_baseline(orc, np, nranks)
