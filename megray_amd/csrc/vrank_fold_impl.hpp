@@ -79,11 +79,14 @@ union VecOf {
     T v[kVecBytes / sizeof(T)];
 };
 
+// 128-bit accesses of single lanes.  The address needs 4-byte alignment only (buffers of 4- and
+// 8-byte elements at any element offset go 16 bytes per lane), which the pointer type says.
+typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 __device__ __forceinline__ u32x4 load_vec(const char* p) {
-    return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4_a4*>(p));
 }
 __device__ __forceinline__ void store_vec(char* p, u32x4 x) {
-    __builtin_nontemporal_store(x, reinterpret_cast<u32x4*>(p));
+    __builtin_nontemporal_store(u32x4_a4(x), reinterpret_cast<u32x4_a4*>(p));
 }
 
 // One tile (1 KiB) of a buffer through buffer instructions with explicit cache policies: measured
@@ -579,10 +582,43 @@ __device__ __forceinline__ T tree_element(const Launch& L, uint32_t n, uint32_t 
     return static_cast<T>(a[0]);
 }
 
+// The same tree on the 16-byte vector at byte offset `off` of up to kMaxRanks buffers, walked depth
+// first: the subtree of SPAN virtual ranks from v0 (v0 < count) is its left half combined with its
+// right half, if there is one.  That is the expression the rounds of the element-wise form build,
+// with at most log2(kMaxRanks) + 1 accumulators alive at a time.
+template <typename T, int OP, uint32_t SPAN>
+__device__ __forceinline__ TreeAccFor<T, OP> tree_node(const TreeLaunch& L, uint64_t off, uint32_t v0) {
+    if constexpr (SPAN == 1) {
+        TreeAccFor<T, OP> a;
+        a.seed(load_vec(static_cast<const char*>(L.in[rotate_rank(L.root, 1, v0, L.nranks)]) + off));
+        return a;
+    } else {
+        TreeAccFor<T, OP> left = tree_node<T, OP, SPAN / 2>(L, off, v0);
+        if (v0 + SPAN / 2 < L.nranks) left.merge(tree_node<T, OP, SPAN / 2>(L, off, v0 + SPAN / 2));
+        return left;
+    }
+}
+
+template <typename T, int OP>
+__device__ __forceinline__ u32x4 tree_vector(const TreeLaunch& L, uint64_t off) {
+    return tree_node<T, OP, kMaxRanks>(L, off, 0).finish();
+}
+
 template <typename T, int OP>
 __global__ void __launch_bounds__(kThreads) fold_tree_kernel(const TreeLaunch L) {
-    const uint64_t el = uint64_t(blockIdx.x) * kThreads + threadIdx.x;
-    if (el < L.count) static_cast<T*>(L.out)[el] = tree_element<T, OP, 0>(L, L.nranks, L.root, el);
+    constexpr uint32_t EPV = kVecBytes / sizeof(T);
+    const uint64_t lane = uint64_t(blockIdx.x) * kThreads + threadIdx.x;
+    if (!L.vector) {
+        if (lane < L.count) static_cast<T*>(L.out)[lane] = tree_element<T, OP, 0>(L, L.nranks, L.root, lane);
+        return;
+    }
+    const uint64_t nvec = L.count / EPV;
+    if (lane < nvec) store_vec(static_cast<char*>(L.out) + lane * kVecBytes, tree_vector<T, OP>(L, lane * kVecBytes));
+    // the elements behind the last whole vector: the first lanes of the last workgroup
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x < L.count % EPV) {
+        const uint64_t el = nvec * EPV + threadIdx.x;
+        static_cast<T*>(L.out)[el] = tree_element<T, OP, 0>(L, L.nranks, L.root, el);
+    }
 }
 
 // The run tables of a flat launch are kernel arguments read through scalar loads.  Written naively

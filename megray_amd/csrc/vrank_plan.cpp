@@ -63,6 +63,15 @@ public:
         m_aligned = m_grid >= kVecBytes;
         m_misalign = uint32_t(first_ptr & (m_grid - 1));  // offset of every base from the grid
         if (m_misalign % elem_size) m_aligned = false;
+        // Buffers whose offsets from a 16-byte boundary differ: the 128-bit accesses of gfx950 need
+        // 4-byte alignment only, so element types of 4 and 8 bytes (in naturally aligned buffers)
+        // still go 16 bytes per lane, every buffer at its own alignment.  Narrower types do not.
+        if (!m_aligned && elem_size >= 4) {
+            m_plain = true;
+            for (uint32_t r = 0; r < kMaxRanks; ++r)
+                for (const void* p : {m_in[r], static_cast<const void*>(m_out[r])})
+                    if (p && reinterpret_cast<uintptr_t>(p) % elem_size) m_plain = false;
+        }
     }
 
     void add_run(uint64_t in_begin, uint64_t out_begin, uint64_t count, uint8_t start, int8_t dir,
@@ -100,8 +109,8 @@ private:
     static bool flat_width(uint32_t n) { return n == 2 || n == 3 || n == 4 || n == 8; }
 
     bool emit_flat() {
-        if (!m_aligned || (m_misalign & (kVecBytes - 1)) || m_nfold != m_nranks || !flat_width(m_nranks) || m_runs.size() > kMaxFlatRuns)
-            return false;
+        const bool vectors = m_plain || (m_aligned && (m_misalign & (kVecBytes - 1)) == 0);
+        if (!vectors || m_nfold != m_nranks || !flat_width(m_nranks) || m_runs.size() > kMaxFlatRuns) return false;
         const uint64_t epv = kVecBytes / m_elem;
         const uint64_t tile = uint64_t(kThreads) * epv;  // elements per tile
         uint64_t expect = 0;
@@ -149,15 +158,16 @@ private:
         const uint64_t epv = kVecBytes / m_elem;
         // long vector bodies take the group form (four wavefronts per workgroup)
         uint64_t vector_elems = 0;
-        if (m_aligned)
-            for (const Run& r : m_runs)
-                if (r.in_begin % epv == r.out_begin % epv) vector_elems += r.count;
+        for (const Run& r : m_runs)
+            if (m_plain || (m_aligned && r.in_begin % epv == r.out_begin % epv)) vector_elems += r.count;
         m_waves = vector_elems / (kThreads * epv) >= kGroupMinTiles ? kGroupWaves : 1;
         open_launch();
         for (const Run& r : m_runs) {
-            const bool vector = m_aligned && (r.in_begin % epv == r.out_begin % epv);
+            const bool vector = m_plain || (m_aligned && (r.in_begin % epv == r.out_begin % epv));
             uint64_t head = 0, body = 0;
-            if (vector) {
+            if (m_plain) {
+                body = r.count / epv * epv;  // no grid to reach: every address is as aligned as it gets
+            } else if (vector) {
                 // the body starts where inputs and outputs both sit on the coarsest grid they share
                 uint64_t grid = m_grid;
                 const uint64_t skew = (r.in_begin - r.out_begin) * m_elem;  // unsigned wrap is fine mod 2^k
@@ -236,6 +246,7 @@ private:
     uint32_t m_nranks, m_nfold, m_nout, m_elem;
     bool m_new_wins;
     bool m_aligned;
+    bool m_plain = false;  // 16-byte accesses on buffers that are only element-aligned (4- and 8-byte types)
     uint32_t m_misalign = 0;
     uint64_t m_grid = kVecBytes;
     bool m_tree = false;
@@ -681,7 +692,13 @@ Status plan_reduce(Plan& plan, const void* const* send, void* recv_root, uint32_
         L.nranks = nranks;
         L.root = root;
         L.elem_size = elem_size;
-        const uint64_t tiles = (len + kThreads - 1) / kThreads;
+        // 16 bytes per lane where every address allows it: 16-byte aligned buffers, or element types of
+        // 4 and 8 bytes (whose 128-bit accesses need 4-byte alignment only)
+        uintptr_t bits = reinterpret_cast<uintptr_t>(recv_root);
+        for (uint32_t r = 0; r < nranks; ++r) bits |= reinterpret_cast<uintptr_t>(send[r]);
+        L.vector = ((bits & (kVecBytes - 1)) == 0 || (elem_size >= 4 && (bits & (elem_size - 1)) == 0)) ? 1 : 0;
+        const uint64_t lanes = L.vector ? std::max<uint64_t>(len / (kVecBytes / elem_size), 1) : len;
+        const uint64_t tiles = (lanes + kThreads - 1) / kThreads;
         if (tiles > 0x7fffffffull) return invalid("buffer too large for one tree launch");
         L.total_tiles = uint32_t(tiles);
         plan.steps.push_back(step);

@@ -119,7 +119,9 @@ struct TreeLaunch {
     uint32_t nranks;
     uint32_t root;
     uint32_t elem_size;
-    uint32_t total_tiles;  // kThreads elements per tile
+    uint32_t total_tiles;  // kThreads lanes per tile
+    uint32_t vector;       // 1: a lane takes a 16-byte vector (the last workgroup also the odd elements at the end);
+                           // 0: a lane takes one element
 };
 
 enum PackMode : uint32_t {
