@@ -112,6 +112,20 @@ def _ptr_array(bufs):
     return arr
 
 
+def _rank_arrays(sendbuffs, recvbuffs, nranks=None):
+    """The two per-rank pointer arrays of a flat call, both `nranks` long (the library indexes both up to
+    nranks): lists of different lengths are rejected here, like any other invalid argument; a shorter list is
+    allowed only where `nranks` says that its missing ranks are not used (root-only forms pad with None)."""
+    n = nranks if nranks is not None else len(sendbuffs)
+    if nranks is None and len(recvbuffs) != len(sendbuffs):
+        raise MegRayError(Status.INVALID_ARGUMENT,
+                          f"{len(sendbuffs)} send buffers but {len(recvbuffs)} receive buffers: one of each per rank")
+    if len(sendbuffs) > n or len(recvbuffs) > n:
+        raise MegRayError(Status.INVALID_ARGUMENT, f"more buffers than ranks ({n})")
+    pad = lambda bufs: list(bufs) + [None] * (n - len(bufs))  # noqa: E731
+    return _ptr_array(pad(sendbuffs)), _ptr_array(pad(recvbuffs)), n
+
+
 def _stream(stream):
     if stream is None:
         return None
@@ -135,22 +149,26 @@ def reduce(i0, i1, o, length, dtype, op, stream=None):
 
 def all_reduce(sendbuffs, recvbuffs, length, dtype, op, order=FoldOrder.UCX, schedule=Schedule.FUSED,
                stream=None):
-    _check(_lib.load().mrv_all_reduce(_ptr_array(sendbuffs), _ptr_array(recvbuffs), len(sendbuffs), length,
+    send, recv, nranks = _rank_arrays(sendbuffs, recvbuffs)
+    _check(_lib.load().mrv_all_reduce(send, recv, nranks, length,
                                       int(dtype), int(op), int(order), int(schedule), _stream(stream)))
 
 
 def reduce_scatter(sendbuffs, recvbuffs, recvlen, dtype, op, order=FoldOrder.UCX, stream=None):
-    _check(_lib.load().mrv_reduce_scatter(_ptr_array(sendbuffs), _ptr_array(recvbuffs), len(sendbuffs), recvlen,
+    send, recv, nranks = _rank_arrays(sendbuffs, recvbuffs)
+    _check(_lib.load().mrv_reduce_scatter(send, recv, nranks, recvlen,
                                           int(dtype), int(op), int(order), _stream(stream)))
 
 
 def all_gather(sendbuffs, recvbuffs, sendlen, dtype, stream=None):
-    _check(_lib.load().mrv_all_gather(_ptr_array(sendbuffs), _ptr_array(recvbuffs), len(sendbuffs), sendlen,
+    send, recv, nranks = _rank_arrays(sendbuffs, recvbuffs)
+    _check(_lib.load().mrv_all_gather(send, recv, nranks, sendlen,
                                       int(dtype), _stream(stream)))
 
 
 def all_to_all(sendbuffs, recvbuffs, length, dtype, stream=None):
-    _check(_lib.load().mrv_all_to_all(_ptr_array(sendbuffs), _ptr_array(recvbuffs), len(sendbuffs), length,
+    send, recv, nranks = _rank_arrays(sendbuffs, recvbuffs)
+    _check(_lib.load().mrv_all_to_all(send, recv, nranks, length,
                                       int(dtype), _stream(stream)))
 
 
@@ -196,12 +214,13 @@ def describe(collective, sendptrs, recvptrs, count, dtype, order=FoldOrder.UCX, 
              root=0, nranks=None):
     """Plan a collective on the host only.  -> (list of run dicts, bytes_read, bytes_written)"""
     nranks = nranks if nranks is not None else max(len(sendptrs), len(recvptrs))
+    send, recv, nranks = _rank_arrays(sendptrs, recvptrs, nranks)
     cap = 4096
     runs = (_lib.PlanRun * cap)()
     n = ctypes.c_size_t(0)
     br = ctypes.c_uint64(0)
     bw = ctypes.c_uint64(0)
-    _check(_lib.load().mrv_describe(int(collective), _ptr_array(sendptrs), _ptr_array(recvptrs), nranks, count,
+    _check(_lib.load().mrv_describe(int(collective), send, recv, nranks, count,
                                     int(dtype), int(order), int(schedule), root, runs, cap, ctypes.byref(n),
                                     ctypes.byref(br), ctypes.byref(bw)))
     out = []
@@ -220,7 +239,8 @@ class CollectivePlan:
         self._h = ctypes.c_void_p()
         self._keep = (sendbuffs, recvbuffs)
         nranks = nranks if nranks is not None else max(len(sendbuffs), len(recvbuffs))
-        _check(_lib.load().mrv_plan_create(int(collective), _ptr_array(sendbuffs), _ptr_array(recvbuffs), nranks,
+        send, recv, nranks = _rank_arrays(sendbuffs, recvbuffs, nranks)
+        _check(_lib.load().mrv_plan_create(int(collective), send, recv, nranks,
                                            count, int(dtype), int(op), int(order), int(schedule), root,
                                            1 if graph else 0, ctypes.byref(self._h)))
         self._launch = _lib.load().mrv_plan_launch

@@ -1,6 +1,7 @@
 // extern "C" face of the library (include/megray_vrank.h).
 #include "megray_vrank.h"
 
+#include <algorithm>
 #include <cstdio>
 #include <cstring>
 #include <exception>
@@ -389,6 +390,10 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                 emit(run);
             } else {
                 const PackLaunch& L = step.pack;
+                // the slice of every block this launch copies
+                const uint64_t per_tile = uint64_t(kThreads) * L.width;
+                const uint64_t slice_begin = L.first_tile * per_tile;
+                const uint64_t slice_bytes = std::min<uint64_t>(L.block_bytes - slice_begin, uint64_t(L.tiles_per_copy) * per_tile);
                 for (uint32_t c = 0; c < L.ncopies; ++c) {
                     mrv_plan_run run;
                     std::memset(&run, 0, sizeof(run));
@@ -400,7 +405,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.waves = L.waves;
                     run.dir = 1;
                     run.tiles = L.tiles_per_copy;
-                    run.count = L.block_bytes;
+                    run.count = slice_bytes;
                     if (L.mode == kPackAllToAll) {
                         run.start = c / L.nranks;
                         run.in_begin = uint64_t(c % L.nranks) * L.block_bytes;
@@ -429,6 +434,8 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                         run.out_first = L.root;
                         run.out_begin = uint64_t(c) * L.block_bytes;
                     }
+                    run.in_begin += slice_begin;
+                    run.out_begin += slice_begin;
                     emit(run);
                 }
             }

@@ -833,6 +833,8 @@ __device__ __forceinline__ void hook_wait(const EdgeHooks& h, uint64_t target) {
 }
 
 // After a one-wavefront workgroup's stores: count it, and let the last one publish the ticket.
+// (Only short launches do this: the release fence writes the L2 back, once per workgroup, and at
+// 2560 workgroups that alone took ten times as long as the fold.)
 __device__ __forceinline__ void hook_publish(const EdgeHooks& h, uint64_t ticket) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // this wavefront's stores before its count
     if (threadIdx.x == 0) {
@@ -989,16 +991,16 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
     } else if (mine < L.total_tiles) {
         flat_tile_by_element<T, OP, K, TREE>(L, mine, tid);  // the buffers' last, partial tile
     }
-    if (!exchange) return;
-    if (tid == 0) folded[wave] = run >= 0 ? 1u : 0u;
-    __syncthreads();
-
+    if (exchange) {
+        if (tid == 0) folded[wave] = run >= 0 ? 1u : 0u;
+        __syncthreads();
 #pragma unroll
-    for (int m = 0; m < K; ++m) {
-        const uint32_t k = (wave + m) % W;
-        if (folded[k]) {
-            const uint64_t tile = uint64_t(first) + k * kGroupStride;
-            store_tile_vec(static_cast<char*>(L.out[m]) + tile * (kThreads * kVecBytes), tid, result[k][tid]);
+        for (int m = 0; m < K; ++m) {
+            const uint32_t k = (wave + m) % W;
+            if (folded[k]) {
+                const uint64_t tile = uint64_t(first) + k * kGroupStride;
+                store_tile_vec(static_cast<char*>(L.out[m]) + tile * (kThreads * kVecBytes), tid, result[k][tid]);
+            }
         }
     }
 }

@@ -54,9 +54,9 @@ __device__ __forceinline__ PackEnds pack_ends(const PackLaunch& L, uint32_t copy
 template <typename W>
 __global__ void __launch_bounds__(kThreads) pack_kernel(const PackLaunch L) {
     const uint32_t copy = blockIdx.x / L.tiles_per_copy;
-    const uint32_t tile = blockIdx.x - copy * L.tiles_per_copy;
+    const uint64_t tile = L.first_tile + (blockIdx.x - copy * L.tiles_per_copy);
     const PackEnds e = pack_ends(L, copy);
-    const uint64_t base = uint64_t(tile) * kThreads * sizeof(W);
+    const uint64_t base = tile * kThreads * sizeof(W);
     const char* src = static_cast<const char*>(L.in[e.src_rank]) + e.src_block * L.block_bytes + base;
     const uint64_t dst_off = e.dst_block * L.block_bytes + base;
     const uint64_t left = (L.block_bytes - base) / sizeof(W);
@@ -94,13 +94,13 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
     const uint32_t wave = uint32_t(__builtin_amdgcn_readfirstlane(int(threadIdx.x / kThreads)));
     const uint32_t copy = blockIdx.x / L.groups_per_copy;
     const uint32_t group = blockIdx.x - copy * L.groups_per_copy;
-    const uint32_t first = (group / kGroupStride) * (W * kGroupStride) + group % kGroupStride;
+    const uint64_t first = L.first_tile + uint64_t(group / kGroupStride) * (W * kGroupStride) + group % kGroupStride;
     const PackEnds e = pack_ends(L, copy);
     const char* src = static_cast<const char*>(L.in[e.src_rank]) + e.src_block * L.block_bytes;
     const uint64_t dst_base = e.dst_block * L.block_bytes;
 
-    const uint32_t mine = first + wave * kGroupStride;
-    const uint64_t mine_off = uint64_t(mine) * kTileBytes;
+    const uint64_t mine = first + wave * kGroupStride;
+    const uint64_t mine_off = mine * kTileBytes;
     const bool whole = mine_off + kTileBytes <= L.block_bytes;
     u32x4 x = {0u, 0u, 0u, 0u};
     if (whole) {
@@ -124,7 +124,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
     for (uint32_t m = 0; m < e.ndst; ++m) {
         const uint32_t k = (wave + m) % W;
         if (staged[k]) {
-            const uint64_t off = (uint64_t(first) + k * kGroupStride) * kTileBytes;
+            const uint64_t off = (first + uint64_t(k) * kGroupStride) * kTileBytes;
             store_tile_vec(static_cast<char*>(L.out[e.dst_rank + m]) + dst_base + off, tid, stage[k][tid]);
         }
     }

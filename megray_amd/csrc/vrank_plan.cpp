@@ -553,13 +553,22 @@ Status add_pack(Plan& plan, const void* const* in, void* const* out, uint32_t nr
     L.width = common_width(block_bytes, in, out_c, nranks);
     const uint64_t per_tile = uint64_t(kThreads) * L.width;
     const uint64_t tiles = (block_bytes + per_tile - 1) / per_tile;
-    if (tiles * ncopies > 0x7fffffffull) return invalid("block too large for one pack launch");
-    L.tiles_per_copy = uint32_t(tiles);
     // long blocks of 16-byte accesses take the group form
     L.waves = (L.width == kVecBytes && tiles >= kGroupMinTiles / 4) ? kGroupWaves : 1;
-    L.groups_per_copy = group_grid(L.tiles_per_copy);
-    if (L.waves == kGroupWaves && uint64_t(L.groups_per_copy) * ncopies > 0x7fffffffull) L.waves = 1;
-    plan.steps.push_back(step);
+    // A grid holds 2^31 - 1 workgroups: blocks whose tiles, over all copies, outnumber that are cut into
+    // slices of tiles, one launch each (the reference's per-peer copies have no such limit either).
+    const uint64_t span = uint64_t(kGroupWaves) * kGroupStride;  // tiles a run of kGroupStride workgroups covers
+    uint64_t slice = 0x7fffffffull / ncopies;                    // workgroups per copy that fit one grid
+    if (L.waves == kGroupWaves) slice = slice / kGroupStride * span;  // in tiles, whole runs of workgroups
+    else slice = slice / span * span;
+    if (!slice) return invalid("too many block copies for one pack launch");
+    for (uint64_t first = 0; first < tiles; first += slice) {
+        const uint64_t take = std::min(slice, tiles - first);
+        L.first_tile = first;
+        L.tiles_per_copy = uint32_t(take);
+        L.groups_per_copy = group_grid(L.tiles_per_copy);
+        plan.steps.push_back(step);
+    }
     plan.bytes_read += block_bytes * ncopies;
     plan.bytes_written += block_bytes * ncopies;
     return MEGRAY_OK;

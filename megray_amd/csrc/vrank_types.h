@@ -146,6 +146,8 @@ struct PackLaunch {
     uint32_t width;   // bytes per lane access: 16, 8, 4, 2 or 1
     uint32_t waves;   // wavefronts per workgroup: 1, or kGroupWaves (16-byte accesses, long blocks)
     uint32_t groups_per_copy;  // group form: workgroups per block copy
+    uint64_t first_tile;  // the launch covers tiles [first_tile, first_tile + tiles_per_copy) of every copy (blocks
+                          // too long for one grid are cut into several launches; a multiple of the group span)
 };
 
 // Tile sizes of the one-wavefront-per-tile kernels.  Measured on MI355X: one 16-byte vector per lane and

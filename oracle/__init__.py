@@ -68,9 +68,10 @@ def lib():
         for name in ("orc_ucx_all_gather", "orc_ucx_all_to_all", "orc_shm_all_gather",
                      "orc_shm_all_to_all"):
             getattr(L, name).argtypes = [u32, pp, pp, sz, i32]
-        for name in ("orc_ucx_scatter", "orc_ucx_gather", "orc_ucx_broadcast"):
+        for name in ("orc_ucx_scatter", "orc_ucx_gather", "orc_ucx_broadcast", "orc_shm_broadcast"):
             getattr(L, name).argtypes = [u32, pp, pp, sz, i32, u32]
         L.orc_ucx_reduce.argtypes = [u32, pp, pp, sz, i32, i32, u32, vp, vp]
+        L.orc_shm_reduce.argtypes = [u32, pp, pp, sz, i32, i32, u32, vp, vp]
         L.orc_test_all_reduce_f32.restype = None
         L.orc_test_all_reduce_f32.argtypes = [u32, pp, pp, sz, i32]
         L.orc_test_reduce_scatter_f32.restype = None
@@ -216,6 +217,21 @@ def ucx_gather(sends, dtype, root):
 
 def ucx_broadcast(sends, dtype, root):
     return _run_copy("orc_ucx_broadcast", sends, sends[root].size, sends[root].size, dtype, root)
+
+
+def shm_reduce(sends, dtype, op, root, trace=False):
+    """Literal replay of src/shm/reduce.cpp:21-100.  Only recvs[root] is meaningful."""
+    n = len(sends)
+    recvs = [np.zeros(sends[0].size, dtype=sends[0].dtype) for _ in range(n)]
+    rc = lib().orc_shm_reduce(n, _ptrs(sends), _ptrs(recvs), sends[0].size, dtype, op, root,
+                              _trace_fn(trace), None)
+    _check(rc, "orc_shm_reduce")
+    return recvs
+
+
+def shm_broadcast(sends, dtype, root):
+    """Literal replay of src/shm/broadcast.cpp:19-51 (only sends[root] is read)."""
+    return _run_copy("orc_shm_broadcast", sends, sends[root].size, sends[root].size, dtype, root)
 
 
 def ucx_reduce(sends, dtype, op, root, trace=False):

@@ -494,6 +494,86 @@ int orc_shm_reduce_scatter(uint32_t N, const void* const* send, void* const* rec
     return rc;
 }
 
+/*
+ * src/shm/reduce.cpp:21-100, replayed with its own bookkeeping.  Every rank m seeds the accumulator
+ * area A with its k = 2 chunks (:55-58), then runs i = k .. chunks-1 (:73-93): before step i it spins
+ * until the right neighbour's mutex has reached i - k (:75-76, an unsigned comparison: the `int` is
+ * converted), stages chunk `work_rank` of its own sendbuff in S and runs
+ * cpu_reduce(A[w], A[w], S[w]) (:83-86), publishes mutex[m] = i - 1 (:87) and moves to the next
+ * chunk; work_rank starts at ring_add(m * k, k, chunks) (:65).  The root then reads all of A
+ * (:95-99).  The ranks run concurrently in the reference; here they are stepped one at a time,
+ * highest rank first, each taking a step whenever its wait condition holds - any interleaving the
+ * mutexes allow gives the same result, and this one differs from the rank-ascending, step-outermost
+ * order of shm_fold above.
+ */
+int orc_shm_reduce(uint32_t N, const void* const* send, void* const* recv, size_t len, int dtype,
+                   int op, uint32_t root, orc_reduce2_fn fn, void* user) {
+    size_t size = orc_dtype_size(dtype);
+    if (!size || !N || root >= N) return ORC_BAD_ARG;
+    size_t k = 2, chunks = (size_t)N * k;
+    size_t* sizes = (size_t*)malloc(sizeof(size_t) * chunks * 2);
+    size_t* offs = sizes + chunks;
+    orc_chunk_partition(len, chunks, sizes, offs);
+    char* A = (char*)xalloc(len * size);
+    char* S = (char*)xalloc(len * size);
+    int* mutex = (int*)malloc(sizeof(int) * N);
+    size_t* step = (size_t*)malloc(sizeof(size_t) * N * 2);
+    size_t* work = step + N;
+    int rc = ORC_OK;
+    for (uint32_t m = 0; m < N; m++) {
+        size_t seeded = 0;
+        for (size_t j = 0; j < k; j++) seeded += sizes[m * k + j];
+        memcpy(A + offs[m * k] * size, (const char*)send[m] + offs[m * k] * size, seeded * size);
+        mutex[m] = 0;
+        step[m] = k;
+        work[m] = orc_ring_add((uint32_t)(m * k), (uint32_t)k, (uint32_t)chunks);
+    }
+    for (int progress = 1; progress && rc == ORC_OK;) {
+        progress = 0;
+        for (uint32_t back = 0; back < N && rc == ORC_OK; back++) {
+            uint32_t m = N - 1 - back;
+            if (step[m] >= chunks) continue;
+            uint32_t right = orc_ring_add(m, 1, N);
+            if ((size_t)mutex[right] < step[m] - k) continue; /* still spinning at :75-76 */
+            size_t w = work[m];
+            memcpy(S + offs[w] * size, (const char*)send[m] + offs[w] * size, sizes[w] * size);
+            rc = shm_reduce2(fn, user, A + offs[w] * size, A + offs[w] * size, S + offs[w] * size,
+                             sizes[w], dtype, op);
+            mutex[m] = (int)(step[m] - 1);
+            work[m] = orc_ring_add((uint32_t)w, 1, (uint32_t)chunks);
+            step[m]++;
+            progress = 1;
+        }
+    }
+    for (uint32_t m = 0; m < N && rc == ORC_OK; m++)
+        if (step[m] < chunks) rc = ORC_BAD_ARG; /* a wait that never ends: cannot happen */
+    if (rc == ORC_OK) memcpy(recv[root], A, len * size);
+    free(step);
+    free(mutex);
+    free(S);
+    free(A);
+    free(sizes);
+    return rc;
+}
+
+/*
+ * src/shm/broadcast.cpp:19-51: the root copies its sendbuff into the arena and into its own recvbuff
+ * (:32-38); after the barrier every other rank copies the arena into its recvbuff (:43-46).
+ */
+int orc_shm_broadcast(uint32_t N, const void* const* send, void* const* recv, size_t len, int dtype,
+                      uint32_t root) {
+    size_t size = orc_dtype_size(dtype);
+    if (!size || !N || root >= N) return ORC_BAD_ARG;
+    size_t bytes = len * size;
+    char* arena = (char*)xalloc(bytes);
+    memcpy(arena, send[root], bytes);
+    memmove(recv[root], send[root], bytes);
+    for (uint32_t m = 0; m < N; m++)
+        if (m != root) memcpy(recv[m], arena, bytes);
+    free(arena);
+    return ORC_OK;
+}
+
 /* src/shm/all_gather.cpp:28-55: slot `rank` of the arena <- sendbuff; everybody reads the arena. */
 int orc_shm_all_gather(uint32_t N, const void* const* send, void* const* recv, size_t sendlen,
                        int dtype) {

@@ -97,6 +97,11 @@ int orc_shm_all_reduce(uint32_t nranks, const void* const* send, void* const* re
                        int dtype, int op, orc_reduce2_fn fn, void* user);
 int orc_shm_reduce_scatter(uint32_t nranks, const void* const* send, void* const* recv,
                            size_t recvlen, int dtype, int op, orc_reduce2_fn fn, void* user);
+/* Only recv[root] is written. */
+int orc_shm_reduce(uint32_t nranks, const void* const* send, void* const* recv, size_t len, int dtype,
+                   int op, uint32_t root, orc_reduce2_fn fn, void* user);
+int orc_shm_broadcast(uint32_t nranks, const void* const* send, void* const* recv, size_t len, int dtype,
+                      uint32_t root);
 int orc_shm_all_gather(uint32_t nranks, const void* const* send, void* const* recv, size_t sendlen,
                        int dtype);
 int orc_shm_all_to_all(uint32_t nranks, const void* const* send, void* const* recv, size_t len,

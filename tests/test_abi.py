@@ -131,3 +131,17 @@ def test_device_code_has_no_packed_fp32_instructions(tmp_path):
     assert text.count("v_add_f32") > 100, "the fp32 kernels are not in this file"
     for bad in ("v_pk_add_f32", "v_pk_mul_f32", "v_pk_fma_f32"):
         assert bad not in text, f"{bad} in the generated code"
+
+
+def test_python_wrappers_reject_lists_of_different_lengths():
+    """The library indexes both per-rank arrays up to nranks: the Python mirror refuses a call whose two lists
+    differ in length before anything reaches the C side, and pads the root-only forms it builds itself."""
+    import megray_amd as mr
+    with pytest.raises(mr.MegRayError, match="one of each per rank"):
+        mr.all_reduce([0x1000, 0x2000, 0x3000], [0x4000, 0x5000], 4, mr.DType.FLOAT32, mr.ReduceOp.SUM)
+    with pytest.raises(mr.MegRayError, match="one of each per rank"):
+        mr.all_to_all([0x1000], [0x4000, 0x5000], 4, mr.DType.UINT8)
+    # describe() with a shorter list: the missing ranks' entries are null, not read past the end
+    runs, _, _ = mr.describe(mr.Collective.GATHER, [0x100000, 0x200000, 0x300000], [None, 0x900000], 16,
+                             mr.DType.UINT8, root=1)
+    assert len(runs) == 3 and all(r["out_first"] == 1 for r in runs)

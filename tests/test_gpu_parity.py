@@ -17,6 +17,8 @@ from gpu_util import (bits_equal, empty_device, first_mismatch, rand_array, to_d
 REDUCE_TYPES = [orc.INT8, orc.UINT8, orc.INT32, orc.UINT32, orc.INT64, orc.UINT64, orc.FLOAT16,
                 orc.FLOAT32, orc.FLOAT64]
 OPS = [orc.SUM, orc.MAX, orc.MIN]
+# the types cpu_reduce() has a loop for (src/shm/utils.cpp:39-69); the shm replays throw for the others
+SHM_REDUCE_TYPES = [orc.INT8, orc.UINT8, orc.INT32, orc.UINT32, orc.INT64, orc.FLOAT32]
 ORDERS = [orc.ORDER_UCX, orc.ORDER_SHM, orc.ORDER_RANK0]
 
 
@@ -358,8 +360,11 @@ def check_pack_collectives(dtype, nranks, length, misalign, rng):
     mr.gather(d_in, d_root, length, dtype, root)
     torch.cuda.synchronize()
     assert_same(to_host(d_root, npdt), want, f"gather dtype={dtype} N={nranks} len={length}")
-    # broadcast
+    # broadcast (the ucx tree of src/ucx/broadcast.cpp:21-76 and the shm arena of src/shm/broadcast.cpp:19-51 agree)
     want = orc.ucx_broadcast(parts, dtype, root)
+    want_shm = orc.shm_broadcast(parts, dtype, root)
+    for r in range(nranks):
+        assert_same(want_shm[r], want[r], "the two broadcast replays")
     d_root = to_device(parts[root], misalign)
     d_out = [empty_device(length * size, misalign) for _ in range(nranks)]
     mr.broadcast(d_root, d_out, length, dtype, root)
@@ -465,8 +470,11 @@ def test_reduce_to_root(dtype):
                         d_out = empty_device(length * size)
                         mr.reduce_to_root(d_in, d_out, length, dtype, op, root, order)
                         torch.cuda.synchronize()
-                        assert_same(to_host(d_out, ins[0].dtype), orc.fold_all_reduce(ins, dtype, op, order)[0],
-                                    f"reduce order={order}")
+                        got = to_host(d_out, ins[0].dtype)
+                        assert_same(got, orc.fold_all_reduce(ins, dtype, op, order)[0], f"reduce order={order}")
+                        if order == orc.ORDER_SHM and dtype in SHM_REDUCE_TYPES:
+                            # the literal replay of src/shm/reduce.cpp:21-100, mutexes and all
+                            assert_same(got, orc.shm_reduce(ins, dtype, op, root)[root], "reduce vs shm replay")
 
 
 def test_planned_collectives_and_graph_replay():

@@ -438,3 +438,79 @@ def test_reduce_scatter_then_all_gather_is_all_reduce_in_same_order():
         ag = orc.ucx_all_gather(rs, orc.FLOAT32)
         ar = orc.fold_all_reduce(ins, orc.FLOAT32, orc.SUM, order)
         assert all(bits_equal(ag[r], ar[r]) for r in range(n))
+
+
+# ----------------------------------------------------------------------------- shm rooted collectives
+
+@pytest.mark.parametrize("nranks", [1, 2, 3, 4, 5, 7, 8, 9, 15])
+def test_shm_reduce_replay_has_the_shm_fold_order(nranks):
+    """src/shm/reduce.cpp:21-100 replayed with its mutexes: the order the operands of every chunk meet in,
+    read off a tracing reduce, is the 2N-chunk descending order of the shm all_reduce (owner w // 2 first,
+    then w // 2 - 1, ...), the accumulator being cpu_reduce's first argument; only the root's buffer is
+    written."""
+    n = nranks
+    want = expected_orders(n)["shm"]
+    for length in (n, 2 * n, 4 * n + 3, 2 * n + 1, 1):
+        ins = [np.full(length, r + 1, dtype=np.uint64) for r in range(n)]
+        for root in sorted({0, n // 2, n - 1}):
+            outs = orc.shm_reduce(ins, orc.UINT64, orc.SUM, root, trace=True)
+            sizes, offs = orc.chunk_partition(length, 2 * n)
+            for w in range(2 * n):
+                for e in range(offs[w], offs[w] + sizes[w]):
+                    assert digits(int(outs[root][e])) == want[w]  # concat(acc, new)
+            for r in range(n):
+                if r != root:
+                    assert not outs[r].any()
+
+
+def test_shm_reduce_replay_equals_the_chunk_fold_and_the_reference_vectors():
+    rng = np.random.default_rng(77)
+    for dtype in (orc.FLOAT32, orc.INT32, orc.UINT8, orc.INT64):
+        for n in (2, 3, 8):
+            for length in (10, 4 * n + 3, 1000):
+                ins = [rand_array(dtype, length, rng) for _ in range(n)]
+                for op in (orc.SUM, orc.MAX, orc.MIN):
+                    root = n - 1
+                    got = orc.shm_reduce(ins, dtype, op, root)[root]
+                    fold = orc.fold_all_reduce(ins, dtype, op, orc.ORDER_SHM)[0]
+                    assert np.array_equal(got.view(np.uint8), fold.view(np.uint8))
+                    # independent statement: numpy left fold in the order expected_orders() writes out
+                    sizes, offs = orc.chunk_partition(length, 2 * n)
+                    want = np.empty_like(ins[0])
+                    for w in range(2 * n):
+                        sl = slice(offs[w], offs[w] + sizes[w])
+                        order = expected_orders(n)["shm"][w]
+                        acc = ins[order[0]][sl].copy()
+                        for r in order[1:]:
+                            with np.errstate(over="ignore"):
+                                acc = {orc.SUM: lambda a, b: a + b, orc.MAX: np.maximum, orc.MIN: np.minimum}[op](acc, ins[r][sl])
+                        want[sl] = acc
+                    if np.issubdtype(ins[0].dtype, np.floating):
+                        ok = np.array_equal(got, want, equal_nan=True)
+                    else:
+                        ok = np.array_equal(got, want)
+                    assert ok, (dtype, n, length, op)
+    # the reference's own vectors: test/test_opr.cpp:482-552 (ReduceSum, 3 ranks, root 1, in = (i+1)(j+1))
+    n, length, root = 3, 10, 1
+    ins = [np.array([(i + 1) * (j + 1) for j in range(length)], dtype=np.float32) for i in range(n)]
+    assert np.array_equal(orc.shm_reduce(ins, orc.FLOAT32, orc.SUM, root)[root], 6.0 * np.arange(1, length + 1, dtype=np.float32))
+    assert np.array_equal(orc.shm_reduce(ins, orc.FLOAT32, orc.MAX, root)[root], ins[2])
+    assert np.array_equal(orc.shm_reduce(ins, orc.FLOAT32, orc.MIN, root)[root], ins[0])
+
+
+def test_shm_broadcast_replay():
+    # test/test_opr.cpp:440-480: 3 ranks, root 1, every rank ends up with the root's (i+1)(j+1)
+    n, length, root = 3, 10, 1
+    ins = [np.array([(i + 1) * (j + 1) for j in range(length)], dtype=np.float32) for i in range(n)]
+    outs = orc.shm_broadcast([ins[r] if r == root else None for r in range(n)], orc.FLOAT32, root)
+    for r in range(n):
+        assert np.array_equal(outs[r], ins[root])
+    rng = np.random.default_rng(5)
+    for dtype in (orc.UINT8, orc.FLOAT16, orc.INT64):
+        ins = [rand_array(dtype, 333, rng) for _ in range(5)]
+        for root in range(5):
+            a = orc.shm_broadcast(ins, dtype, root)
+            b = orc.ucx_broadcast(ins, dtype, root)
+            for r in range(5):
+                assert np.array_equal(a[r].view(np.uint8), ins[root].view(np.uint8))
+                assert np.array_equal(a[r].view(np.uint8), b[r].view(np.uint8))

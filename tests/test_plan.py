@@ -23,8 +23,8 @@ def rand_array(dtype, n, rng):
     return (rng.standard_normal(n) * np.exp(rng.uniform(-20, 20, n))).astype(npdt)
 
 
-def fake_ptrs(base, n, offsets):
-    return [base + r * STRIDE + offsets[r] for r in range(n)]
+def fake_ptrs(base, n, offsets, stride=None):
+    return [base + r * (stride or STRIDE) + offsets[r] for r in range(n)]
 
 
 def combine(acc, x, op, new_wins):
@@ -321,3 +321,41 @@ def test_group_form_tile_mapping_covers_every_tile_once():
     sp, rp = fake_ptrs(SEND_BASE, 8, [0] * 8), fake_ptrs(RECV_BASE, 8, [0] * 8)
     runs, _, _ = mr.describe(mr.Collective.ALL_REDUCE, sp, rp, 1 << 28, orc.FLOAT32)
     assert sum(r["tiles"] for r in runs) == 1 << 20 and all(r["waves"] == 4 for r in runs)
+
+
+def test_blocks_too_long_for_one_grid_are_cut_into_several_pack_launches():
+    """A grid holds 2^31 - 1 workgroups.  16 ranks' all_to_all is 256 block copies; with byte-misaligned buffers
+    (64 bytes per workgroup) a block beyond 512 MiB no longer fits one launch and is cut into slices, one launch
+    each, that cover every block exactly once.  Pointers are synthetic: describe() never dereferences them."""
+    nranks = 16
+    block = 600 * 2 ** 20 + 3  # bytes; odd, and the buffers sit at odd addresses: width 1
+    sp = fake_ptrs(1 << 44, nranks, [1] * nranks, stride=1 << 40)
+    rp = fake_ptrs(1 << 46, nranks, [1] * nranks, stride=1 << 40)
+    runs, bytes_read, bytes_written = mr.describe(mr.Collective.ALL_TO_ALL, sp, rp, block, mr.DType.UINT8)
+    assert bytes_read == bytes_written == nranks * nranks * block
+    steps = sorted({r["step"] for r in runs})
+    assert len(steps) >= 2, "one launch cannot hold 256 x 600 MiB / 64 B workgroups"
+    for step in steps:
+        launch = [r for r in runs if r["step"] == step]
+        assert len(launch) == nranks * nranks
+        assert sum(r["tiles"] for r in launch) <= 2 ** 31 - 1
+        assert all(r["vector"] == 1 for r in launch)
+    # per copy (source rank, source block): the slices tile [0, block) in order
+    for src in range(nranks):
+        for dst in range(nranks):
+            mine = sorted((r for r in runs if r["start"] == src and r["out_first"] == dst), key=lambda r: r["in_begin"])
+            pos = 0
+            for r in mine:
+                assert r["in_begin"] == dst * block + pos and r["out_begin"] == src * block + pos
+                pos += r["count"]
+            assert pos == block
+    # the group form (16-byte accesses) is cut on whole groups of workgroups
+    sp = fake_ptrs(1 << 44, nranks, [0] * nranks, stride=1 << 40)
+    rp = fake_ptrs(1 << 46, nranks, [0] * nranks, stride=1 << 40)
+    block = 40 * 2 ** 30  # 40 GiB blocks: 256 copies x 2.6 M workgroups
+    runs, _, _ = mr.describe(mr.Collective.ALL_TO_ALL, sp, rp, block, mr.DType.UINT8)
+    steps = sorted({r["step"] for r in runs})
+    assert len(steps) >= 2 and all(r["waves"] == 4 and r["vector"] == 16 for r in runs)
+    first = sorted((r for r in runs if r["start"] == 0 and r["out_first"] == 0), key=lambda r: r["in_begin"])
+    assert sum(r["count"] for r in first) == block
+    assert all(r["in_begin"] % (128 * 1024) == 0 for r in first)
