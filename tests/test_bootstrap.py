@@ -135,3 +135,27 @@ def test_group_rendezvous_without_gpu():
         c.close()
     with pytest.raises(mr.MegRayError):
         mr.Communicator(17, 0)  # more ranks than the backend takes
+
+
+def test_a_rank_that_rejects_its_arguments_releases_the_others_without_gpu():
+    """A rank whose own arguments fail validation throws on its own thread, as in the reference
+    (src/ucx/kernel.cu:95-96), and tells the group: the other ranks' calls come back with
+    MEGRAY_INVALID_USAGE and the reason instead of waiting for it.  No device call is made on this path (the
+    rank that arrives last and finds everyone else there enqueues nothing on its stream before it looks at
+    the group), so the rendezvous logic runs without a GPU."""
+    nranks, port = 2, mr.get_free_port()
+    mr.create_server(nranks, port)
+    comms = [mr.get_communicator(nranks, r) for r in range(nranks)]
+    run_ranks(nranks, lambda rank: comms[rank].init("localhost", port))
+    fake = 0x10000000  # never dereferenced: nothing is launched
+    with pytest.raises(mr.MegRayError, match="unknown dtype"):
+        comms[0].all_reduce(fake, fake, 16, mr.DType.CHAR, mr.ReduceOp.SUM)
+    # a second rejected call on the same rank does not wait for the first one's collective to end
+    with pytest.raises(mr.MegRayError, match="unknown reduce op"):
+        comms[0].all_reduce(fake, fake, 16, mr.DType.FLOAT32, 9)
+    with pytest.raises(mr.MegRayError) as info:
+        comms[1].all_reduce(fake + 4096, fake + 4096, 16, mr.DType.FLOAT32, mr.ReduceOp.SUM)
+    assert info.value.status == mr.Status.INVALID_USAGE
+    assert "rank 0 left the collective" in info.value.message and "unknown dtype" in info.value.message
+    for c in comms:
+        c.close()

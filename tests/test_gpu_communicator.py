@@ -307,3 +307,53 @@ def test_contract_violations_throw_on_the_calling_rank():
     fresh = mr.get_communicator(2, 0)
     with pytest.raises(mr.MegRayError):
         fresh.all_reduce(buf, buf, 16, mr.DType.FLOAT32, mr.ReduceOp.SUM)  # before init()
+
+
+def test_parked_ranks_are_released_when_another_rank_rejects_its_arguments():
+    """Two ranks are already waiting in all_reduce, each on a stream of its own, when the third calls with a
+    dtype no reduce exists for: the third throws as the reference does (src/ucx/kernel.cu:95-96), the two get
+    MEGRAY_INVALID_USAGE with the same text, and the group goes on to the next collective as if nothing had been."""
+    import time
+    nranks, n = 3, 1000
+    port = mr.get_free_port()
+    mr.create_server(nranks, port)
+    comms = [mr.get_communicator(nranks, r, mr.Backend.VRANK) for r in range(nranks)]
+    data = [np.arange(n, dtype=np.float32) * (r + 1) for r in range(nranks)]
+    results, messages = [None] * nranks, [None] * nranks
+    errors = []
+
+    def rank_main(rank):
+        try:
+            torch.cuda.set_device(0)
+            comm = comms[rank]
+            comm.init("localhost", port)
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                src, dst = to_device(data[rank]), empty_device(n * 4)
+                if rank == 2:
+                    time.sleep(0.3)  # the others are parked by now
+                try:
+                    comm.all_reduce(src, dst, n, mr.DType.CHAR if rank == 2 else mr.DType.FLOAT32, mr.ReduceOp.SUM, stream)
+                except mr.MegRayError as exc:
+                    messages[rank] = (exc.status, exc.message)
+                comm.all_reduce(src, dst, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream)  # the group still works
+                stream.synchronize()
+                results[rank] = to_host(dst, np.float32)
+        except BaseException as exc:  # noqa: BLE001
+            errors.append((rank, repr(exc)))
+
+    threads = [threading.Thread(target=rank_main, args=(r,), daemon=True) for r in range(nranks)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(120)
+        assert not t.is_alive(), "a rank hung"
+    assert not errors, errors
+    assert messages[2][0] == mr.Status.INVALID_ARGUMENT and "unknown dtype" in messages[2][1]
+    assert messages[0] == messages[1]
+    assert messages[0][0] == mr.Status.INVALID_USAGE and "rank 2 left the collective: unknown dtype" in messages[0][1]
+    want = orc.ucx_all_reduce(data, orc.FLOAT32, orc.SUM)
+    for r in range(nranks):
+        assert bits_equal(results[r], want[r])
+    for c in comms:
+        c.close()
