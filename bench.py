@@ -221,11 +221,12 @@ def copy_yardstick(torch, mr):
 
 def cpu_baseline(orc, np, nranks):
     """The reference tests' expected-value loop on the host: single thread (as the reference runs
-    it) on a 2^25-element-per-rank sample of the headline workload, plus the same loop split over
-    all host cores for scale."""
+    it) on a 2^26-element-per-rank sample of the headline workload (the first quarter of every rank's
+    buffer), plus the same loop split over all host cores for scale, plus the reference's own ring
+    schedule replayed on the host.  About ten seconds of CPU work."""
     from megray_amd import synth
-    n = 1 << 25
-    ins = [synth.fill_np(np.float32, n, r) for r in range(nranks)]  # the first 2^25 elements of the GPU's buffers
+    n = 1 << 26
+    ins = [synth.fill_np(np.float32, n, r) for r in range(nranks)]  # the first 2^26 elements of the GPU's buffers
     bmin = 2 * nranks * n * 4
 
     def timed(threads, reps):
@@ -238,12 +239,12 @@ def cpu_baseline(orc, np, nranks):
         times.sort()
         return times[len(times) // 2]
 
-    t1 = timed(0, 5)
+    t1 = timed(0, 7)
     cores = min(os.cpu_count() or 1, 16)
-    tn = timed(cores, 5)
+    tn = timed(cores, 7)
     # the reference's own schedule on the host: 2(N-1) ring steps of the two-input reduce loop
-    # (src/ucx/all_reduce.cpp:53-101 over src/ucx/kernel.cu:16-22), single thread, 2^24 elements per rank
-    m = 1 << 24
+    # (src/ucx/all_reduce.cpp:53-101 over src/ucx/kernel.cu:16-22), single thread, 2^25 elements per rank
+    m = 1 << 25
     part = [a[:m] for a in ins]
     orc.ucx_all_reduce(part, orc.FLOAT32, orc.SUM)
     t0 = time.perf_counter()
@@ -251,11 +252,11 @@ def cpu_baseline(orc, np, nranks):
     tr = time.perf_counter() - t0
     return {
         "value": round(bmin / t1 / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-        "sample": f"all_reduce SUM fp32, {nranks} ranks x 2^25 elements, test/test_opr.cpp:321-330 loop, "
-                  f"median of 5, {t1 * 1e3:.1f} ms per pass",
+        "sample": f"all_reduce SUM fp32, {nranks} ranks x 2^26 elements, test/test_opr.cpp:321-330 loop, "
+                  f"median of 7, {t1 * 1e3:.1f} ms per pass",
         "all_cores": {"value": round(bmin / tn / 1e9, 3), "cores": cores, "ms": round(tn * 1e3, 1)},
         "ring_replay": {"value": round(2 * nranks * m * 4 / tr / 1e9, 3), "cores": 1, "ms": round(tr * 1e3, 1),
-                        "sample": f"literal 2(N-1)-step ring replay, {nranks} ranks x 2^24 elements, B_min / t"},
+                        "sample": f"literal 2(N-1)-step ring replay, {nranks} ranks x 2^25 elements, B_min / t"},
     }
 
 

@@ -268,6 +268,14 @@ MRV_API int mrv_comm_broadcast(mrv_comm* comm, const void* sendbuff, void* recvb
                                uint32_t root, void* stream);
 MRV_API int mrv_comm_reduce(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t len, int dtype, int op,
                             uint32_t root, void* stream);
+/*
+ * Diagnostic, no counterpart in the reference.  The kernels that make one stream wait for another
+ * (thread-per-rank API with a stream per rank) give up after a time limit instead of spinning for
+ * ever.  This launches one such wait on `stream` for a count that nothing ever raises, with a limit
+ * of `limit_us` microseconds, waits for the stream, and returns how many waits gave up (1) in
+ * *gave_up: a way to see, from the host and without hanging anything, that the limit works.
+ */
+MRV_API int mrv_probe_bounded_wait(uint64_t limit_us, void* stream, uint64_t* gave_up);
 MRV_API int mrv_comm_group_start(mrv_comm* comm);
 MRV_API int mrv_comm_group_end(mrv_comm* comm);
 

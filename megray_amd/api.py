@@ -192,6 +192,14 @@ def reduce_to_root(sendbuffs, recvbuff_root, length, dtype, op, root, order=Fold
                                           int(dtype), int(op), int(order), root, _stream(stream)))
 
 
+def probe_bounded_wait(limit_us, stream=None):
+    """Launch one cross-stream wait that nothing will ever satisfy, with a time limit of `limit_us`; returns how
+    many waits gave up (1).  mrv_probe_bounded_wait."""
+    gave_up = ctypes.c_uint64(0)
+    _check(_lib.load().mrv_probe_bounded_wait(int(limit_us), _stream(stream), ctypes.byref(gave_up)))
+    return gave_up.value
+
+
 def chunk_partition(length, nchunks):
     sizes = (ctypes.c_size_t * nchunks)()
     offs = (ctypes.c_size_t * nchunks)()

@@ -12,6 +12,7 @@
 
 #include "megray.h"
 #include "vrank_communicator.h"
+#include "vrank_edges.h"
 #include "megray/hip_context.h"
 #include "vrank_engine.h"
 #include "vrank_kernels.h"
@@ -453,6 +454,31 @@ int mrv_reduce_to_root(const void* const* sendbuffs, void* recvbuff_root, uint32
         need(sendbuffs, "sendbuffs is null");
         return reduce_to_root(sendbuffs, recvbuff_root, nranks, len, static_cast<DType>(dtype),
                               static_cast<ReduceOp>(op), as_order(order), root, as_stream(stream));
+    });
+}
+
+int mrv_probe_bounded_wait(uint64_t limit_us, void* stream, uint64_t* gave_up) {
+    return guarded([&] {
+        need(gave_up, "gave_up is null");
+        *gave_up = 0;
+        int device = 0, khz = 0;
+        HIP_CHECK(hipGetDevice(&device));
+        HIP_CHECK(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, device));
+        EdgeWords* words = nullptr;
+        HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&words), sizeof(EdgeWords)));
+        Status st = MEGRAY_OK;
+        EdgeWords host{};
+        // nothing ever counts itself in: the wait can only end by giving up
+        if (hipMemset(words, 0, sizeof(EdgeWords)) != hipSuccess ||
+            edge_wait_arrived(words, 1, limit_us * uint64_t(khz) / 1000, nullptr, as_stream(stream)) != hipSuccess ||
+            hipStreamSynchronize(as_stream(stream)) != hipSuccess ||
+            hipMemcpy(&host, words, sizeof(host), hipMemcpyDeviceToHost) != hipSuccess) {
+            (void)hipGetLastError();
+            st = MEGRAY_HIP_ERR;
+        }
+        (void)hipFree(words);
+        *gave_up = host.timeouts;
+        return st;
     });
 }
 

@@ -357,3 +357,19 @@ def test_parked_ranks_are_released_when_another_rank_rejects_its_arguments():
         assert bits_equal(results[r], want[r])
     for c in comms:
         c.close()
+
+
+def test_a_stream_wait_that_nothing_satisfies_gives_up_at_its_limit():
+    """The kernels that make one stream wait for another poll a counter and give up after a time limit, so that a
+    lost mark cannot hold a wavefront (and the stream behind it) for ever.  Forced from the host: a wait for a count
+    nothing raises, with limits of 200 us and 20 ms; the kernel ends by itself, reports one wait given up, and
+    takes about as long as its limit."""
+    import time
+    stream = torch.cuda.Stream()
+    for limit_us in (200, 20000):
+        t0 = time.perf_counter()
+        gave_up = mr.probe_bounded_wait(limit_us, stream)
+        elapsed_us = (time.perf_counter() - t0) * 1e6
+        assert gave_up == 1
+        assert elapsed_us >= limit_us * 0.9, (limit_us, elapsed_us)
+        assert elapsed_us < limit_us + 500000, (limit_us, elapsed_us)
