@@ -373,3 +373,38 @@ def test_a_stream_wait_that_nothing_satisfies_gives_up_at_its_limit():
         assert gave_up == 1
         assert elapsed_us >= limit_us * 0.9, (limit_us, elapsed_us)
         assert elapsed_us < limit_us + 500000, (limit_us, elapsed_us)
+
+
+@pytest.mark.parametrize("length", [3000, 100000, (1 << 18) + 11])
+def test_back_to_back_rounds_with_fresh_data_on_rank_streams(length):
+    """Five all_reduces back to back, every round with different inputs that each rank copies into the SAME device
+    buffer on its own stream right before the call, and with the result copied out of the SAME device buffer on
+    that stream right after, no host synchronisation in between.  A collective that started before some rank's
+    copy-in had landed, or a copy-in that overtook the previous collective's reads, or a copy-out that overtook
+    the collective's writes, shows as a wrong round.  The three lengths run the short kernel that carries the
+    stream ordering itself (12 and 391 tiles) and the group kernel with separate wait / notify kernels (1025 tiles)."""
+    nranks, rounds = 8, 5
+    rng = np.random.default_rng(length)
+    data = [[rand_array(orc.FLOAT32, length, rng) for _ in range(nranks)] for _ in range(rounds)]
+    wants = [orc.ucx_all_reduce(ins, orc.FLOAT32, orc.SUM) for ins in data]
+    outs = [[None] * nranks for _ in range(rounds)]
+
+    def main(comm, rank, _inp, stream):
+        with torch.cuda.stream(stream):
+            staged = [torch.from_numpy(data[r][rank].view(np.uint8).copy()).pin_memory() for r in range(rounds)]
+            host_out = [torch.empty(length * 4, dtype=torch.uint8).pin_memory() for _ in range(rounds)]
+            src = torch.empty(length * 4, dtype=torch.uint8, device="cuda:0")
+            dst = torch.full((length * 4,), 0x5A, dtype=torch.uint8, device="cuda:0")
+            for r in range(rounds):
+                src.copy_(staged[r], non_blocking=True)
+                comm.all_reduce(src, dst, length, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream)
+                host_out[r].copy_(dst, non_blocking=True)
+            stream.synchronize()
+            for r in range(rounds):
+                outs[r][rank] = host_out[r].numpy().view(np.float32).copy()
+        return None
+
+    run_test(nranks, [None] * nranks, [None] * nranks, main)
+    for r in range(rounds):
+        for rank in range(nranks):
+            assert bits_equal(outs[r][rank], wants[r][rank]), f"round {r} rank {rank}"
