@@ -106,6 +106,8 @@ public:
               m_mail(size_t(nranks) * nranks) {}
 
     ~Group() {
+        // wait kernels of the last collectives may still be polling the counters
+        if (m_edges[0].words || m_edges[1].words) (void)hipDeviceSynchronize();
         for (hipEvent_t ev : m_events) (void)hipEventDestroy(ev);
         for (hipEvent_t ev : m_arrive)
             if (ev) (void)hipEventDestroy(ev);
