@@ -473,12 +473,12 @@ private:
         const uint64_t ticket = m_generation.load(std::memory_order_relaxed) + 1;
         // A short flat launch waits for the marks and publishes its completion itself: two launches
         // less on this thread, on which every rank is waiting.
-        // (Only the short form: a launch of many tiles must not wait inside the kernel - workgroups that
-        // hold a whole CU's LDS would spin on streams that may need that CU - and announcing completion
-        // costs an L2 write-back per workgroup.  Those get a wait kernel before and a notify kernel after.)
+        // (Only short launches: one of many tiles must not wait inside the kernel - workgroups that hold a
+        // whole CU's LDS would spin on streams that may need that CU - and announcing completion costs
+        // an L2 write-back per workgroup.  Those get a wait kernel before and a notify kernel after.)
         FlatLaunch* hooked = nullptr;
         if (set.words && !one_stream && cp->plan.steps.size() == 1 && cp->plan.steps[0].kind == Step::kFlat &&
-            cp->plan.steps[0].flat.waves == 1)
+            cp->plan.steps[0].flat.waves == 1 && cp->plan.steps[0].flat.total_tiles < kHookMaxTiles)
             hooked = &cp->plan.steps[0].flat;
         if (hooked) {
             hooked->hooks = EdgeHooks{reinterpret_cast<uint64_t*>(set.words), set.status, m_limit_ticks};

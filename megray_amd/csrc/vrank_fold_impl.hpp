@@ -10,7 +10,7 @@
 //
 //   flat launches     K == rank count in {2, 3, 4, 8}, buffers 16-byte aligned: tile t is the same
 //                     KiB of every buffer, so loads need nothing but the block index.
-//                     fold_group_kernel (512 tiles and more) / fold_flat_kernel (fewer).
+//                     fold_group_kernel (2048 tiles and more) / fold_flat_kernel (fewer).
 //   segment launches  any K, buffers that share an offset from a 16-byte boundary or none at all,
 //                     shifted copies: head / vector body / tail segments cut by the planner.
 //                     fold_segment_group_kernel (long vector bodies) / fold_kernel.

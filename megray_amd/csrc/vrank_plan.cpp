@@ -147,7 +147,7 @@ private:
         // the inputs' offsets) also exchange the results between the wavefronts of a group
         bool unshifted = true;
         for (const Run& r : m_runs) unshifted = unshifted && r.in_begin == r.out_begin;
-        L.waves = total >= kGroupMinTiles ? kGroupWaves : 1;
+        L.waves = total >= kFlatGroupMinTiles ? kGroupWaves : 1;
         L.exchange = (L.waves == kGroupWaves && !m_tree && m_nout == m_nranks && unshifted) ? 1 : 0;
         L.unshifted = unshifted ? 1 : 0;
         m_plan.steps.push_back(step);

@@ -100,12 +100,19 @@ struct FlatLaunch {
     EdgeHooks hooks;               // one wavefront per tile only
 };
 
-// Group form of the flat fold: a workgroup of kGroupWaves wavefronts owns kGroupWaves tiles that lie
-// kGroupStride tiles apart; launches of fewer than kGroupMinTiles tiles keep one wavefront per tile
-// (measured: the group form is as fast or faster from 512 tiles per buffer upwards).
+// Group form: a workgroup of kGroupWaves wavefronts owns kGroupWaves tiles that lie kGroupStride tiles
+// apart.  Short launches keep one wavefront per tile.  Measured crossovers on MI355X: the flat fold
+// from 2048 tiles per buffer (8 ranks, all_reduce fp32: 1 MiB per rank 3.95 us against 4.54 in the
+// group form, 2 MiB 5.3 against 5.75, 3.5 MiB 7.3 against 7.5, 4 MiB 11.1 against 8.5; reduce_scatter
+// and 2 or 4 ranks cross between 2 and 4 MiB as well), the segment and pack kernels from 512.
 constexpr uint32_t kGroupWaves = 4;
 constexpr uint32_t kGroupStride = 32;
 constexpr uint32_t kGroupMinTiles = 512;
+constexpr uint32_t kFlatGroupMinTiles = 2048;
+// Launches of the flat fold below this many tiles can carry the thread-per-rank API's stream
+// ordering themselves (EdgeHooks).  Beyond it the release fence every workgroup then executes costs
+// more than the two launches it saves (1024 tiles: 42 us per all_reduce against 24).
+constexpr uint32_t kHookMaxTiles = 512;
 constexpr uint32_t group_grid(uint32_t total_tiles) {
     return (total_tiles + kGroupWaves * kGroupStride - 1) / (kGroupWaves * kGroupStride) * kGroupStride;
 }

@@ -55,7 +55,7 @@ def test_all_reduce_fused_all_orders(dtype, nranks):
 
 @pytest.mark.parametrize("dtype", REDUCE_TYPES)
 def test_all_reduce_group_form(dtype):
-    """Launches of 512 tiles and more take the group form of the flat kernel (four wavefronts per
+    """Launches of 2048 tiles and more take the group form of the flat kernel (four wavefronts per
     workgroup, four tiles 32 tiles apart): ragged lengths, so that chunk borders fall inside tiles and the
     last group of tiles is incomplete; out of place and in place."""
     size = orc.dtype_size(dtype)
@@ -245,8 +245,8 @@ def test_float_special_values_and_tie_conventions():
         with np.errstate(over="ignore", under="ignore"):
             vals = base.astype(npdt)
         ins = [rng.choice(vals, size=4096 + 5).astype(npdt) for _ in range(n)]
-        # the same through the group kernels: 600 tiles per buffer
-        long_ins = [rng.choice(vals, size=600 * 1024 // orc.dtype_size(dtype) + 5).astype(npdt) for _ in range(n)]
+        # the same through the group kernels: 2600 tiles per buffer
+        long_ins = [rng.choice(vals, size=2600 * 1024 // orc.dtype_size(dtype) + 5).astype(npdt) for _ in range(n)]
         for op in OPS:
             for order in ORDERS:
                 for data in (ins, long_ins):
@@ -484,7 +484,7 @@ def test_planned_collectives_and_graph_replay():
     nranks = 8
     # the second length runs the group kernels (workgroups of 256 threads) also as graph nodes
     for sched, length in ((mr.Schedule.FUSED, 40000 + 3), (mr.Schedule.TWO_PHASE, 40000 + 3),
-                          (mr.Schedule.RING, 40000 + 3), (mr.Schedule.FUSED, 700 * 256 + 5),
+                          (mr.Schedule.RING, 40000 + 3), (mr.Schedule.FUSED, 2700 * 256 + 5),
                           (mr.Schedule.TWO_PHASE, 5000 * 256 + 5)):
         ins = [rand_array(orc.FLOAT32, length, rng) for _ in range(nranks)]
         want = orc.ucx_all_reduce(ins, orc.FLOAT32, orc.SUM)
