@@ -833,8 +833,9 @@ __device__ __forceinline__ void hook_wait(const EdgeHooks& h, uint64_t target) {
 }
 
 // After a one-wavefront workgroup's stores: count it, and let the last one publish the ticket.
-// (Only short launches do this: the release fence writes the L2 back, once per workgroup, and at
-// 2560 workgroups that alone took ten times as long as the fold.)
+// (Only short launches do this: the release fence writes the L2 back, once per workgroup; from a few
+// hundred workgroups on that costs more than a separate notify kernel, and at 2560 workgroups it
+// alone took ten times as long as the fold.)
 __device__ __forceinline__ void hook_publish(const EdgeHooks& h, uint64_t ticket) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // this wavefront's stores before its count
     if (threadIdx.x == 0) {

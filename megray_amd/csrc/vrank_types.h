@@ -109,10 +109,12 @@ constexpr uint32_t kGroupWaves = 4;
 constexpr uint32_t kGroupStride = 32;
 constexpr uint32_t kGroupMinTiles = 512;
 constexpr uint32_t kFlatGroupMinTiles = 2048;
-// Launches of the flat fold below this many tiles can carry the thread-per-rank API's stream
-// ordering themselves (EdgeHooks).  Beyond it the release fence every workgroup then executes costs
-// more than the two launches it saves (1024 tiles: 42 us per all_reduce against 24).
-constexpr uint32_t kHookMaxTiles = 512;
+// Launches of the flat fold below this many tiles carry the thread-per-rank API's stream ordering
+// themselves (EdgeHooks).  Beyond it the release fence every workgroup then executes costs more than
+// the two launches it saves.  Measured, 8 ranks, a stream per rank, microseconds per all_reduce with /
+// without: 16 - 128 tiles 16 - 18 / 22 - 23, 256 tiles 18 / 22.5, 384 tiles 21 - 34 / 22 - 23, 508 tiles
+// 30 / 22, 1024 tiles 42 / 24.
+constexpr uint32_t kHookMaxTiles = 288;
 constexpr uint32_t group_grid(uint32_t total_tiles) {
     return (total_tiles + kGroupWaves * kGroupStride - 1) / (kGroupWaves * kGroupStride) * kGroupStride;
 }

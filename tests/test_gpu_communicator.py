@@ -375,14 +375,15 @@ def test_a_stream_wait_that_nothing_satisfies_gives_up_at_its_limit():
         assert elapsed_us < limit_us + 500000, (limit_us, elapsed_us)
 
 
-@pytest.mark.parametrize("length", [3000, 100000, (1 << 18) + 11])
+@pytest.mark.parametrize("length", [3000, 70000, 100000, (1 << 19) + 11])
 def test_back_to_back_rounds_with_fresh_data_on_rank_streams(length):
     """Five all_reduces back to back, every round with different inputs that each rank copies into the SAME device
     buffer on its own stream right before the call, and with the result copied out of the SAME device buffer on
     that stream right after, no host synchronisation in between.  A collective that started before some rank's
     copy-in had landed, or a copy-in that overtook the previous collective's reads, or a copy-out that overtook
-    the collective's writes, shows as a wrong round.  The three lengths run the short kernel that carries the
-    stream ordering itself (12 and 391 tiles) and the group kernel with separate wait / notify kernels (1025 tiles)."""
+    the collective's writes, shows as a wrong round.  The lengths run the short kernel that carries the stream
+    ordering itself (12 and 274 tiles), the short kernel between separate wait / notify kernels (391 tiles) and the
+    group kernel between them (2049 tiles)."""
     nranks, rounds = 8, 5
     rng = np.random.default_rng(length)
     data = [[rand_array(orc.FLOAT32, length, rng) for _ in range(nranks)] for _ in range(rounds)]
