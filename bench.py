@@ -15,9 +15,11 @@ with all buffers already resident in HBM.  Prints ONE JSON line:
   small_msg_us  the same sizes through the flat C ABI (one caller, one stream)
   other_configs the other benchmark configurations (reduce_scatter / all_gather fp16, MAX int32,
              MIN int64, all_to_all uint8, SUM int8), each timed with HIP events
+  other_layout  the headline launches again on buffers placed the other way (--layout: where the ranks'
+             buffers lie in HBM relative to each other decides 6 - 10 points of the peak)
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--log2n 28] [--no-cpu] [--no-small] [--no-comm]
-                       [--no-others]
+                       [--no-others] [--layout placed|separate]
 """
 import argparse
 import hashlib
@@ -82,11 +84,40 @@ def parse_args():
     ap.add_argument("--no-check", action="store_true", help="skip the correctness checks")
     ap.add_argument("--no-comm", action="store_true", help="skip the thread-per-rank Communicator API leg")
     ap.add_argument("--no-others", action="store_true", help="skip the other benchmark configurations")
+    ap.add_argument("--layout", choices=("placed", "separate"), default="placed",
+                    help="where the ranks' buffers lie in HBM: placed = one allocation laid out by the library "
+                         "(mrv_rank_buffers_layout), separate = one torch allocation per buffer")
     return ap.parse_args()
 
 
+LAYOUT_TEXT = {
+    "placed": "one allocation, buffers an odd multiple of 128 MiB apart (mrv_rank_buffers_layout)",
+    "separate": "one torch allocation per buffer",
+}
+
+
+def alloc_buffers(torch, mr, specs, layout):
+    """Tensors for (numel, dtype) pairs in HBM.  "placed": views into one allocation at the distances the
+    library recommends for buffers that a collective walks through in step; "separate": one torch allocation
+    each, wherever the caching allocator puts them."""
+    if layout == "placed":
+        return mr.place_tensors(torch, specs, "cuda:0")
+    return [torch.empty(numel, dtype=dtype, device="cuda:0") for numel, dtype in specs]
+
+
+def make_buffers(torch, mr, nranks, n, layout):
+    """Inputs and outputs of the headline workload.  Inputs: uniform[-1, 1) fp32 from the counter-based generator,
+    element i of rank r depends only on (seed, r, i)."""
+    from megray_amd import synth
+    bufs = alloc_buffers(torch, mr, [(n, torch.float32)] * (2 * nranks), layout)
+    ins, outs = bufs[:nranks], bufs[nranks:]
+    for r, t in enumerate(ins):
+        synth.fill_torch(torch.float32, n, r, out=t)
+    return ins, outs
+
+
 def make_inputs(torch, nranks, n):
-    """uniform[-1, 1) fp32 from the counter-based generator: element i of rank r depends only on (seed, r, i)."""
+    """The same inputs as separate tensors (small sizes)."""
     from megray_amd import synth
     return [synth.fill_torch(torch.float32, n, r) for r in range(nranks)]
 
@@ -198,8 +229,8 @@ def copy_yardstick(torch, mr):
     through this library's copy kernel and through torch (GB/s, read + write)."""
     from megray_amd import synth
     n = 1 << 30
-    src = synth.fill_torch(torch.uint8, n, 0)  # random bytes: the rate depends on the data (zeros copy faster)
-    dst = torch.empty_like(src)
+    src, dst = alloc_buffers(torch, mr, [(n, torch.uint8)] * 2, "placed")
+    synth.fill_torch(torch.uint8, n, 0, out=src)  # random bytes: the rate depends on the data (zeros copy faster)
     st = torch.cuda.current_stream()
 
     def timed(fn):
@@ -260,34 +291,36 @@ def cpu_baseline(orc, np, nranks):
     }
 
 
-def time_workload(w, torch, mr, steps, warmup):
+def time_workload(w, torch, mr, steps, warmup, layout="placed"):
     """One of the non-headline workloads: builds its inputs in HBM, times `steps` collectives with HIP
     events on the launch stream and returns the figures."""
     dev = "cuda:0"
     st = torch.cuda.current_stream()
     n8 = 8
 
-    def rnd(n, dtype, rank):
+    def buffers(n_in, n_out, dtype, count_in=n8, count_out=n8):
+        """count_in inputs of n_in elements (filled) and count_out outputs of n_out elements."""
         from megray_amd import synth
-        return synth.fill_torch(dtype, n, rank, "normal" if dtype.is_floating_point else "uniform", device=dev)
+        bufs = alloc_buffers(torch, mr, [(n_in, dtype)] * count_in + [(n_out, dtype)] * count_out, layout)
+        for rank, t in enumerate(bufs[:count_in]):
+            synth.fill_torch(dtype, n_in, rank, "normal" if dtype.is_floating_point else "uniform", device=dev, out=t)
+        return bufs[:count_in], bufs[count_in:]
 
     if w == "copy":
         n = 1 << 30
-        src, dst = [rnd(n, torch.uint8, 0)], [torch.empty(n, dtype=torch.uint8, device=dev)]
+        src, dst = buffers(n, n, torch.uint8, 1, 1)
         step = lambda: mr.broadcast(src[0], dst, n, mr.DType.UINT8, 0, stream=st)  # noqa: E731
         desc = (mr.Collective.BROADCAST, src, dst, n, mr.DType.UINT8)
         text, dt = "plain copy of 2^30 bytes (one rank, broadcast to itself)", "u8"
     elif w == "c2_reduce_scatter":
         recvlen = 1 << 23
-        src = [rnd(n8 * recvlen, torch.float16, r) for r in range(n8)]
-        dst = [torch.empty(recvlen, dtype=torch.float16, device=dev) for _ in range(n8)]
+        src, dst = buffers(n8 * recvlen, recvlen, torch.float16)
         step = lambda: mr.reduce_scatter(src, dst, recvlen, mr.DType.FLOAT16, mr.ReduceOp.SUM, stream=st)  # noqa: E731
         desc = (mr.Collective.REDUCE_SCATTER, src, dst, recvlen, mr.DType.FLOAT16)
         text, dt = "reduce_scatter SUM fp16 (fp32 accumulate), 8 ranks x 2^26 elements in, 2^23 out", "f16"
     elif w == "c2_all_gather":
         sendlen = 1 << 23
-        src = [rnd(sendlen, torch.float16, r) for r in range(n8)]
-        dst = [torch.empty(n8 * sendlen, dtype=torch.float16, device=dev) for _ in range(n8)]
+        src, dst = buffers(sendlen, n8 * sendlen, torch.float16)
         step = lambda: mr.all_gather(src, dst, sendlen, mr.DType.FLOAT16, stream=st)  # noqa: E731
         desc = (mr.Collective.ALL_GATHER, src, dst, sendlen, mr.DType.FLOAT16)
         text, dt = "all_gather fp16, 8 ranks x 2^23 elements in, 2^26 out", "f16"
@@ -295,22 +328,19 @@ def time_workload(w, torch, mr, steps, warmup):
         tdt, mdt, op = ((torch.int32, mr.DType.INT32, mr.ReduceOp.MAX) if w == "c3_max_int32"
                         else (torch.int64, mr.DType.INT64, mr.ReduceOp.MIN))
         n = 1 << 28
-        src = [rnd(n, tdt, r) for r in range(n8)]
-        dst = [torch.empty(n, dtype=tdt, device=dev) for _ in range(n8)]
+        src, dst = buffers(n, n, tdt)
         step = lambda: mr.all_reduce(src, dst, n, mdt, op, stream=st)  # noqa: E731
         desc = (mr.Collective.ALL_REDUCE, src, dst, n, mdt)
         text, dt = f"all_reduce {op.name} {mdt.name.lower()}, 8 ranks x 2^28 elements", mdt.name.lower()
     elif w == "c5_all_to_all":
         blk = 1 << 24
-        src = [rnd(n8 * blk, torch.uint8, r) for r in range(n8)]
-        dst = [torch.empty(n8 * blk, dtype=torch.uint8, device=dev) for _ in range(n8)]
+        src, dst = buffers(n8 * blk, n8 * blk, torch.uint8)
         step = lambda: mr.all_to_all(src, dst, blk, mr.DType.UINT8, stream=st)  # noqa: E731
         desc = (mr.Collective.ALL_TO_ALL, src, dst, blk, mr.DType.UINT8)
         text, dt = "all_to_all uint8, 8 ranks x 8 blocks of 16 MiB", "u8"
     elif w == "c5_sum_int8":
         n = 1 << 27
-        src = [rnd(n, torch.int8, r) for r in range(n8)]
-        dst = [torch.empty(n, dtype=torch.int8, device=dev) for _ in range(n8)]
+        src, dst = buffers(n, n, torch.int8)
         step = lambda: mr.all_reduce(src, dst, n, mr.DType.INT8, mr.ReduceOp.SUM, stream=st)  # noqa: E731
         desc = (mr.Collective.ALL_REDUCE, src, dst, n, mr.DType.INT8)
         text, dt = "all_reduce SUM int8 (wrap-around), 8 ranks x 2^27 elements", "i8"
@@ -341,13 +371,13 @@ def time_workload(w, torch, mr, steps, warmup):
 
 def run_other_workload(args, torch, mr):
     """A non-headline workload on its own: same timing, one JSON line, no CPU / small-message legs."""
-    r = time_workload(args.workload, torch, mr, args.steps, args.warmup)
+    r = time_workload(args.workload, torch, mr, args.steps, args.warmup, args.layout)
     value = r["bytes"] / (r["wall_s"] / args.steps) / 1e9
     print(json.dumps({
         "metric": "achieved HBM GB/s (% of peak)", "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(r["wall_s"] * 1e3 / args.steps, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": r["dtype"], "data": "synthetic",
-        "config": {"workload": r["workload"], "launches_per_step": r["launches"]},
+        "config": {"workload": r["workload"], "launches_per_step": r["launches"], "layout": args.layout},
         "pct_of_peak": round(100.0 * value / HBM_PEAK_GBPS, 2), "bytes_executed": r["bytes"],
         "roofline": {"bound": "hbm", "achieved": round(r["achieved"], 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(r["achieved"] / HBM_PEAK_GBPS, 4), "traffic": r["traffic"],
@@ -357,13 +387,13 @@ def run_other_workload(args, torch, mr):
     return 0
 
 
-def other_configs(torch, mr):
+def other_configs(torch, mr, layout):
     """The other benchmark configurations, ten timed steps each: milliseconds per collective (HIP events),
     GB/s on the collective's minimum bytes (which is what each of them executes) and that as a fraction of
     the HBM peak."""
     out = {}
     for w in ("c2_reduce_scatter", "c2_all_gather", "c3_max_int32", "c3_min_int64", "c5_all_to_all", "c5_sum_int8"):
-        r = time_workload(w, torch, mr, 10, 2)
+        r = time_workload(w, torch, mr, 10, 2, layout)
         out[w] = {"workload": r["workload"], "ms": round(r["kernel_ms"] * r["launches"], 4),
                   "gbps": round(r["achieved"], 1), "frac": round(r["achieved"] / HBM_PEAK_GBPS, 4),
                   "bytes_min": r["bytes"], "traffic": r["traffic"]}
@@ -400,26 +430,28 @@ def main():
         import oracle as orc
         check_small(torch, mr, orc, np)
 
-    ins = make_inputs(torch, nranks, n)
-    outs = [torch.empty_like(t) for t in ins]
     st = torch.cuda.current_stream()
 
-    def step():
-        mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, order=mr.FoldOrder.UCX, schedule=sched,
-                      stream=st)
+    def timed(ins, outs, steps, warmup):
+        """-> (wall seconds, HIP-event milliseconds) of `steps` collectives after `warmup` untimed ones."""
+        def step():
+            mr.all_reduce(ins, outs, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, order=mr.FoldOrder.UCX, schedule=sched,
+                          stream=st)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record(st)
-    for _ in range(args.steps):
-        step()
-    e1.record(st)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    event_ms = e0.elapsed_time(e1)
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record(st)
+        for _ in range(steps):
+            step()
+        e1.record(st)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, e0.elapsed_time(e1)
+
+    ins, outs = make_buffers(torch, mr, nranks, n, args.layout)
+    wall, event_ms = timed(ins, outs, args.steps, args.warmup)
 
     if not args.no_check:
         check_full(torch, mr, ins, outs, n)
@@ -450,6 +482,7 @@ def main():
         "config": {
             "workload": f"all_reduce SUM fp32, {nranks} virtual ranks x 2^{args.log2n} elements, ucx ring order, "
                         f"{args.schedule} schedule, buffers resident in HBM",
+            "layout": LAYOUT_TEXT[args.layout],
             "ranks": nranks, "elements_per_rank": n, "order": "ucx", "schedule": args.schedule,
             "launches_per_step": launches,
         },
@@ -465,6 +498,14 @@ def main():
     }
     del ins, outs
     torch.cuda.empty_cache()
+    if not args.no_others:  # the same launches on buffers placed the other way, for the record
+        other = "separate" if args.layout == "placed" else "placed"
+        ins, outs = make_buffers(torch, mr, nranks, n, other)
+        _, other_ms = timed(ins, outs, 5, 2)
+        result["other_layout"] = {"layout": LAYOUT_TEXT[other], "ms_per_step": round(other_ms / 5, 4),
+                                  "pct_of_peak": round(100.0 * bmin / (other_ms / 5 * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2)}
+        del ins, outs
+        torch.cuda.empty_cache()
     props = torch.cuda.get_device_properties(0)
     result["device"] = {"name": props.name, "compute_units": props.multi_processor_count,
                         "hbm_gib": round(props.total_memory / 2 ** 30, 1)}
@@ -474,7 +515,7 @@ def main():
     if comm_api is not None:
         result["comm_api_us"] = comm_api
     if not args.no_others:
-        result["other_configs"] = other_configs(torch, mr)
+        result["other_configs"] = other_configs(torch, mr, args.layout)
     if not args.no_cpu:
         import oracle as orc
         result["cpu_baseline"] = cpu_baseline(orc, np, nranks)

@@ -276,6 +276,28 @@ MRV_API int mrv_comm_reduce(mrv_comm* comm, const void* sendbuff, void* recvbuff
  * *gave_up: a way to see, from the host and without hanging anything, that the limit works.
  */
 MRV_API int mrv_probe_bounded_wait(uint64_t limit_us, void* stream, uint64_t* gave_up);
+
+/*
+ * Placement of the ranks' buffers in HBM.  No counterpart in the reference, whose ranks are devices and allocate
+ * their own buffers (test/performance.cpp:108-110, test/test_base.h:57-66); optional: every entry point of this
+ * library takes buffers from anywhere.
+ *
+ * A collective touches the same offset of up to 2N buffers at the same time, and the memory system derives channel
+ * and bank from address bits: buffers whose starts differ by a multiple of a large power of two (what separate
+ * allocations of a power-of-two size give) are served 6 - 10 points of the HBM peak slower than buffers an odd
+ * multiple of 128 MiB apart (8-rank fp32 all_reduce, 1 GiB per rank: 75 - 78 % against 84 %; 16 MiB per rank: 66 %
+ * against 78 %).  These calls lay `count` buffers of bytes[i] bytes out in ONE allocation accordingly: buffers of
+ * 8 MiB and more start an odd multiple of 128 MiB after the one before, smaller ones (they live in the caches) at
+ * the next 2 MiB or 4 KiB boundary.  Pass the buffers of one collective together, inputs and outputs, in any order.
+ *
+ * mrv_rank_buffers_layout  only computes: offsets[i] from a common base (2 MiB aligned or better) and *total, the
+ *                          bytes to allocate, for callers with an allocator of their own.  Needs no GPU.
+ * mrv_rank_buffers_alloc   allocates (hipMalloc) and returns the addresses in ptrs[0..count) and the allocation in
+ *                          *base; mrv_rank_buffers_free(base) releases it (null is allowed).
+ */
+MRV_API int mrv_rank_buffers_layout(int count, const size_t* bytes, size_t* offsets, size_t* total);
+MRV_API int mrv_rank_buffers_alloc(int count, const size_t* bytes, void** ptrs, void** base);
+MRV_API int mrv_rank_buffers_free(void* base);
 MRV_API int mrv_comm_group_start(mrv_comm* comm);
 MRV_API int mrv_comm_group_end(mrv_comm* comm);
 

@@ -67,6 +67,9 @@ def load():
     L.mrv_reduce_to_root.argtypes = [pp, vp, u32, sz, i32, i32, i32, u32, vp]
     L.mrv_probe_bounded_wait.argtypes = [ctypes.c_uint64, vp, ctypes.POINTER(ctypes.c_uint64)]
     L.mrv_probe_bounded_wait.restype = i32
+    L.mrv_rank_buffers_layout.argtypes = [i32, ctypes.POINTER(sz), ctypes.POINTER(sz), ctypes.POINTER(sz)]
+    L.mrv_rank_buffers_alloc.argtypes = [i32, ctypes.POINTER(sz), ctypes.POINTER(vp), ctypes.POINTER(vp)]
+    L.mrv_rank_buffers_free.argtypes = [vp]
     L.mrv_get_free_port.argtypes = []
     L.mrv_create_server.argtypes = [u32, i32]
     L.mrv_comm_create.argtypes = [u32, u32, i32, ctypes.POINTER(vp)]

@@ -200,6 +200,62 @@ def probe_bounded_wait(limit_us, stream=None):
     return gave_up.value
 
 
+def rank_buffers_layout(sizes):
+    """-> (offsets, total): where buffers of `sizes` bytes go inside one allocation so that a collective over them is
+    served well by the memory system (buffers of 8 MiB and more an odd multiple of 128 MiB apart).
+    mrv_rank_buffers_layout; needs no GPU."""
+    count = len(sizes)
+    arr = (ctypes.c_size_t * max(count, 1))(*[int(b) for b in sizes])
+    offs = (ctypes.c_size_t * max(count, 1))()
+    total = ctypes.c_size_t(0)
+    _check(_lib.load().mrv_rank_buffers_layout(count, arr, offs, ctypes.byref(total)))
+    return list(offs)[:count], total.value
+
+
+class RankBuffers:
+    """Buffers of `sizes` bytes in one device allocation, placed by mrv_rank_buffers_alloc; `.ptrs` are their
+    addresses.  free() (or the end of a with block) releases the allocation."""
+
+    def __init__(self, sizes):
+        count = len(sizes)
+        arr = (ctypes.c_size_t * max(count, 1))(*[int(b) for b in sizes])
+        ptrs = (ctypes.c_void_p * max(count, 1))()
+        base = ctypes.c_void_p(None)
+        _check(_lib.load().mrv_rank_buffers_alloc(count, arr, ptrs, ctypes.byref(base)))
+        self.ptrs = [int(p or 0) for p in ptrs][:count]
+        self.sizes = [int(b) for b in sizes]
+        self._base = base
+
+    def free(self):
+        if self._base is not None and self._base.value:
+            _check(_lib.load().mrv_rank_buffers_free(self._base))
+        self._base = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.free()
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def place_tensors(torch, specs, device="cuda"):
+    """Tensors of the given (numel, dtype) pairs as views into ONE torch allocation, placed by rank_buffers_layout:
+    the way to hand torch-owned memory to a collective in the placement the library recommends.  The views keep the
+    allocation alive."""
+    sizes = [int(numel) * torch.empty((), dtype=dtype).element_size() for numel, dtype in specs]
+    offsets, total = rank_buffers_layout(sizes)
+    align = 2 << 20
+    arena = torch.empty(total + align, dtype=torch.uint8, device=device)
+    skew = (-arena.data_ptr()) % align
+    return [arena[skew + off:skew + off + size].view(dtype) for off, size, (_, dtype) in zip(offsets, sizes, specs)]
+
+
 def chunk_partition(length, nchunks):
     sizes = (ctypes.c_size_t * nchunks)()
     offs = (ctypes.c_size_t * nchunks)()

@@ -23,6 +23,7 @@
 #include <vector>
 
 #include "megray.h"
+#include "megray_vrank.h"
 
 namespace {
 
@@ -43,6 +44,8 @@ struct Arguments {
     hipStream_t shared_stream = nullptr;  // -S: every rank enqueues on this one stream
     bool share = false;
     std::string json_path;  // -J: per-size results as JSON lines, with the spread of the per-call times
+    bool own_allocations = false;  // -M: every rank hipMallocs its own buffers, as the reference's harness does
+    std::vector<void*> placed;     // otherwise: in buffers of ranks 0..N-1, then out buffers, in one allocation
 };
 
 // What rank 0's thread measured for one buffer size.
@@ -83,8 +86,13 @@ void worker(const Func& func, Arguments args, int dev, int port, Timing* res) {
     auto comm = MegRay::get_communicator(args.n_devs, dev, MegRay::MEGRAY_VRANK);
     if (comm->init(args.master_ip.c_str(), port) != MegRay::MEGRAY_OK) std::exit(1);
     void *in_ptr = nullptr, *out_ptr = nullptr;
-    CHECK_HIP(hipMalloc(&in_ptr, args.in_bufsize ? args.in_bufsize : 1));
-    CHECK_HIP(hipMalloc(&out_ptr, args.out_bufsize ? args.out_bufsize : 1));
+    if (args.own_allocations) {
+        CHECK_HIP(hipMalloc(&in_ptr, args.in_bufsize ? args.in_bufsize : 1));
+        CHECK_HIP(hipMalloc(&out_ptr, args.out_bufsize ? args.out_bufsize : 1));
+    } else {
+        in_ptr = args.placed[size_t(dev)];
+        out_ptr = args.placed[size_t(args.n_devs + dev)];
+    }
     CHECK_HIP(hipMemset(in_ptr, 0, args.in_bufsize));
     Kernel kernel = func.make(args, dev);
     for (int i = 0; i < args.warmup_iters; i++) kernel(comm, in_ptr, out_ptr, context);
@@ -99,8 +107,10 @@ void worker(const Func& func, Arguments args, int dev, int port, Timing* res) {
     }
     CHECK_HIP(hipStreamSynchronize(stream));
     const double t1 = now_us();
-    CHECK_HIP(hipFree(in_ptr));
-    CHECK_HIP(hipFree(out_ptr));
+    if (args.own_allocations) {
+        CHECK_HIP(hipFree(in_ptr));
+        CHECK_HIP(hipFree(out_ptr));
+    }
     if (!args.share) CHECK_HIP(hipStreamDestroy(stream));
     if (dev == 0) {
         std::vector<double> gaps;
@@ -112,13 +122,31 @@ void worker(const Func& func, Arguments args, int dev, int port, Timing* res) {
     }
 }
 
-Timing run_test(const Func& func, const Arguments& args) {
+Timing run_test(const Func& func, Arguments args) {
     Timing res;
     int port = MegRay::get_free_port();
     if (MegRay::create_server(args.n_devs, port) != MegRay::MEGRAY_OK) std::exit(1);
+    void* base = nullptr;
+    if (!args.own_allocations) {
+        // all ranks' buffers in one allocation, at the distances the library recommends for buffers that
+        // a collective walks through in step (the ranks share one HBM here)
+        const size_t n = size_t(args.n_devs);
+        std::vector<size_t> sizes(2 * n);
+        for (size_t i = 0; i < n; ++i) {
+            sizes[i] = args.in_bufsize ? args.in_bufsize : 1;
+            sizes[n + i] = args.out_bufsize ? args.out_bufsize : 1;
+        }
+        args.placed.resize(2 * n);
+        CHECK_HIP(hipSetDevice(0));
+        if (mrv_rank_buffers_alloc(int(2 * n), sizes.data(), args.placed.data(), &base) != 0) {
+            std::fprintf(stderr, "mrv_rank_buffers_alloc: %s\n", mrv_last_error());
+            std::exit(1);
+        }
+    }
     std::vector<std::thread> threads;
     for (int i = 0; i < args.n_devs; i++) threads.emplace_back(worker, std::cref(func), args, i, port, &res);
     for (auto& t : threads) t.join();
+    if (base && mrv_rank_buffers_free(base) != 0) std::exit(1);
     return res;
 }
 
@@ -195,6 +223,9 @@ void show_help(const char* argv0) {
                  "      -i[int]     timed iterations (default 100)\n"
                  "      -J[path]    also append one JSON line per size to this file: avg, median and 99th percentile\n"
                  "                  of the per-call time on rank 0 (not in the reference's harness)\n"
+                 "      -M          every rank allocates its own buffers with hipMalloc, as the reference's harness\n"
+                 "                  does; without it all buffers lie in one allocation, placed by the library\n"
+                 "                  (mrv_rank_buffers_alloc: large buffers an odd multiple of 128 MiB apart)\n"
                  "      -S          all ranks enqueue on ONE stream (not in the reference's harness: its ranks\n"
                  "                  are devices); without it every rank has a stream of its own\n"
                  "      -A -B       send/recv: sending node rank / dev (default 0 / 0)\n"
@@ -213,10 +244,11 @@ void print(T value) {
 int main(int argc, char* argv[]) {
     Arguments args;
     int ch;
-    while ((ch = getopt(argc, argv, "hSd:I:P:n:r:e:f:s:w:i:A:B:C:D:J:")) != EOF) {
+    while ((ch = getopt(argc, argv, "hSMd:I:P:n:r:e:f:s:w:i:A:B:C:D:J:")) != EOF) {
         switch (ch) {
             case 'h': show_help(argv[0]); return 0;
             case 'S': args.share = true; break;
+            case 'M': args.own_allocations = true; break;
             case 'J': args.json_path = optarg; break;
             case 'd': args.n_devs = std::atoi(optarg); break;
             case 'I': args.master_ip = optarg; break;

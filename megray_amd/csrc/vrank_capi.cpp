@@ -16,6 +16,7 @@
 #include "megray/hip_context.h"
 #include "vrank_engine.h"
 #include "vrank_kernels.h"
+#include "vrank_placement.h"
 #include "vrank_plan.h"
 
 struct mrv_comm {
@@ -479,6 +480,44 @@ int mrv_probe_bounded_wait(uint64_t limit_us, void* stream, uint64_t* gave_up) {
         (void)hipFree(words);
         *gave_up = host.timeouts;
         return st;
+    });
+}
+
+int mrv_rank_buffers_layout(int count, const size_t* bytes, size_t* offsets, size_t* total) {
+    return guarded([&] {
+        if (count < 0) MEGRAY_THROW("negative buffer count");
+        need(total, "total is null");
+        if (count > 0) {
+            need(bytes, "bytes is null");
+            need(offsets, "offsets is null");
+        }
+        if (!placement_layout(count, bytes, offsets, total)) MEGRAY_THROW("the buffers do not fit the address space");
+        return MEGRAY_OK;
+    });
+}
+
+int mrv_rank_buffers_alloc(int count, const size_t* bytes, void** ptrs, void** base) {
+    return guarded([&] {
+        if (count <= 0) MEGRAY_THROW("no buffers asked for");
+        need(bytes, "bytes is null");
+        need(ptrs, "ptrs is null");
+        need(base, "base is null");
+        *base = nullptr;
+        std::vector<size_t> offsets(static_cast<size_t>(count));
+        size_t total = 0;
+        if (!placement_layout(count, bytes, offsets.data(), &total)) MEGRAY_THROW("the buffers do not fit the address space");
+        void* p = nullptr;
+        HIP_CHECK(hipMalloc(&p, total));
+        for (int i = 0; i < count; ++i) ptrs[i] = static_cast<char*>(p) + offsets[size_t(i)];
+        *base = p;
+        return MEGRAY_OK;
+    });
+}
+
+int mrv_rank_buffers_free(void* base) {
+    return guarded([&] {
+        if (base) HIP_CHECK(hipFree(base));
+        return MEGRAY_OK;
     });
 }
 
