@@ -393,9 +393,13 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
             } else {
                 const PackLaunch& L = step.pack;
                 // the slice of every block this launch copies
-                const uint64_t per_tile = uint64_t(kThreads) * L.width;
+                // (blocks on 4-byte boundaries: tiles count whole 16-byte vectors, which start at the destination's
+                // first 16-byte boundary; a launch that reaches the last tile takes the block's end with it)
+                const uint64_t per_tile = uint64_t(kThreads) * pack_access_bytes(L.width);
                 const uint64_t slice_begin = L.first_tile * per_tile;
-                const uint64_t slice_bytes = std::min<uint64_t>(L.block_bytes - slice_begin, uint64_t(L.tiles_per_copy) * per_tile);
+                const bool last = L.first_tile + L.tiles_per_copy >= pack_tiles(L.block_bytes, L.width);
+                const uint64_t slice_bytes = last ? L.block_bytes - slice_begin
+                                                  : uint64_t(L.tiles_per_copy) * per_tile;
                 for (uint32_t c = 0; c < L.ncopies; ++c) {
                     mrv_plan_run run;
                     std::memset(&run, 0, sizeof(run));

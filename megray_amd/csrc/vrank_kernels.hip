@@ -50,31 +50,76 @@ __device__ __forceinline__ PackEnds pack_ends(const PackLaunch& L, uint32_t copy
     return {copy, 0, 0, copy, n};  // kPackAllGather: read once, write the block into every rank's buffer
 }
 
+// Where the 16-byte vectors of one block copy lie.  They start at the (first) destination's first 16-byte boundary,
+// `head` bytes into the block; `nvec` whole vectors follow, then `tail` bytes (head and tail are multiples of 4 below
+// 16, and 0 for blocks on 16-byte boundaries).  Lane `tid` of tile `t` takes vector t * kThreads + tid - pad, where
+// `pad` (below kThreads) is chosen so that tile 1 starts on a 1 KiB boundary of the destination: whole tiles then
+// store whole cache lines whatever the block's offset.
+struct PackVectors {
+    uint32_t head, tail, pad;
+    uint64_t nvec;
+};
+__device__ __forceinline__ PackVectors pack_vectors(const PackLaunch& L, const PackEnds& e, uint64_t dst_off) {
+    constexpr uint64_t kTileBytes = uint64_t(kThreads) * kVecBytes;
+    const uintptr_t dst = reinterpret_cast<uintptr_t>(L.out[e.dst_rank]) + dst_off;
+    uint64_t head = (0 - dst) & (kVecBytes - 1);
+    if (head > L.block_bytes) head = L.block_bytes;
+    const uint64_t nvec = (L.block_bytes - head) / kVecBytes;
+    const uint64_t before = ((0 - (dst + head)) & (kTileBytes - 1)) / kVecBytes;  // vectors in front of the 1 KiB boundary
+    const uint32_t pad = uint32_t((kThreads - before) % kThreads);
+    return {uint32_t(head), uint32_t(L.block_bytes - head - nvec * kVecBytes), pad, nvec};
+}
+
+// The 4-byte words in front of the first and behind the last vector of a block copy: lanes 0 .. 5 of one wavefront.
+__device__ __forceinline__ void pack_edge_words(const PackLaunch& L, const PackEnds& e, const PackVectors& pv,
+                                                const char* src, uint64_t dst_off, uint32_t tid) {
+    const uint32_t hw = pv.head / 4, tw = pv.tail / 4;
+    if (tid >= hw + tw) return;
+    const uint64_t off = tid < hw ? uint64_t(tid) * 4 : pv.head + pv.nvec * kVecBytes + uint64_t(tid - hw) * 4;
+    const uint32_t x = load_w<uint32_t>(src + off);
+    for (uint32_t m = 0; m < e.ndst; ++m) store_w<uint32_t>(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + off, x);
+}
+
+// Tile `tile` of a block copy, by one wavefront: whole tiles through buffer instructions, the partial ones at the
+// block's ends lane by lane.  `src` and `dst_off` address the block's first byte.
+__device__ __forceinline__ void pack_vector_tile(const PackLaunch& L, const PackEnds& e, const PackVectors& pv,
+                                                 const char* src, uint64_t dst_off, uint64_t tile, uint32_t tid) {
+    const uint64_t t0 = tile * kThreads;  // this tile's lanes take vectors [t0 - pad, t0 - pad + kThreads)
+    if (t0 >= pv.pad && t0 - pv.pad + kThreads <= pv.nvec) {
+        const uint64_t off = pv.head + (t0 - pv.pad) * kVecBytes;
+        const u32x4 x = load_tile_vec(src + off, tid);
+        for (uint32_t m = 0; m < e.ndst; ++m)
+            store_tile_vec(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + off, tid, x);
+    } else if (t0 + tid >= pv.pad && t0 + tid - pv.pad < pv.nvec) {
+        const uint64_t off = pv.head + (t0 + tid - pv.pad) * kVecBytes;
+        const u32x4 x = load_vec(src + off);
+        for (uint32_t m = 0; m < e.ndst; ++m) store_vec(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + off, x);
+    }
+}
+
 // One wavefront per tile of kThreads accesses of W bytes: short or narrow block copies.
 template <typename W>
 __global__ void __launch_bounds__(kThreads) pack_kernel(const PackLaunch L) {
     const uint32_t copy = blockIdx.x / L.tiles_per_copy;
     const uint64_t tile = L.first_tile + (blockIdx.x - copy * L.tiles_per_copy);
     const PackEnds e = pack_ends(L, copy);
-    const uint64_t base = tile * kThreads * sizeof(W);
-    const char* src = static_cast<const char*>(L.in[e.src_rank]) + e.src_block * L.block_bytes + base;
-    const uint64_t dst_off = e.dst_block * L.block_bytes + base;
-    const uint64_t left = (L.block_bytes - base) / sizeof(W);
     const uint32_t tid = threadIdx.x;
-    if (left >= kThreads) {
-        if constexpr (sizeof(W) == kVecBytes) {
-            const u32x4 x = load_tile_vec(src, tid);
-            for (uint32_t m = 0; m < e.ndst; ++m)
-                store_tile_vec(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off, tid, x);
-        } else {
+    if constexpr (sizeof(W) == kVecBytes) {
+        const char* src = static_cast<const char*>(L.in[e.src_rank]) + e.src_block * L.block_bytes;
+        const uint64_t dst_off = e.dst_block * L.block_bytes;
+        const PackVectors pv = pack_vectors(L, e, dst_off);
+        pack_vector_tile(L, e, pv, src, dst_off, tile, tid);
+        if (tile == 0) pack_edge_words(L, e, pv, src, dst_off, tid);
+    } else {
+        const uint64_t base = tile * kThreads * sizeof(W);
+        const char* src = static_cast<const char*>(L.in[e.src_rank]) + e.src_block * L.block_bytes + base;
+        const uint64_t dst_off = e.dst_block * L.block_bytes + base;
+        const uint64_t left = (L.block_bytes - base) / sizeof(W);
+        if (tid < left) {
             const W x = load_w<W>(src + tid * sizeof(W));
             for (uint32_t m = 0; m < e.ndst; ++m)
                 store_w<W>(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + tid * sizeof(W), x);
         }
-    } else if (tid < left) {
-        const W x = load_w<W>(src + tid * sizeof(W));
-        for (uint32_t m = 0; m < e.ndst; ++m)
-            store_w<W>(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + tid * sizeof(W), x);
     }
 }
 
@@ -87,7 +132,6 @@ __global__ void __launch_bounds__(kThreads) pack_kernel(const PackLaunch L) {
 // 1 -> 1 copies 84 - 87 % against 83 - 84 %.
 __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(const PackLaunch L) {
     constexpr uint32_t W = kGroupWaves;
-    constexpr uint32_t kTileBytes = kThreads * kVecBytes;
     __shared__ u32x4 stage[W][kThreads];
     __shared__ uint32_t staged[W];
     const uint32_t tid = threadIdx.x % kThreads;
@@ -97,25 +141,22 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
     const uint64_t first = L.first_tile + uint64_t(group / kGroupStride) * (W * kGroupStride) + group % kGroupStride;
     const PackEnds e = pack_ends(L, copy);
     const char* src = static_cast<const char*>(L.in[e.src_rank]) + e.src_block * L.block_bytes;
-    const uint64_t dst_base = e.dst_block * L.block_bytes;
+    const uint64_t dst_off = e.dst_block * L.block_bytes;
+    const PackVectors pv = pack_vectors(L, e, dst_off);
+    if (first == 0 && wave == 0) pack_edge_words(L, e, pv, src, dst_off, tid);
 
+    // tile t holds vectors [t * kThreads - pad, ...): whole if all of them exist
     const uint64_t mine = first + wave * kGroupStride;
-    const uint64_t mine_off = mine * kTileBytes;
-    const bool whole = mine_off + kTileBytes <= L.block_bytes;
+    const auto whole_tile = [&](uint64_t t) { return t * kThreads >= pv.pad && t * kThreads - pv.pad + kThreads <= pv.nvec; };
+    const auto tile_off = [&](uint64_t t) { return pv.head + (t * kThreads - pv.pad) * kVecBytes; };  // whole tiles only
+    const bool whole = whole_tile(mine);
     u32x4 x = {0u, 0u, 0u, 0u};
-    if (whole) {
-        x = load_tile_vec(src + mine_off, tid);
-    } else if (mine_off < L.block_bytes) {
-        // the block's last, partial tile: this wavefront copies it to every destination itself
-        const uint64_t off = mine_off + tid * kVecBytes;
-        if (off < L.block_bytes) {
-            const u32x4 v = load_w<u32x4>(src + off);
-            for (uint32_t m = 0; m < e.ndst; ++m)
-                store_w<u32x4>(static_cast<char*>(L.out[e.dst_rank + m]) + dst_base + off, v);
-        }
-    }
+    if (whole)
+        x = load_tile_vec(src + tile_off(mine), tid);
+    else
+        pack_vector_tile(L, e, pv, src, dst_off, mine, tid);  // a partial tile at either end: copied to every destination here
     if (e.ndst == 1) {
-        if (whole) store_tile_vec(static_cast<char*>(L.out[e.dst_rank]) + dst_base + mine_off, tid, x);
+        if (whole) store_tile_vec(static_cast<char*>(L.out[e.dst_rank]) + dst_off + tile_off(mine), tid, x);
         return;
     }
     stage[wave][tid] = x;
@@ -123,10 +164,9 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
     __syncthreads();
     for (uint32_t m = 0; m < e.ndst; ++m) {
         const uint32_t k = (wave + m) % W;
-        if (staged[k]) {
-            const uint64_t off = (first + uint64_t(k) * kGroupStride) * kTileBytes;
-            store_tile_vec(static_cast<char*>(L.out[e.dst_rank + m]) + dst_base + off, tid, stage[k][tid]);
-        }
+        if (staged[k])
+            store_tile_vec(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + tile_off(first + uint64_t(k) * kGroupStride),
+                           tid, stage[k][tid]);
     }
 }
 
@@ -192,11 +232,10 @@ const void* tree_kernel_for(const TreeLaunch&, DType dtype, ReduceOp op) {
 
 const void* pack_kernel_for(const PackLaunch& L) {
     void (*fn)(const PackLaunch) = nullptr;
-    if (L.waves == kGroupWaves) return L.width == kVecBytes ? reinterpret_cast<const void*>(&pack_group_kernel) : nullptr;
-    switch (L.width) {
+    const uint32_t access = pack_access_bytes(L.width);
+    if (L.waves == kGroupWaves) return access == kVecBytes ? reinterpret_cast<const void*>(&pack_group_kernel) : nullptr;
+    switch (access) {
         case 16: fn = pack_kernel<u32x4>; break;
-        case 8: fn = pack_kernel<u32x2>; break;
-        case 4: fn = pack_kernel<uint32_t>; break;
         case 2: fn = pack_kernel<uint16_t>; break;
         case 1: fn = pack_kernel<uint8_t>; break;
         default: break;

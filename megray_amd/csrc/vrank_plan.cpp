@@ -157,23 +157,35 @@ private:
     void emit_general() {
         const uint64_t epv = kVecBytes / m_elem;
         // long vector bodies take the group form (four wavefronts per workgroup)
+        // Element types of 4 and 8 bytes go 16 bytes per lane whatever the offsets (4-byte alignment suffices for
+        // the 128-bit accesses of gfx950): buffers whose offsets from a 16-byte boundary differ (m_plain), and runs
+        // whose outputs are shifted against their inputs by a part of a vector (reduce_scatter with a receive
+        // length that is no multiple of 16 bytes, the copies of the two-phase and ring schedules).
+        const bool natural = m_plain || (m_aligned && m_elem >= 4);
+        auto same_phase = [&](const Run& r) { return m_aligned && r.in_begin % epv == r.out_begin % epv; };
         uint64_t vector_elems = 0;
         for (const Run& r : m_runs)
-            if (m_plain || (m_aligned && r.in_begin % epv == r.out_begin % epv)) vector_elems += r.count;
+            if (natural || same_phase(r)) vector_elems += r.count;
         m_waves = vector_elems / (kThreads * epv) >= kGroupMinTiles ? kGroupWaves : 1;
         open_launch();
         for (const Run& r : m_runs) {
-            const bool vector = m_plain || (m_aligned && (r.in_begin % epv == r.out_begin % epv));
+            const bool vector = natural || same_phase(r);
             uint64_t head = 0, body = 0;
             if (m_plain) {
                 body = r.count / epv * epv;  // no grid to reach: every address is as aligned as it gets
-            } else if (vector) {
+            } else if (same_phase(r)) {
                 // the body starts where inputs and outputs both sit on the coarsest grid they share
                 uint64_t grid = m_grid;
                 const uint64_t skew = (r.in_begin - r.out_begin) * m_elem;  // unsigned wrap is fine mod 2^k
                 while (grid > kVecBytes && (skew & (grid - 1))) grid >>= 1;
                 const uint64_t at = (m_misalign + r.in_begin * m_elem) & (grid - 1);
                 head = std::min<uint64_t>(((grid - at) & (grid - 1)) / m_elem, r.count);
+                body = (r.count - head) / epv * epv;
+            } else if (vector) {
+                // shifted by a part of a vector: the body starts where the OUTPUTS sit on the grid, so the stores
+                // are aligned and cover whole cache lines; the loads take the inputs as they lie
+                const uint64_t at = (m_misalign + r.out_begin * m_elem) & (m_grid - 1);
+                head = std::min<uint64_t>(((m_grid - at) & (m_grid - 1)) / m_elem, r.count);
                 body = (r.count - head) / epv * epv;
             }
             if (!body) {
@@ -551,10 +563,10 @@ Status add_pack(Plan& plan, const void* const* in, void* const* out, uint32_t nr
     L.root = root;
     L.ncopies = ncopies;
     L.width = common_width(block_bytes, in, out_c, nranks);
-    const uint64_t per_tile = uint64_t(kThreads) * L.width;
-    const uint64_t tiles = (block_bytes + per_tile - 1) / per_tile;
+    const uint32_t access = pack_access_bytes(L.width);
+    const uint64_t tiles = pack_tiles(block_bytes, L.width);
     // long blocks of 16-byte accesses take the group form
-    L.waves = (L.width == kVecBytes && tiles >= kGroupMinTiles / 4) ? kGroupWaves : 1;
+    L.waves = (access == kVecBytes && tiles >= kGroupMinTiles / 4) ? kGroupWaves : 1;
     // A grid holds 2^31 - 1 workgroups: blocks whose tiles, over all copies, outnumber that are cut into
     // slices of tiles, one launch each (the reference's per-peer copies have no such limit either).
     const uint64_t span = uint64_t(kGroupWaves) * kGroupStride;  // tiles a run of kGroupStride workgroups covers

@@ -1,0 +1,142 @@
+"""Blocks and runs that start on 4- or 8-byte boundaries only (fp32 / int64 buffers with lengths that are no multiple
+of 16 bytes, buffers at differing offsets): the pack kernels move 16 bytes per lane from the destination's first
+16-byte boundary on and copy the few words around the vectors one by one; reduce_scatter with such a receive length
+folds 16 bytes per lane with stores on 16-byte boundaries.  Checked against the oracle's literal replays, with
+guard bytes around every output."""
+import numpy as np
+import pytest
+import torch
+
+import megray_amd as mr
+import oracle as orc
+from gpu_util import rand_array
+
+pytestmark = pytest.mark.gpu
+GUARD = 64
+FILL = 0x5C
+
+
+def device_in(arr, offset):
+    raw = np.ascontiguousarray(arr).view(np.uint8).reshape(-1)
+    buf = torch.empty(raw.size + offset + 64, dtype=torch.uint8, device="cuda")
+    view = buf[offset:offset + raw.size]
+    if raw.size:
+        view.copy_(torch.from_numpy(raw.copy()))
+    return view
+
+
+class Guarded:
+    """An output of `nbytes` bytes at `offset` from a 256-byte boundary with GUARD bytes of a fill pattern on
+    both sides."""
+
+    def __init__(self, nbytes, offset):
+        self.buf = torch.full((256 + nbytes + 2 * GUARD + 64,), FILL, dtype=torch.uint8, device="cuda")
+        lo = 256 - GUARD + offset  # the torch allocation is 256-byte aligned
+        self.lo, self.nbytes = lo + GUARD, nbytes
+        self.view = self.buf[self.lo:self.lo + nbytes]
+
+    def check(self, want, what):
+        host = self.buf.cpu().numpy()
+        got = host[self.lo:self.lo + self.nbytes]
+        assert np.array_equal(got, np.ascontiguousarray(want).view(np.uint8).reshape(-1)), what
+        assert (host[self.lo - GUARD:self.lo] == FILL).all(), what + ": bytes in front of the output were written"
+        assert (host[self.lo + self.nbytes:self.lo + self.nbytes + GUARD] == FILL).all(), what + ": bytes behind the output were written"
+
+
+# lengths in elements: a few words, under one tile, several tiles with an odd end, group form (>= 128 tiles per block)
+LENGTHS = {orc.FLOAT32: (1, 2, 3, 5, 7, 250, 1027, 4099, 33001 * 4 + 1, 33001 * 4 + 2, 33001 * 4 + 3),
+           orc.INT64: (1, 3, 125, 1027, 16501 * 4 + 1)}
+
+
+@pytest.mark.parametrize("dtype", [orc.FLOAT32, orc.INT64])
+@pytest.mark.parametrize("nranks", [2, 3, 8])
+def test_pack_collectives_on_word_boundaries(dtype, nranks):
+    rng = np.random.default_rng(700 + dtype * 10 + nranks)
+    size = orc.dtype_size(dtype)
+    for length in LENGTHS[dtype]:
+        if nranks == 8 and length > 40000 and dtype == orc.INT64:
+            continue
+        for variant in range(2):
+            # 0: every buffer on a 256-byte boundary (only the block length is odd); 1: every buffer at its own offset
+            in_off = [0] * nranks if variant == 0 else [size * ((3 * r + 1) % 4) for r in range(nranks)]
+            out_off = [0] * nranks if variant == 0 else [size * ((r + 2) % 4) for r in range(nranks)]
+            what = f"dtype={dtype} N={nranks} len={length} offsets={variant}"
+            ins = [rand_array(dtype, nranks * length, rng) for _ in range(nranks)]
+            parts = [x[:length] for x in ins]
+            # all_to_all
+            d_in = [device_in(x, in_off[r]) for r, x in enumerate(ins)]
+            outs = [Guarded(nranks * length * size, out_off[r]) for r in range(nranks)]
+            mr.all_to_all(d_in, [o.view for o in outs], length, dtype)
+            torch.cuda.synchronize()
+            for r, w in enumerate(orc.ucx_all_to_all(ins, dtype)):
+                outs[r].check(w, "all_to_all " + what)
+            # all_gather (every destination has its own alignment in variant 1)
+            d_in = [device_in(x, in_off[r]) for r, x in enumerate(parts)]
+            outs = [Guarded(nranks * length * size, out_off[r]) for r in range(nranks)]
+            mr.all_gather(d_in, [o.view for o in outs], length, dtype)
+            torch.cuda.synchronize()
+            for r, w in enumerate(orc.ucx_all_gather(parts, dtype)):
+                outs[r].check(w, "all_gather " + what)
+            root = nranks - 1
+            # scatter
+            d_root = device_in(ins[root], in_off[root])
+            outs = [Guarded(length * size, out_off[r]) for r in range(nranks)]
+            mr.scatter(d_root, [o.view for o in outs], length, dtype, root)
+            torch.cuda.synchronize()
+            want = orc.ucx_scatter([ins[root] if r == root else None for r in range(nranks)], dtype, root)
+            for r in range(nranks):
+                outs[r].check(want[r], "scatter " + what)
+            # gather
+            d_in = [device_in(x, in_off[r]) for r, x in enumerate(parts)]
+            out = Guarded(nranks * length * size, out_off[root])
+            mr.gather(d_in, out.view, length, dtype, root)
+            torch.cuda.synchronize()
+            out.check(orc.ucx_gather(parts, dtype, root)[root], "gather " + what)
+            # broadcast
+            d_root = device_in(parts[root], in_off[root])
+            outs = [Guarded(length * size, out_off[r]) for r in range(nranks)]
+            mr.broadcast(d_root, [o.view for o in outs], length, dtype, root)
+            torch.cuda.synchronize()
+            want = orc.ucx_broadcast(parts, dtype, root)
+            for r in range(nranks):
+                outs[r].check(want[r], "broadcast " + what)
+
+
+def test_the_vector_forms_are_what_runs():
+    """describe(): blocks on 4-byte boundaries still go through the 16-byte kernels (group form when long), and a
+    reduce_scatter whose receive length is no multiple of 16 bytes keeps vector bodies."""
+    nranks, length = 8, 33001 * 4 + 1
+    send = [(1 << 40) + (r << 32) for r in range(nranks)]
+    recv = [(2 << 40) + (r << 34) for r in range(nranks)]
+    runs, _, _ = mr.describe(mr.Collective.ALL_TO_ALL, send, recv, length, orc.FLOAT32)
+    assert runs and all(r["vector"] == 4 and r["waves"] == 4 for r in runs)
+    runs, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, send, recv, length, orc.FLOAT32)
+    body = sum(r["count"] for r in runs if r["vector"] == 1)
+    assert body >= nranks * length - nranks * 3 * 300  # all but heads and tails of at most a tile's worth per run
+    assert all(r["waves"] == 4 for r in runs)
+
+
+@pytest.mark.parametrize("dtype", [orc.FLOAT32, orc.INT32, orc.FLOAT64, orc.INT64])
+def test_reduce_scatter_with_receive_lengths_off_the_vector_grid(dtype):
+    rng = np.random.default_rng(800 + dtype)
+    size = orc.dtype_size(dtype)
+    for nranks in (2, 3, 5, 8):
+        for recvlen in (3, 1027, 4099, (33001 * 16 + 4) // size * 1 + 1):
+            ins = [rand_array(dtype, nranks * recvlen, rng) for _ in range(nranks)]
+            for op in (orc.SUM, orc.MAX):
+                for order in (orc.ORDER_UCX, orc.ORDER_SHM):
+                    want = orc.fold_reduce_scatter(ins, dtype, op, order)
+                    d_in = [device_in(x, 0) for x in ins]
+                    outs = [Guarded(recvlen * size, 0) for _ in range(nranks)]
+                    mr.reduce_scatter(d_in, [o.view for o in outs], recvlen, dtype, op, order)
+                    torch.cuda.synchronize()
+                    for r in range(nranks):
+                        outs[r].check(want[r], f"reduce_scatter dtype={dtype} N={nranks} recvlen={recvlen} op={op} order={order}")
+            if dtype in (orc.FLOAT32, orc.FLOAT64):
+                want = orc.ucx_reduce_scatter(ins, dtype, orc.SUM)  # the literal replay
+                d_in = [device_in(x, 0) for x in ins]
+                outs = [Guarded(recvlen * size, 0) for _ in range(nranks)]
+                mr.reduce_scatter(d_in, [o.view for o in outs], recvlen, dtype, orc.SUM)
+                torch.cuda.synchronize()
+                for r in range(nranks):
+                    outs[r].check(want[r], "reduce_scatter vs literal replay")
