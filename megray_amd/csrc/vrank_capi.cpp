@@ -393,11 +393,12 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
             } else {
                 const PackLaunch& L = step.pack;
                 // the slice of every block this launch copies
-                // (blocks on 4-byte boundaries: tiles count whole 16-byte vectors, which start at the destination's
-                // first 16-byte boundary; a launch that reaches the last tile takes the block's end with it)
-                const uint64_t per_tile = uint64_t(kThreads) * pack_access_bytes(L.width);
-                const uint64_t slice_begin = L.first_tile * per_tile;
-                const bool last = L.first_tile + L.tiles_per_copy >= pack_tiles(L.block_bytes, L.width);
+                // (tiles count whole 16-byte vectors, which start at the destination's first 16-byte boundary, so
+                // this is the slice up to a tile's worth of bytes; a launch that reaches the last tile takes the
+                // block's end with it)
+                const uint64_t per_tile = uint64_t(kThreads) * kVecBytes;
+                const uint64_t slice_begin = std::min(L.first_tile * per_tile, L.block_bytes);
+                const bool last = L.first_tile + L.tiles_per_copy >= pack_tiles(L.block_bytes);
                 const uint64_t slice_bytes = last ? L.block_bytes - slice_begin
                                                   : uint64_t(L.tiles_per_copy) * per_tile;
                 for (uint32_t c = 0; c < L.ncopies; ++c) {

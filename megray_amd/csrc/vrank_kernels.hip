@@ -37,6 +37,18 @@ __device__ __forceinline__ void store_w(char* p, W x) {
     __builtin_nontemporal_store(x, reinterpret_cast<W*>(p));
 }
 
+// 128-bit accesses of single lanes at any byte address.
+typedef uint32_t u32x4_a1 __attribute__((ext_vector_type(4), aligned(1)));
+__device__ __forceinline__ u32x4 load_vec_bytes(const char* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4_a1*>(p));
+}
+__device__ __forceinline__ void store_vec_bytes(char* p, u32x4 x) {
+    __builtin_nontemporal_store(u32x4_a1(x), reinterpret_cast<u32x4_a1*>(p));
+}
+__device__ __forceinline__ bool on_words(const void* p) {
+    return (reinterpret_cast<uintptr_t>(p) & 3u) == 0;
+}
+
 // Decodes copy `copy` of a pack launch into its endpoints.
 struct PackEnds {
     uint32_t src_rank, src_block, dst_rank, dst_block, ndst;
@@ -51,10 +63,10 @@ __device__ __forceinline__ PackEnds pack_ends(const PackLaunch& L, uint32_t copy
 }
 
 // Where the 16-byte vectors of one block copy lie.  They start at the (first) destination's first 16-byte boundary,
-// `head` bytes into the block; `nvec` whole vectors follow, then `tail` bytes (head and tail are multiples of 4 below
-// 16, and 0 for blocks on 16-byte boundaries).  Lane `tid` of tile `t` takes vector t * kThreads + tid - pad, where
-// `pad` (below kThreads) is chosen so that tile 1 starts on a 1 KiB boundary of the destination: whole tiles then
-// store whole cache lines whatever the block's offset.
+// `head` bytes into the block; `nvec` whole vectors follow, then `tail` bytes (both below 16, and 0 for blocks on
+// 16-byte boundaries).  Lane `tid` of tile `t` takes vector t * kThreads + tid - pad, where `pad` (below kThreads)
+// is chosen so that tile 1 starts on a 1 KiB boundary of the destination: whole tiles then store whole cache lines
+// whatever the block's offset.
 struct PackVectors {
     uint32_t head, tail, pad;
     uint64_t nvec;
@@ -70,14 +82,33 @@ __device__ __forceinline__ PackVectors pack_vectors(const PackLaunch& L, const P
     return {uint32_t(head), uint32_t(L.block_bytes - head - nvec * kVecBytes), pad, nvec};
 }
 
-// The 4-byte words in front of the first and behind the last vector of a block copy: lanes 0 .. 5 of one wavefront.
-__device__ __forceinline__ void pack_edge_words(const PackLaunch& L, const PackEnds& e, const PackVectors& pv,
+// The bytes in front of the first and behind the last vector of a block copy, in units of the blocks' common
+// alignment (4 bytes at most): at most 30 lanes of one wavefront.
+template <typename U>
+__device__ __forceinline__ void pack_edge_units(const PackLaunch& L, const PackEnds& e, const PackVectors& pv,
                                                 const char* src, uint64_t dst_off, uint32_t tid) {
-    const uint32_t hw = pv.head / 4, tw = pv.tail / 4;
-    if (tid >= hw + tw) return;
-    const uint64_t off = tid < hw ? uint64_t(tid) * 4 : pv.head + pv.nvec * kVecBytes + uint64_t(tid - hw) * 4;
-    const uint32_t x = load_w<uint32_t>(src + off);
-    for (uint32_t m = 0; m < e.ndst; ++m) store_w<uint32_t>(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + off, x);
+    const uint32_t hu = pv.head / sizeof(U), tu = pv.tail / sizeof(U);
+    if (tid >= hu + tu) return;
+    const uint64_t off = tid < hu ? uint64_t(tid) * sizeof(U)
+                                  : pv.head + pv.nvec * kVecBytes + uint64_t(tid - hu) * sizeof(U);
+    const U x = load_w<U>(src + off);
+    for (uint32_t m = 0; m < e.ndst; ++m) store_w<U>(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + off, x);
+}
+__device__ __forceinline__ void pack_edges(const PackLaunch& L, const PackEnds& e, const PackVectors& pv,
+                                           const char* src, uint64_t dst_off, uint32_t tid) {
+    if (L.width >= 4) pack_edge_units<uint32_t>(L, e, pv, src, dst_off, tid);
+    else if (L.width == 2) pack_edge_units<uint16_t>(L, e, pv, src, dst_off, tid);
+    else pack_edge_units<uint8_t>(L, e, pv, src, dst_off, tid);
+}
+
+// One whole tile to destination `m`: a buffer store where the address allows it (4-byte boundary; destination 0 is
+// on a 16-byte boundary by construction, the others usually share its offset), else lane by lane.
+__device__ __forceinline__ void pack_store_tile(char* dst, uint32_t tid, u32x4 x) {
+    if (on_words(dst)) store_tile_vec(dst, tid, x);
+    else store_vec_bytes(dst + tid * kVecBytes, x);
+}
+__device__ __forceinline__ u32x4 pack_load_tile(const char* src, uint32_t tid) {
+    return on_words(src) ? load_tile_vec(src, tid) : load_vec_bytes(src + tid * kVecBytes);
 }
 
 // Tile `tile` of a block copy, by one wavefront: whole tiles through buffer instructions, the partial ones at the
@@ -87,43 +118,31 @@ __device__ __forceinline__ void pack_vector_tile(const PackLaunch& L, const Pack
     const uint64_t t0 = tile * kThreads;  // this tile's lanes take vectors [t0 - pad, t0 - pad + kThreads)
     if (t0 >= pv.pad && t0 - pv.pad + kThreads <= pv.nvec) {
         const uint64_t off = pv.head + (t0 - pv.pad) * kVecBytes;
-        const u32x4 x = load_tile_vec(src + off, tid);
+        const u32x4 x = pack_load_tile(src + off, tid);
         for (uint32_t m = 0; m < e.ndst; ++m)
-            store_tile_vec(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + off, tid, x);
+            pack_store_tile(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + off, tid, x);
     } else if (t0 + tid >= pv.pad && t0 + tid - pv.pad < pv.nvec) {
         const uint64_t off = pv.head + (t0 + tid - pv.pad) * kVecBytes;
-        const u32x4 x = load_vec(src + off);
-        for (uint32_t m = 0; m < e.ndst; ++m) store_vec(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + off, x);
+        const u32x4 x = load_vec_bytes(src + off);
+        for (uint32_t m = 0; m < e.ndst; ++m)
+            store_vec_bytes(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + off, x);
     }
 }
 
-// One wavefront per tile of kThreads accesses of W bytes: short or narrow block copies.
-template <typename W>
+// One wavefront per tile: short block copies.
 __global__ void __launch_bounds__(kThreads) pack_kernel(const PackLaunch L) {
     const uint32_t copy = blockIdx.x / L.tiles_per_copy;
     const uint64_t tile = L.first_tile + (blockIdx.x - copy * L.tiles_per_copy);
     const PackEnds e = pack_ends(L, copy);
     const uint32_t tid = threadIdx.x;
-    if constexpr (sizeof(W) == kVecBytes) {
-        const char* src = static_cast<const char*>(L.in[e.src_rank]) + e.src_block * L.block_bytes;
-        const uint64_t dst_off = e.dst_block * L.block_bytes;
-        const PackVectors pv = pack_vectors(L, e, dst_off);
-        pack_vector_tile(L, e, pv, src, dst_off, tile, tid);
-        if (tile == 0) pack_edge_words(L, e, pv, src, dst_off, tid);
-    } else {
-        const uint64_t base = tile * kThreads * sizeof(W);
-        const char* src = static_cast<const char*>(L.in[e.src_rank]) + e.src_block * L.block_bytes + base;
-        const uint64_t dst_off = e.dst_block * L.block_bytes + base;
-        const uint64_t left = (L.block_bytes - base) / sizeof(W);
-        if (tid < left) {
-            const W x = load_w<W>(src + tid * sizeof(W));
-            for (uint32_t m = 0; m < e.ndst; ++m)
-                store_w<W>(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + tid * sizeof(W), x);
-        }
-    }
+    const char* src = static_cast<const char*>(L.in[e.src_rank]) + e.src_block * L.block_bytes;
+    const uint64_t dst_off = e.dst_block * L.block_bytes;
+    const PackVectors pv = pack_vectors(L, e, dst_off);
+    pack_vector_tile(L, e, pv, src, dst_off, tile, tid);
+    if (tile == 0) pack_edges(L, e, pv, src, dst_off, tid);
 }
 
-// Group form of the pack kernel for long blocks of 16-byte accesses: a workgroup of kGroupWaves
+// Group form of the pack kernel for long blocks: a workgroup of kGroupWaves
 // wavefronts owns kGroupWaves tiles of one block copy, kGroupStride tiles apart; wavefront w loads
 // tile w.  With one destination it stores that tile; with N destinations (all_gather) the tiles are
 // exchanged through LDS and wavefront w stores destination m of tile (w + m) % kGroupWaves, so the
@@ -143,7 +162,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
     const char* src = static_cast<const char*>(L.in[e.src_rank]) + e.src_block * L.block_bytes;
     const uint64_t dst_off = e.dst_block * L.block_bytes;
     const PackVectors pv = pack_vectors(L, e, dst_off);
-    if (first == 0 && wave == 0) pack_edge_words(L, e, pv, src, dst_off, tid);
+    if (first == 0 && wave == 0) pack_edges(L, e, pv, src, dst_off, tid);
 
     // tile t holds vectors [t * kThreads - pad, ...): whole if all of them exist
     const uint64_t mine = first + wave * kGroupStride;
@@ -152,11 +171,11 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
     const bool whole = whole_tile(mine);
     u32x4 x = {0u, 0u, 0u, 0u};
     if (whole)
-        x = load_tile_vec(src + tile_off(mine), tid);
+        x = pack_load_tile(src + tile_off(mine), tid);
     else
         pack_vector_tile(L, e, pv, src, dst_off, mine, tid);  // a partial tile at either end: copied to every destination here
     if (e.ndst == 1) {
-        if (whole) store_tile_vec(static_cast<char*>(L.out[e.dst_rank]) + dst_off + tile_off(mine), tid, x);
+        if (whole) pack_store_tile(static_cast<char*>(L.out[e.dst_rank]) + dst_off + tile_off(mine), tid, x);
         return;
     }
     stage[wave][tid] = x;
@@ -165,8 +184,8 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
     for (uint32_t m = 0; m < e.ndst; ++m) {
         const uint32_t k = (wave + m) % W;
         if (staged[k])
-            store_tile_vec(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + tile_off(first + uint64_t(k) * kGroupStride),
-                           tid, stage[k][tid]);
+            pack_store_tile(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + tile_off(first + uint64_t(k) * kGroupStride),
+                            tid, stage[k][tid]);
     }
 }
 
@@ -231,16 +250,8 @@ const void* tree_kernel_for(const TreeLaunch&, DType dtype, ReduceOp op) {
 }
 
 const void* pack_kernel_for(const PackLaunch& L) {
-    void (*fn)(const PackLaunch) = nullptr;
-    const uint32_t access = pack_access_bytes(L.width);
-    if (L.waves == kGroupWaves) return access == kVecBytes ? reinterpret_cast<const void*>(&pack_group_kernel) : nullptr;
-    switch (access) {
-        case 16: fn = pack_kernel<u32x4>; break;
-        case 2: fn = pack_kernel<uint16_t>; break;
-        case 1: fn = pack_kernel<uint8_t>; break;
-        default: break;
-    }
-    return reinterpret_cast<const void*>(fn);
+    return L.waves == kGroupWaves ? reinterpret_cast<const void*>(&pack_group_kernel)
+                                  : reinterpret_cast<const void*>(&pack_kernel);
 }
 
 hipError_t enqueue(const void* kernel, uint32_t grid, uint32_t block, const void* launch, hipStream_t stream) {

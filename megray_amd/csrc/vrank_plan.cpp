@@ -563,10 +563,8 @@ Status add_pack(Plan& plan, const void* const* in, void* const* out, uint32_t nr
     L.root = root;
     L.ncopies = ncopies;
     L.width = common_width(block_bytes, in, out_c, nranks);
-    const uint32_t access = pack_access_bytes(L.width);
-    const uint64_t tiles = pack_tiles(block_bytes, L.width);
-    // long blocks of 16-byte accesses take the group form
-    L.waves = (access == kVecBytes && tiles >= kGroupMinTiles / 4) ? kGroupWaves : 1;
+    const uint64_t tiles = pack_tiles(block_bytes);
+    L.waves = tiles >= kGroupMinTiles / 4 ? kGroupWaves : 1;  // long blocks take the group form
     // A grid holds 2^31 - 1 workgroups: blocks whose tiles, over all copies, outnumber that are cut into
     // slices of tiles, one launch each (the reference's per-peer copies have no such limit either).
     const uint64_t span = uint64_t(kGroupWaves) * kGroupStride;  // tiles a run of kGroupStride workgroups covers
@@ -666,19 +664,11 @@ Status plan_broadcast(Plan& plan, const void* send_root, void* const* recv, uint
     }
     const void* in[kMaxRanks] = {};
     in[root] = send_root;
-    // 16-byte aligned everywhere: one pack copy, read once and written into every rank's buffer
-    const void* recv_c[kMaxRanks] = {};
-    for (uint32_t r = 0; r < nranks; ++r) recv_c[r] = recv[r];
-    if (bytes && common_width(bytes, in, recv_c, nranks) == kVecBytes) {
-        const uint64_t before = plan.steps.size();
-        Status st = add_pack(plan, in, recv, nranks, bytes, kPackBroadcast, root, 1);
-        if (st == MEGRAY_OK && plan.steps.size() > before) plan.bytes_written += bytes * (nranks - 1);
-        return st;
-    }
-    FoldBuilder copy(plan, in, recv, nranks, 1, nranks, elem_size, false);
-    copy.add_run(0, 0, len, uint8_t(root), 1, 0);
-    copy.finish();
-    return MEGRAY_OK;
+    // one pack copy, read once and written into every rank's buffer
+    const uint64_t before = plan.steps.size();
+    Status st = add_pack(plan, in, recv, nranks, bytes, kPackBroadcast, root, 1);
+    if (st == MEGRAY_OK && plan.steps.size() > before) plan.bytes_written += bytes * (nranks - 1);
+    return st;
 }
 
 Status plan_reduce(Plan& plan, const void* const* send, void* recv_root, uint32_t nranks, uint64_t len,

@@ -153,28 +153,24 @@ struct PackLaunch {
     uint32_t ncopies;
     uint32_t tiles_per_copy;
     uint32_t width;   // what every block address and the block size are a multiple of: 16, 8, 4, 2 or 1
-    uint32_t waves;   // wavefronts per workgroup: 1, or kGroupWaves (16-byte accesses, long blocks)
+    uint32_t waves;   // wavefronts per workgroup: 1, or kGroupWaves (long blocks)
     uint32_t groups_per_copy;  // group form: workgroups per block copy
     uint64_t first_tile;  // the launch covers tiles [first_tile, first_tile + tiles_per_copy) of every copy (blocks
                           // too long for one grid are cut into several launches; a multiple of the group span)
 };
 
-// Bytes a lane of the pack kernels moves per access.  Blocks on 4-byte boundaries go 16 bytes per lane like blocks on
-// 16-byte boundaries (the 128-bit accesses of gfx950 need 4-byte alignment only).  Each copy lays its tiles out from
-// the destination's side: vectors start at the destination's first 16-byte boundary and tile 1 starts at its first
-// 1 KiB boundary (tile 0 holds the up to 63 vectors in front of it), so that every whole tile's stores cover whole
-// cache lines whatever the block's offset; only the loads take the source as it lies.  The up to three 4-byte words
-// in front of the first and behind the last vector are copied one by one.
-inline uint32_t pack_access_bytes(uint32_t width) {
-    return width >= 4 ? 16u : width;
-}
-// Tiles (kThreads accesses each) of one block copy.  With 16-byte accesses a block has at most block_bytes / 16
-// whole vectors wherever they start, in whole tiles plus one partial tile at each end; there is always a tile 0,
-// which also takes the words around the vectors.
-inline uint64_t pack_tiles(uint64_t block_bytes, uint32_t width) {
-    const uint64_t access = pack_access_bytes(width);
-    if (access == 16) return (block_bytes / 16 + kThreads - 1) / kThreads + 1;
-    return (block_bytes + kThreads * access - 1) / (kThreads * access);
+// The pack kernels move 16 bytes per lane whatever the blocks' alignment.  Each copy lays its tiles out from the
+// destination's side: vectors start at the destination's first 16-byte boundary and tile 1 starts at its first 1 KiB
+// boundary (tile 0 holds the up to 63 vectors in front of it), so that every whole tile's stores cover whole cache
+// lines wherever the block lies; only the loads take the source as it lies (gfx950 serves 128-bit loads at any
+// byte address).  The up to 15 bytes in front of the first and behind the last vector are copied one by one, in
+// units of the blocks' common alignment (4 bytes at most).
+//
+// Tiles (kThreads vectors each) of one block copy: at most block_bytes / 16 whole vectors wherever they start, in
+// whole tiles plus one partial tile at each end; there is always a tile 0, which also takes the bytes around the
+// vectors.
+inline uint64_t pack_tiles(uint64_t block_bytes) {
+    return (block_bytes / 16 + kThreads - 1) / kThreads + 1;
 }
 // Tile sizes of the one-wavefront-per-tile kernels.  Measured on MI355X: one 16-byte vector per lane and
 // access beats every deeper unroll, for every fold width; a vector tile is kVecIters such groups

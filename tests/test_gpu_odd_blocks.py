@@ -1,8 +1,8 @@
-"""Blocks and runs that start on 4- or 8-byte boundaries only (fp32 / int64 buffers with lengths that are no multiple
-of 16 bytes, buffers at differing offsets): the pack kernels move 16 bytes per lane from the destination's first
-16-byte boundary on and copy the few words around the vectors one by one; reduce_scatter with such a receive length
-folds 16 bytes per lane with stores on 16-byte boundaries.  Checked against the oracle's literal replays, with
-guard bytes around every output."""
+"""Blocks and runs that do not start on 16-byte boundaries (lengths that are no multiple of 16 bytes, buffers at
+differing offsets): the pack kernels move 16 bytes per lane from the destination's first 16-byte boundary on, whatever
+the source's byte address, and copy the few bytes around the vectors one by one; reduce_scatter of 4- and 8-byte
+elements with such a receive length folds 16 bytes per lane with stores on 16-byte boundaries.  Checked against the
+oracle's literal replays, with guard bytes around every output."""
 import numpy as np
 import pytest
 import torch
@@ -45,21 +45,30 @@ class Guarded:
 
 # lengths in elements: a few words, under one tile, several tiles with an odd end, group form (>= 128 tiles per block)
 LENGTHS = {orc.FLOAT32: (1, 2, 3, 5, 7, 250, 1027, 4099, 33001 * 4 + 1, 33001 * 4 + 2, 33001 * 4 + 3),
-           orc.INT64: (1, 3, 125, 1027, 16501 * 4 + 1)}
+           orc.INT64: (1, 3, 125, 1027, 16501 * 4 + 1),
+           orc.UINT8: (1, 3, 15, 17, 31, 33, 1000, 4099, 33001 * 16 + 5),
+           orc.FLOAT16: (1, 3, 9, 1027, 33001 * 8 + 3)}
 
 
-@pytest.mark.parametrize("dtype", [orc.FLOAT32, orc.INT64])
+@pytest.mark.parametrize("dtype", [orc.FLOAT32, orc.INT64, orc.UINT8, orc.FLOAT16])
 @pytest.mark.parametrize("nranks", [2, 3, 8])
-def test_pack_collectives_on_word_boundaries(dtype, nranks):
+def test_pack_collectives_off_the_vector_grid(dtype, nranks):
     rng = np.random.default_rng(700 + dtype * 10 + nranks)
     size = orc.dtype_size(dtype)
     for length in LENGTHS[dtype]:
         if nranks == 8 and length > 40000 and dtype == orc.INT64:
             continue
-        for variant in range(2):
-            # 0: every buffer on a 256-byte boundary (only the block length is odd); 1: every buffer at its own offset
-            in_off = [0] * nranks if variant == 0 else [size * ((3 * r + 1) % 4) for r in range(nranks)]
-            out_off = [0] * nranks if variant == 0 else [size * ((r + 2) % 4) for r in range(nranks)]
+        slots = 16 // size  # element offsets within a 16-byte vector
+        for variant in range(3):
+            # 0: every buffer on a 256-byte boundary (only the block length is odd); 1: every buffer at its own
+            # offset; 2: all outputs at one offset, all inputs at another
+            if variant == 0:
+                in_off, out_off = [0] * nranks, [0] * nranks
+            elif variant == 1:
+                in_off = [size * ((3 * r + 1) % slots) for r in range(nranks)]
+                out_off = [size * ((r + 2) % slots) for r in range(nranks)]
+            else:
+                in_off, out_off = [size * (slots - 1)] * nranks, [size * (1 % slots)] * nranks
             what = f"dtype={dtype} N={nranks} len={length} offsets={variant}"
             ins = [rand_array(dtype, nranks * length, rng) for _ in range(nranks)]
             parts = [x[:length] for x in ins]

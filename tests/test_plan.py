@@ -329,22 +329,23 @@ def test_group_form_tile_mapping_covers_every_tile_once():
 
 
 def test_blocks_too_long_for_one_grid_are_cut_into_several_pack_launches():
-    """A grid holds 2^31 - 1 workgroups.  16 ranks' all_to_all is 256 block copies; with byte-misaligned buffers
-    (64 bytes per workgroup) a block beyond 512 MiB no longer fits one launch and is cut into slices, one launch
-    each, that cover every block exactly once.  Pointers are synthetic: describe() never dereferences them."""
+    """A grid holds 2^31 - 1 workgroups.  16 ranks' all_to_all is 256 block copies; a workgroup of the group form
+    takes 4 KiB of a block whatever the buffers' alignment, so a block beyond 32 GiB no longer fits one launch and
+    is cut into slices, one launch each, that cover every block exactly once.  Pointers are synthetic: describe()
+    never dereferences them."""
     nranks = 16
-    block = 600 * 2 ** 20 + 3  # bytes; odd, and the buffers sit at odd addresses: width 1
+    block = 40 * 2 ** 30 + 3  # bytes; odd, and the buffers sit at odd addresses: width 1
     sp = fake_ptrs(1 << 44, nranks, [1] * nranks, stride=1 << 40)
     rp = fake_ptrs(1 << 46, nranks, [1] * nranks, stride=1 << 40)
     runs, bytes_read, bytes_written = mr.describe(mr.Collective.ALL_TO_ALL, sp, rp, block, mr.DType.UINT8)
     assert bytes_read == bytes_written == nranks * nranks * block
     steps = sorted({r["step"] for r in runs})
-    assert len(steps) >= 2, "one launch cannot hold 256 x 600 MiB / 64 B workgroups"
+    assert len(steps) >= 2, "one launch cannot hold 256 x 40 GiB / 4 KiB workgroups"
     for step in steps:
         launch = [r for r in runs if r["step"] == step]
         assert len(launch) == nranks * nranks
-        assert sum(r["tiles"] for r in launch) <= 2 ** 31 - 1
-        assert all(r["vector"] == 1 for r in launch)
+        assert all(r["vector"] == 1 and r["waves"] == 4 for r in launch)
+        assert sum(-(-r["tiles"] // 4) for r in launch) <= 2 ** 31 - 1  # a workgroup of four wavefronts takes four tiles
     # per copy (source rank, source block): the slices tile [0, block) in order
     for src in range(nranks):
         for dst in range(nranks):
