@@ -264,7 +264,7 @@ struct SegmentView {
     uint64_t in_begin, out_begin, count;
     uint32_t local_tile, start, out_first;
     int dir;
-    bool vector;
+    bool vector, deal;
 };
 __device__ __forceinline__ SegmentView find_segment(const FoldLaunch& L, uint32_t tile) {
     uint32_t s = 0;
@@ -282,6 +282,7 @@ __device__ __forceinline__ SegmentView find_segment(const FoldLaunch& L, uint32_
     sv.dir = L.seg[s].dir;
     sv.out_first = L.seg[s].out_first;
     sv.vector = (L.seg[s].flags & kSegVector) != 0;
+    sv.deal = (L.seg[s].flags & kSegDeal) != 0;
     return sv;
 }
 
@@ -450,8 +451,22 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
     }
     const uint64_t nvec = sv.count / EPV;
     const uint64_t whole_groups = nvec / kThreads;  // groups of kThreads vectors that are complete
-    const uint64_t first =
-            uint64_t(sv.local_tile / kGroupStride) * (W * kGroupStride) + sv.local_tile % kGroupStride;
+    // Consecutive workgroups run on different XCDs, each with an L2 of its own.  Where the tiles do not sit on the
+    // cache lines of every buffer (inputs shifted against the outputs), neighbouring tiles share a line, so the
+    // workgroups of eight runs of kGroupStride (one run = 4 * kGroupStride consecutive tiles) are dealt out such
+    // that a whole run goes to one XCD and the shared lines are fetched into one L2 only (reduce_scatter of 8 x
+    // 32 MiB fp32 with an odd receive length: 74 -> 83 % of the HBM peak).  Tiles on line boundaries keep the
+    // plain order, which serves them 1 - 4 points better.
+    uint32_t local = sv.local_tile;
+    if (sv.deal) {
+        constexpr uint32_t kXcds = 8, kDeal = kXcds * kGroupStride;
+        const uint32_t wgs = uint32_t((nvec + kThreads - 1) / kThreads + W * kGroupStride - 1) / (W * kGroupStride) * kGroupStride;
+        if (local < wgs / kDeal * kDeal) {
+            const uint32_t w = local % kDeal;
+            local = local - w + (w % kXcds) * kGroupStride + w / kXcds;
+        }
+    }
+    const uint64_t first = uint64_t(local / kGroupStride) * (W * kGroupStride) + local % kGroupStride;
     const uint64_t mine = first + wave * kGroupStride;
     const bool have = mine < whole_groups;
     const uint64_t in_base = sv.in_begin * sizeof(T), out_base = sv.out_begin * sizeof(T);
@@ -939,9 +954,17 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
     const uint32_t tid = threadIdx.x % kThreads;
     // wavefront index, made known to be uniform so that it selects pointers in scalar registers
     const uint32_t wave = uint32_t(__builtin_amdgcn_readfirstlane(int(threadIdx.x / kThreads)));
-    const uint32_t first = (blockIdx.x / kGroupStride) * (W * kGroupStride) + blockIdx.x % kGroupStride;
+    uint32_t block = blockIdx.x;
+    if (L.exchange & 2u) {  // deal whole runs of kGroupStride workgroups to one XCD each
+        constexpr uint32_t kXcds = 8, kDeal = kXcds * kGroupStride;
+        if (block < gridDim.x / kDeal * kDeal) {
+            const uint32_t w = block % kDeal;
+            block = block - w + (w % kXcds) * kGroupStride + w / kXcds;
+        }
+    }
+    const uint32_t first = (block / kGroupStride) * (W * kGroupStride) + block % kGroupStride;
     const uint32_t mine = first + wave * kGroupStride;
-    const bool exchange = L.exchange != 0;
+    const bool exchange = (L.exchange & 1u) != 0;
 
     // tile k of the group is first + k * kGroupStride; it is loaded if it lies inside the buffers
     u32x4 x[K];

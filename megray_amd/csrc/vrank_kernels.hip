@@ -156,12 +156,22 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
     const uint32_t tid = threadIdx.x % kThreads;
     const uint32_t wave = uint32_t(__builtin_amdgcn_readfirstlane(int(threadIdx.x / kThreads)));
     const uint32_t copy = blockIdx.x / L.groups_per_copy;
-    const uint32_t group = blockIdx.x - copy * L.groups_per_copy;
-    const uint64_t first = L.first_tile + uint64_t(group / kGroupStride) * (W * kGroupStride) + group % kGroupStride;
+    uint32_t group = blockIdx.x - copy * L.groups_per_copy;
     const PackEnds e = pack_ends(L, copy);
     const char* src = static_cast<const char*>(L.in[e.src_rank]) + e.src_block * L.block_bytes;
     const uint64_t dst_off = e.dst_block * L.block_bytes;
     const PackVectors pv = pack_vectors(L, e, dst_off);
+    // The tiles sit on the destination's cache lines.  If the source lies differently, neighbouring tiles share
+    // source lines: consecutive workgroups run on different XCDs, each with an L2 of its own, so whole runs of
+    // kGroupStride workgroups (4 * kGroupStride consecutive tiles) are dealt to one XCD each.
+    if ((reinterpret_cast<uintptr_t>(src) - (reinterpret_cast<uintptr_t>(L.out[e.dst_rank]) + dst_off)) & 127u) {
+        constexpr uint32_t kXcds = 8, kDeal = kXcds * kGroupStride;
+        if (group < L.groups_per_copy / kDeal * kDeal) {
+            const uint32_t w = group % kDeal;
+            group = group - w + (w % kXcds) * kGroupStride + w / kXcds;
+        }
+    }
+    const uint64_t first = L.first_tile + uint64_t(group / kGroupStride) * (W * kGroupStride) + group % kGroupStride;
     if (first == 0 && wave == 0) pack_edges(L, e, pv, src, dst_off, tid);
 
     // tile t holds vectors [t * kThreads - pad, ...): whole if all of them exist

@@ -105,6 +105,13 @@ private:
         uint8_t out_first;
     };
 
+    // Do tiles that start on the buffers' common grid cover whole cache lines of every buffer, inputs and outputs
+    // (which lie `shift_bytes` before the inputs)?
+    bool lines_shared(uint64_t shift_bytes) const {
+        constexpr uint64_t kLine = 128;
+        return !m_plain && m_aligned && m_grid >= kLine && shift_bytes % kLine == 0;
+    }
+
     // The flat kernel folds exactly nranks inputs with the rank count known at compile time.
     static bool flat_width(uint32_t n) { return n == 2 || n == 3 || n == 4 || n == 8; }
 
@@ -149,6 +156,10 @@ private:
         for (const Run& r : m_runs) unshifted = unshifted && r.in_begin == r.out_begin;
         L.waves = total >= kFlatGroupMinTiles ? kGroupWaves : 1;
         L.exchange = (L.waves == kGroupWaves && !m_tree && m_nout == m_nranks && unshifted) ? 1 : 0;
+        // tiles that do not sit on the cache lines of every buffer share lines with their neighbours
+        bool on_lines = lines_shared(0) && m_misalign % 128 == 0;  // flat tiles start at the buffers' first byte
+        for (const Run& r : m_runs) on_lines = on_lines && lines_shared((r.in_begin - r.out_begin) * m_elem);
+        if (L.waves == kGroupWaves && !on_lines) L.exchange |= 2u;
         L.unshifted = unshifted ? 1 : 0;
         m_plan.steps.push_back(step);
         return true;
@@ -172,7 +183,13 @@ private:
             const bool vector = natural || same_phase(r);
             uint64_t head = 0, body = 0;
             if (m_plain) {
-                body = r.count / epv * epv;  // no grid to reach: every address is as aligned as it gets
+                // no grid that all buffers share: the body starts where the run's first output sits on a tile
+                // boundary, so that at least the stores of the other outputs miss whole cache lines by a few
+                // elements only instead of by the run's arbitrary offset
+                const uint64_t tile_bytes = uint64_t(kThreads) * kVecBytes;
+                const uint64_t at = (reinterpret_cast<uintptr_t>(m_out[r.out_first]) + r.out_begin * m_elem) & (tile_bytes - 1);
+                head = std::min<uint64_t>(((tile_bytes - at) & (tile_bytes - 1)) / m_elem, r.count);
+                body = (r.count - head) / epv * epv;
             } else if (same_phase(r)) {
                 // the body starts where inputs and outputs both sit on the coarsest grid they share
                 uint64_t grid = m_grid;
@@ -194,7 +211,10 @@ private:
             }
             const uint64_t tail = r.count - head - body;
             if (head) add_segment(r.in_begin, r.out_begin, head, r, 0);
-            add_segment(r.in_begin + head, r.out_begin + head, body, r, kSegVector);
+            // (a body that starts on the common grid sits on the lines of inputs and outputs alike unless the
+            // outputs are shifted by a part of a line)
+            const bool on_lines = lines_shared((r.in_begin - r.out_begin) * m_elem) && same_phase(r);
+            add_segment(r.in_begin + head, r.out_begin + head, body, r, kSegVector | (on_lines ? 0 : kSegDeal));
             if (tail) add_segment(r.in_begin + head + body, r.out_begin + head + body, tail, r, 0);
         }
         close_launch();

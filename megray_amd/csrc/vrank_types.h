@@ -16,6 +16,8 @@ constexpr uint32_t kVecBytes = 16;            // one 128-bit global load / store
 
 enum SegmentFlags : uint8_t {
     kSegVector = 1,  // tile is walked in 16-byte vectors; begin offsets are vector aligned
+    kSegDeal = 2,    // group form: the tiles do not sit on the cache lines of every buffer, so neighbouring tiles
+                     // share lines; whole runs of kGroupStride workgroups are dealt to one XCD (one L2) each
 };
 
 // A run of elements that all share one fold order and one set of destinations.
@@ -91,7 +93,8 @@ struct FlatLaunch {
     uint32_t elem_size;
     uint32_t tree;  // 1: combine in binomial-tree order towards rank `start` instead of a left fold
     uint32_t waves;     // wavefronts per workgroup: 1, or kGroupWaves for the group form (launches of many tiles)
-    uint32_t exchange;  // group form: 1 = every rank is an output at the inputs' offsets, results are exchanged too
+    uint32_t exchange;  // group form: bit 0 = every rank is an output at the inputs' offsets, results are exchanged too;
+                        // bit 1 = tiles share cache lines with their neighbours, deal runs of workgroups to XCDs
     uint32_t unshifted; // 1 = every run's outputs sit at the inputs' offsets (shift == 0 throughout)
     // run i covers elements [end[i - 1], end[i]) (from 0 for the first); unused entries are 0
     uint64_t end[kMaxFlatRuns];
