@@ -79,14 +79,14 @@ union VecOf {
     T v[kVecBytes / sizeof(T)];
 };
 
-// 128-bit accesses of single lanes.  The address needs 4-byte alignment only (buffers of 4- and
-// 8-byte elements at any element offset go 16 bytes per lane), which the pointer type says.
-typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+// 128-bit accesses of single lanes at any byte address (gfx950 serves them; the pointer type tells the compiler
+// not to assume more): buffers at any element offset go 16 bytes per lane.
+typedef uint32_t u32x4_a1 __attribute__((ext_vector_type(4), aligned(1)));
 __device__ __forceinline__ u32x4 load_vec(const char* p) {
-    return __builtin_nontemporal_load(reinterpret_cast<const u32x4_a4*>(p));
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4_a1*>(p));
 }
 __device__ __forceinline__ void store_vec(char* p, u32x4 x) {
-    __builtin_nontemporal_store(u32x4_a4(x), reinterpret_cast<u32x4_a4*>(p));
+    __builtin_nontemporal_store(u32x4_a1(x), reinterpret_cast<u32x4_a1*>(p));
 }
 
 // One tile (1 KiB) of a buffer through buffer instructions with explicit cache policies: measured
@@ -106,6 +106,18 @@ __device__ __forceinline__ void store_tile_vec(void* tile_base, uint32_t lane, u
     __amdgpu_buffer_rsrc_t rsrc =
             __builtin_amdgcn_make_buffer_rsrc(tile_base, 0, int(kThreads * kVecBytes), kRsrcFlags);
     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, x), rsrc, int(lane * kVecBytes), 0, kStorePolicy);
+}
+
+// The same for tiles that may start at any byte address (segments of 1- and 2-byte elements whose inputs are
+// shifted against the outputs, or whose buffers lie at differing offsets): buffer instructions need a 4-byte
+// boundary, so other tiles go lane by lane.  The test is uniform over the wavefront.
+__device__ __forceinline__ u32x4 load_tile_any(const char* tile_base, uint32_t lane) {
+    if ((reinterpret_cast<uintptr_t>(tile_base) & 3u) == 0) return load_tile_vec(tile_base, lane);
+    return load_vec(tile_base + lane * kVecBytes);
+}
+__device__ __forceinline__ void store_tile_any(char* tile_base, uint32_t lane, u32x4 x) {
+    if ((reinterpret_cast<uintptr_t>(tile_base) & 3u) == 0) store_tile_vec(tile_base, lane, x);
+    else store_vec(tile_base + lane * kVecBytes, x);
 }
 
 __device__ __forceinline__ uint32_t rotate_rank(uint32_t start, int dir, uint32_t j, uint32_t n) {
@@ -393,29 +405,29 @@ __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
                 u32x4 x[K];
 #pragma unroll
                 for (int j = 0; j < K; ++j)
-                    x[j] = load_tile_vec(static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off, tid);
+                    x[j] = load_tile_any(static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off, tid);
                 acc.seed(x[0]);
 #pragma unroll
                 for (int j = 1; j < K; ++j) acc.fold(x[j], new_wins);
             } else {
-                acc.seed(load_tile_vec(static_cast<const char*>(L.in[start]) + in_off, tid));
+                acc.seed(load_tile_any(static_cast<const char*>(L.in[start]) + in_off, tid));
                 uint32_t j = 1;
                 for (; j + 4 <= nfold; j += 4) {
                     u32x4 x[4];
 #pragma unroll
                     for (int q = 0; q < 4; ++q)
-                        x[q] = load_tile_vec(
+                        x[q] = load_tile_any(
                                 static_cast<const char*>(L.in[rotate_rank(start, dir, j + q, nr)]) + in_off, tid);
 #pragma unroll
                     for (int q = 0; q < 4; ++q) acc.fold(x[q], new_wins);
                 }
                 for (; j < nfold; ++j)
-                    acc.fold(load_tile_vec(static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off, tid),
+                    acc.fold(load_tile_any(static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off, tid),
                              new_wins);
             }
             const u32x4 res = acc.finish();
             for (uint32_t m = 0; m < nout; ++m)
-                store_tile_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, nr)]) + out_off, tid, res);
+                store_tile_any(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, nr)]) + out_off, tid, res);
         }
     } else {
         fold_element_tile<T, OP>(L, sv, nfold, local_tile, tid);
@@ -474,7 +486,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
     AccFor<T, OP> acc;
     if constexpr (K == 1) {
         // a copy: nothing to skew on the load side
-        if (have) acc.seed(load_tile_vec(static_cast<const char*>(L.in[sv.start]) + in_base + mine * kGroupBytes, tid));
+        if (have) acc.seed(load_tile_any(static_cast<const char*>(L.in[sv.start]) + in_base + mine * kGroupBytes, tid));
     } else {
         for (uint32_t j0 = 0; j0 < nfold; j0 += SK) {
             u32x4 x[SK];
@@ -482,7 +494,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
             for (uint32_t q = 0; q < SK; ++q) {
                 const uint64_t group = first + ((wave + q) % W) * kGroupStride;
                 if (j0 + q < nfold && group < whole_groups)
-                    x[q] = load_tile_vec(static_cast<const char*>(L.in[rotate_rank(sv.start, sv.dir, j0 + q, nr)]) +
+                    x[q] = load_tile_any(static_cast<const char*>(L.in[rotate_rank(sv.start, sv.dir, j0 + q, nr)]) +
                                                  in_base + group * kGroupBytes,
                                          tid);
                 else
@@ -510,7 +522,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
 
     if (nout == 1) {
         if (have)
-            store_tile_vec(static_cast<char*>(L.out[sv.out_first]) + out_base + mine * kGroupBytes, tid, acc.finish());
+            store_tile_any(static_cast<char*>(L.out[sv.out_first]) + out_base + mine * kGroupBytes, tid, acc.finish());
         return;
     }
     if (have) result[wave][tid] = acc.finish();
@@ -519,7 +531,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
     for (uint32_t m = 0; m < nout; ++m) {
         const uint32_t k = (wave + m) % W;
         if (folded[k])
-            store_tile_vec(static_cast<char*>(L.out[rotate_rank(sv.out_first, 1, m, nr)]) + out_base +
+            store_tile_any(static_cast<char*>(L.out[rotate_rank(sv.out_first, 1, m, nr)]) + out_base +
                                    (first + uint64_t(k) * kGroupStride) * kGroupBytes,
                            tid, result[k][tid]);
     }

@@ -37,14 +37,7 @@ __device__ __forceinline__ void store_w(char* p, W x) {
     __builtin_nontemporal_store(x, reinterpret_cast<W*>(p));
 }
 
-// 128-bit accesses of single lanes at any byte address.
-typedef uint32_t u32x4_a1 __attribute__((ext_vector_type(4), aligned(1)));
-__device__ __forceinline__ u32x4 load_vec_bytes(const char* p) {
-    return __builtin_nontemporal_load(reinterpret_cast<const u32x4_a1*>(p));
-}
-__device__ __forceinline__ void store_vec_bytes(char* p, u32x4 x) {
-    __builtin_nontemporal_store(u32x4_a1(x), reinterpret_cast<u32x4_a1*>(p));
-}
+// (load_vec / store_vec: 128-bit accesses of single lanes at any byte address)
 __device__ __forceinline__ bool on_words(const void* p) {
     return (reinterpret_cast<uintptr_t>(p) & 3u) == 0;
 }
@@ -101,16 +94,6 @@ __device__ __forceinline__ void pack_edges(const PackLaunch& L, const PackEnds& 
     else pack_edge_units<uint8_t>(L, e, pv, src, dst_off, tid);
 }
 
-// One whole tile to destination `m`: a buffer store where the address allows it (4-byte boundary; destination 0 is
-// on a 16-byte boundary by construction, the others usually share its offset), else lane by lane.
-__device__ __forceinline__ void pack_store_tile(char* dst, uint32_t tid, u32x4 x) {
-    if (on_words(dst)) store_tile_vec(dst, tid, x);
-    else store_vec_bytes(dst + tid * kVecBytes, x);
-}
-__device__ __forceinline__ u32x4 pack_load_tile(const char* src, uint32_t tid) {
-    return on_words(src) ? load_tile_vec(src, tid) : load_vec_bytes(src + tid * kVecBytes);
-}
-
 // Tile `tile` of a block copy, by one wavefront: whole tiles through buffer instructions, the partial ones at the
 // block's ends lane by lane.  `src` and `dst_off` address the block's first byte.
 __device__ __forceinline__ void pack_vector_tile(const PackLaunch& L, const PackEnds& e, const PackVectors& pv,
@@ -118,14 +101,14 @@ __device__ __forceinline__ void pack_vector_tile(const PackLaunch& L, const Pack
     const uint64_t t0 = tile * kThreads;  // this tile's lanes take vectors [t0 - pad, t0 - pad + kThreads)
     if (t0 >= pv.pad && t0 - pv.pad + kThreads <= pv.nvec) {
         const uint64_t off = pv.head + (t0 - pv.pad) * kVecBytes;
-        const u32x4 x = pack_load_tile(src + off, tid);
+        const u32x4 x = load_tile_any(src + off, tid);
         for (uint32_t m = 0; m < e.ndst; ++m)
-            pack_store_tile(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + off, tid, x);
+            store_tile_any(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + off, tid, x);
     } else if (t0 + tid >= pv.pad && t0 + tid - pv.pad < pv.nvec) {
         const uint64_t off = pv.head + (t0 + tid - pv.pad) * kVecBytes;
-        const u32x4 x = load_vec_bytes(src + off);
+        const u32x4 x = load_vec(src + off);
         for (uint32_t m = 0; m < e.ndst; ++m)
-            store_vec_bytes(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + off, x);
+            store_vec(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + off, x);
     }
 }
 
@@ -181,11 +164,11 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
     const bool whole = whole_tile(mine);
     u32x4 x = {0u, 0u, 0u, 0u};
     if (whole)
-        x = pack_load_tile(src + tile_off(mine), tid);
+        x = load_tile_any(src + tile_off(mine), tid);
     else
         pack_vector_tile(L, e, pv, src, dst_off, mine, tid);  // a partial tile at either end: copied to every destination here
     if (e.ndst == 1) {
-        if (whole) pack_store_tile(static_cast<char*>(L.out[e.dst_rank]) + dst_off + tile_off(mine), tid, x);
+        if (whole) store_tile_any(static_cast<char*>(L.out[e.dst_rank]) + dst_off + tile_off(mine), tid, x);
         return;
     }
     stage[wave][tid] = x;
@@ -194,7 +177,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
     for (uint32_t m = 0; m < e.ndst; ++m) {
         const uint32_t k = (wave + m) % W;
         if (staged[k])
-            pack_store_tile(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + tile_off(first + uint64_t(k) * kGroupStride),
+            store_tile_any(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + tile_off(first + uint64_t(k) * kGroupStride),
                             tid, stage[k][tid]);
     }
 }

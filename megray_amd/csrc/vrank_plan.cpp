@@ -66,11 +66,15 @@ public:
         // Buffers whose offsets from a 16-byte boundary differ: the 128-bit accesses of gfx950 need
         // 4-byte alignment only, so element types of 4 and 8 bytes (in naturally aligned buffers)
         // still go 16 bytes per lane, every buffer at its own alignment.  Narrower types do not.
-        if (!m_aligned && elem_size >= 4) {
-            m_plain = true;
+        // 1- and 2-byte elements go 16 bytes per lane as well (m_bytes), through the segment kernels only, whose
+        // tiles may start at any byte address.
+        if (!m_aligned) {
+            bool natural = true;
             for (uint32_t r = 0; r < kMaxRanks; ++r)
                 for (const void* p : {m_in[r], static_cast<const void*>(m_out[r])})
-                    if (p && reinterpret_cast<uintptr_t>(p) % elem_size) m_plain = false;
+                    if (p && reinterpret_cast<uintptr_t>(p) % elem_size) natural = false;
+            m_plain = natural && elem_size >= 4;
+            m_bytes = natural && elem_size < 4;
         }
     }
 
@@ -109,7 +113,7 @@ private:
     // (which lie `shift_bytes` before the inputs)?
     bool lines_shared(uint64_t shift_bytes) const {
         constexpr uint64_t kLine = 128;
-        return !m_plain && m_aligned && m_grid >= kLine && shift_bytes % kLine == 0;
+        return m_aligned && m_grid >= kLine && shift_bytes % kLine == 0;
     }
 
     // The flat kernel folds exactly nranks inputs with the rank count known at compile time.
@@ -168,11 +172,11 @@ private:
     void emit_general() {
         const uint64_t epv = kVecBytes / m_elem;
         // long vector bodies take the group form (four wavefronts per workgroup)
-        // Element types of 4 and 8 bytes go 16 bytes per lane whatever the offsets (4-byte alignment suffices for
-        // the 128-bit accesses of gfx950): buffers whose offsets from a 16-byte boundary differ (m_plain), and runs
-        // whose outputs are shifted against their inputs by a part of a vector (reduce_scatter with a receive
-        // length that is no multiple of 16 bytes, the copies of the two-phase and ring schedules).
-        const bool natural = m_plain || (m_aligned && m_elem >= 4);
+        // Elements go 16 bytes per lane whatever the offsets (gfx950 serves 128-bit accesses at any byte address):
+        // buffers whose offsets from a 16-byte boundary differ (m_plain, m_bytes), and runs whose outputs are
+        // shifted against their inputs by a part of a vector (reduce_scatter with a receive length that is no
+        // multiple of 16 bytes, the copies of the two-phase and ring schedules).
+        const bool natural = m_plain || m_bytes || m_aligned;
         auto same_phase = [&](const Run& r) { return m_aligned && r.in_begin % epv == r.out_begin % epv; };
         uint64_t vector_elems = 0;
         for (const Run& r : m_runs)
@@ -182,7 +186,7 @@ private:
         for (const Run& r : m_runs) {
             const bool vector = natural || same_phase(r);
             uint64_t head = 0, body = 0;
-            if (m_plain) {
+            if (m_plain || m_bytes) {
                 // no grid that all buffers share: the body starts where the run's first output sits on a tile
                 // boundary, so that at least the stores of the other outputs miss whole cache lines by a few
                 // elements only instead of by the run's arbitrary offset
@@ -279,6 +283,7 @@ private:
     bool m_new_wins;
     bool m_aligned;
     bool m_plain = false;  // 16-byte accesses on buffers that are only element-aligned (4- and 8-byte types)
+    bool m_bytes = false;  // the same for 1- and 2-byte types: tiles start at any byte address
     uint32_t m_misalign = 0;
     uint64_t m_grid = kVecBytes;
     bool m_tree = false;

@@ -125,7 +125,7 @@ def test_the_vector_forms_are_what_runs():
     assert all(r["waves"] == 4 for r in runs)
 
 
-@pytest.mark.parametrize("dtype", [orc.FLOAT32, orc.INT32, orc.FLOAT64, orc.INT64])
+@pytest.mark.parametrize("dtype", [orc.FLOAT32, orc.INT32, orc.FLOAT64, orc.INT64, orc.FLOAT16, orc.INT8, orc.UINT8])
 def test_reduce_scatter_with_receive_lengths_off_the_vector_grid(dtype):
     rng = np.random.default_rng(800 + dtype)
     size = orc.dtype_size(dtype)
@@ -141,7 +141,7 @@ def test_reduce_scatter_with_receive_lengths_off_the_vector_grid(dtype):
                     torch.cuda.synchronize()
                     for r in range(nranks):
                         outs[r].check(want[r], f"reduce_scatter dtype={dtype} N={nranks} recvlen={recvlen} op={op} order={order}")
-            if dtype in (orc.FLOAT32, orc.FLOAT64):
+            if dtype in (orc.FLOAT32, orc.FLOAT64, orc.INT8):
                 want = orc.ucx_reduce_scatter(ins, dtype, orc.SUM)  # the literal replay
                 d_in = [device_in(x, 0) for x in ins]
                 outs = [Guarded(recvlen * size, 0) for _ in range(nranks)]
@@ -149,3 +149,26 @@ def test_reduce_scatter_with_receive_lengths_off_the_vector_grid(dtype):
                 torch.cuda.synchronize()
                 for r in range(nranks):
                     outs[r].check(want[r], "reduce_scatter vs literal replay")
+
+
+@pytest.mark.parametrize("dtype", [orc.FLOAT16, orc.INT8, orc.UINT8, orc.FLOAT32, orc.INT64])
+def test_all_reduce_with_every_buffer_at_its_own_element_offset(dtype):
+    """Inputs and outputs at differing offsets from a 16-byte boundary, in whole elements: 16 bytes per lane all the
+    same, short (one wavefront per tile) and long (group form), for rank counts with and without a kernel of
+    their own."""
+    rng = np.random.default_rng(900 + dtype)
+    size = orc.dtype_size(dtype)
+    slots = 16 // size
+    for nranks in (2, 5, 8):
+        for length in (7, 1027, (700 * 1024) // size + 5):
+            ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+            in_off = [size * ((5 * r + 1) % slots) for r in range(nranks)]
+            out_off = [size * ((3 * r + 2) % slots) for r in range(nranks)]
+            for op, order in ((orc.SUM, orc.ORDER_UCX), (orc.MAX, orc.ORDER_SHM), (orc.MIN, orc.ORDER_RANK0)):
+                want = orc.fold_all_reduce(ins, dtype, op, order)
+                d_in = [device_in(x, in_off[r]) for r, x in enumerate(ins)]
+                outs = [Guarded(length * size, out_off[r]) for r in range(nranks)]
+                mr.all_reduce(d_in, [o.view for o in outs], length, dtype, op, order)
+                torch.cuda.synchronize()
+                for r in range(nranks):
+                    outs[r].check(want[r], f"all_reduce dtype={dtype} N={nranks} len={length} op={op} order={order}")

@@ -68,22 +68,24 @@ def execute(runs, sends, recvs, nranks, op, elem_size, send_ptrs, recv_ptrs):
                 if run["vector"]:
                     epv = 16 // elem_size
                     base_in = recv_ptrs if run["reads_recv"] else send_ptrs
-                    # 16-byte accesses sit on 16-byte boundaries, except that 4- and 8-byte elements are taken as
-                    # they lie (4-byte alignment suffices): buffers whose offsets from such a boundary differ, and
-                    # inputs that are shifted against the outputs by a part of a vector (the outputs, i.e. the
-                    # stores, then still sit on 16-byte boundaries)
+                    # 16-byte accesses sit on 16-byte boundaries, except that elements are taken as they lie (gfx950
+                    # serves 128-bit accesses at any byte address): buffers whose offsets from such a boundary
+                    # differ, and inputs that are shifted against the outputs by a part of a vector (the outputs,
+                    # i.e. the stores, then still sit on 16-byte boundaries).  The flat kernels use buffer
+                    # instructions throughout, which need 4-byte boundaries.
                     touched = [p for p in list(send_ptrs) + list(recv_ptrs) if p]
-                    need_out = 16 if len({p % 16 for p in touched}) == 1 else 4
+                    need_out = 16 if len({p % 16 for p in touched}) == 1 else elem_size
                     need_in = need_out
                     if run["vector"] == 1:
                         assert cnt % epv == 0
                         if (lo - run["out_begin"]) % epv:
-                            need_in = 4
-                    elif need_out == 16:  # flat launch: bases aligned, outputs shifted by whole vectors
-                        assert (lo - run["out_begin"]) % epv == 0
-                        lo = 0
-                        run = dict(run, out_begin=0)
-                    assert min(need_in, need_out) == 16 or elem_size >= 4
+                            need_in = elem_size
+                    else:
+                        assert need_out == 16 or elem_size >= 4
+                        if need_out == 16:  # flat launch: bases aligned, outputs shifted by whole vectors
+                            assert (lo - run["out_begin"]) % epv == 0
+                            lo = 0
+                            run = dict(run, out_begin=0)
                     for r in ranks:
                         assert (base_in[r] + lo * elem_size) % need_in == 0
                     for m in range(run["nout"]):
