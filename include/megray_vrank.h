@@ -159,7 +159,8 @@ typedef struct mrv_plan_run {
     uint32_t nout;          /* destinations: ranks out_first .. out_first + nout - 1 (mod nranks) */
     uint32_t new_wins_ties; /* fold */
     uint32_t vector;        /* fold: 0 = element by element, 1 = 16-byte vectors, 2 = run of a flat launch
-                               (vectors on the buffer's own 1 KiB tile grid); pack: bytes per lane access */
+                               (vectors on the buffer's own 1 KiB tile grid); pack: what every block address and the
+                               block size are a multiple of (16, 8, 4, 2 or 1; lanes move 16 bytes whichever it is) */
     uint32_t start;         /* fold: seed rank; pack: source rank */
     int32_t dir;            /* fold: +1 / -1; 0 = binomial tree towards rank `start` */
     uint32_t out_first;     /* fold: first destination rank; pack: destination rank */
@@ -169,6 +170,9 @@ typedef struct mrv_plan_run {
     uint64_t in_begin;      /* fold: first element in the inputs; pack: source byte offset */
     uint64_t out_begin;     /* fold: first element in the outputs; pack: destination byte offset */
     uint64_t count;         /* fold: elements; pack: bytes */
+    uint32_t deal;          /* fold, group form: 1 = the run's tiles share cache lines with their neighbours, so runs of
+                               workgroups are dealt to one XCD (one L2) each; pack decides this per copy on the device */
+    uint32_t reserved;
 } mrv_plan_run;
 
 /*

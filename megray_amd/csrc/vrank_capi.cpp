@@ -333,6 +333,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.new_wins_ties = L.new_wins_ties;
                     run.vector = (sg.flags & kSegVector) ? 1 : 0;
                     run.waves = L.waves;
+                    run.deal = (L.waves == kGroupWaves && (sg.flags & kSegDeal)) ? 1 : 0;
                     run.start = sg.start;
                     run.dir = sg.dir;
                     run.out_first = sg.out_first;
@@ -362,6 +363,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.new_wins_ties = L.new_wins_ties;
                     run.vector = 2;
                     run.waves = L.waves;
+                    run.deal = (L.exchange & 2u) ? 1 : 0;
                     run.start = start;
                     run.dir = L.tree ? 0 : int(int8_t((L.meta[s] >> 8) & 0xffu));
                     run.out_first = out_first;

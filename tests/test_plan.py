@@ -367,3 +367,44 @@ def test_blocks_too_long_for_one_grid_are_cut_into_several_pack_launches():
     first = sorted((r for r in runs if r["start"] == 0 and r["out_first"] == 0), key=lambda r: r["in_begin"])
     assert sum(r["count"] for r in first) == block
     assert all(r["in_begin"] % (128 * 1024) == 0 for r in first)
+
+
+def test_runs_whose_tiles_share_cache_lines_are_dealt_to_xcds():
+    """Consecutive workgroups run on different XCDs, each with an L2 of its own.  Where tiles do not sit on the
+    cache lines of every buffer, a line is shared by two tiles, and the planner asks the group kernels to deal runs
+    of workgroups to one XCD each; tiles on line boundaries keep the plain order."""
+    nranks = 8
+    send = fake_ptrs(1 << 44, nranks, [0] * nranks, stride=1 << 40)
+    recv = fake_ptrs(1 << 46, nranks, [0] * nranks, stride=1 << 40)
+    big = 1 << 24
+
+    def vector_runs(*args, **kw):
+        runs, _, _ = mr.describe(*args, **kw)
+        return [r for r in runs if r["vector"] and r["waves"] == 4]
+
+    # everything on 256-byte boundaries: plain order, flat and segment kernels
+    runs = vector_runs(mr.Collective.ALL_REDUCE, send, recv, big, mr.DType.FLOAT32)
+    assert runs and all(r["deal"] == 0 for r in runs)
+    runs = vector_runs(mr.Collective.REDUCE_SCATTER, send, recv, big // nranks, mr.DType.FLOAT32)
+    assert runs and all(r["deal"] == 0 for r in runs)
+    five_s, five_r = send[:5], recv[:5]
+    runs = vector_runs(mr.Collective.ALL_REDUCE, five_s, five_r, 5 * (1 << 20), mr.DType.FLOAT32)
+    assert runs and all(r["vector"] == 1 and r["deal"] == 0 for r in runs)
+    # a receive length off the line grid shifts the outputs against the inputs
+    for dtype, recvlen in ((mr.DType.FLOAT32, big // nranks - 1), (mr.DType.FLOAT16, big // nranks - 3),
+                           (mr.DType.FLOAT32, big // nranks - 4)):
+        runs = vector_runs(mr.Collective.REDUCE_SCATTER, send, recv, recvlen, dtype)
+        dealt = [r for r in runs if r["out_first"] != 0]  # rank 0's block starts where its output does
+        assert dealt and all(r["deal"] == 1 for r in dealt)
+    # every input at its own offset: flat launch (4-byte elements) or segments (2-byte elements), dealt
+    offs = [4 * (r % 3) for r in range(nranks)]
+    runs = vector_runs(mr.Collective.ALL_REDUCE, fake_ptrs(1 << 44, nranks, offs, stride=1 << 40), recv, big, mr.DType.FLOAT32)
+    assert runs and all(r["vector"] == 2 and r["deal"] == 1 for r in runs)
+    offs = [2 * (r % 5) for r in range(nranks)]
+    runs = vector_runs(mr.Collective.ALL_REDUCE, fake_ptrs(1 << 44, nranks, offs, stride=1 << 40), recv, big, mr.DType.FLOAT16)
+    assert runs and all(r["vector"] == 1 and r["deal"] == 1 for r in runs)
+    # a common offset of 16 bytes: flat tiles start at the buffers' first byte, off the lines
+    offs = [16] * nranks
+    runs = vector_runs(mr.Collective.ALL_REDUCE, fake_ptrs(1 << 44, nranks, offs, stride=1 << 40),
+                       fake_ptrs(1 << 46, nranks, offs, stride=1 << 40), big, mr.DType.FLOAT32)
+    assert runs and all(r["deal"] == 1 for r in runs)
