@@ -613,22 +613,26 @@ __device__ __forceinline__ T tree_element(const Launch& L, uint32_t n, uint32_t 
 // first: the subtree of SPAN virtual ranks from v0 (v0 < count) is its left half combined with its
 // right half, if there is one.  That is the expression the rounds of the element-wise form build,
 // with at most log2(kMaxRanks) + 1 accumulators alive at a time.
-template <typename T, int OP, uint32_t SPAN>
-__device__ __forceinline__ TreeAccFor<T, OP> tree_node(const TreeLaunch& L, uint64_t off, uint32_t v0) {
+// TILE: `off` is the byte offset of a whole tile, loaded with one buffer instruction per rank (lane `tid`
+// takes its vector of it); otherwise `off` is the lane's own vector.
+template <typename T, int OP, uint32_t SPAN, bool TILE>
+__device__ __forceinline__ TreeAccFor<T, OP> tree_node(const TreeLaunch& L, uint64_t off, uint32_t v0, uint32_t tid) {
     if constexpr (SPAN == 1) {
         TreeAccFor<T, OP> a;
-        a.seed(load_vec(static_cast<const char*>(L.in[rotate_rank(L.root, 1, v0, L.nranks)]) + off));
+        const char* base = static_cast<const char*>(L.in[rotate_rank(L.root, 1, v0, L.nranks)]) + off;
+        if constexpr (TILE) a.seed(load_tile_any(base, tid));
+        else a.seed(load_vec(base));
         return a;
     } else {
-        TreeAccFor<T, OP> left = tree_node<T, OP, SPAN / 2>(L, off, v0);
-        if (v0 + SPAN / 2 < L.nranks) left.merge(tree_node<T, OP, SPAN / 2>(L, off, v0 + SPAN / 2));
+        TreeAccFor<T, OP> left = tree_node<T, OP, SPAN / 2, TILE>(L, off, v0, tid);
+        if (v0 + SPAN / 2 < L.nranks) left.merge(tree_node<T, OP, SPAN / 2, TILE>(L, off, v0 + SPAN / 2, tid));
         return left;
     }
 }
 
 template <typename T, int OP>
 __device__ __forceinline__ u32x4 tree_vector(const TreeLaunch& L, uint64_t off) {
-    return tree_node<T, OP, kMaxRanks>(L, off, 0).finish();
+    return tree_node<T, OP, kMaxRanks, false>(L, off, 0, 0).finish();
 }
 
 template <typename T, int OP>
@@ -640,7 +644,14 @@ __global__ void __launch_bounds__(kThreads) fold_tree_kernel(const TreeLaunch L)
         return;
     }
     const uint64_t nvec = L.count / EPV;
-    if (lane < nvec) store_vec(static_cast<char*>(L.out) + lane * kVecBytes, tree_vector<T, OP>(L, lane * kVecBytes));
+    const uint64_t tile_off = uint64_t(blockIdx.x) * kThreads * kVecBytes;
+    if ((uint64_t(blockIdx.x) + 1) * kThreads <= nvec) {
+        // a whole tile: buffer instructions with the streaming cache policies
+        const u32x4 r = tree_node<T, OP, kMaxRanks, true>(L, tile_off, 0, threadIdx.x).finish();
+        store_tile_any(static_cast<char*>(L.out) + tile_off, threadIdx.x, r);
+    } else if (lane < nvec) {
+        store_vec(static_cast<char*>(L.out) + lane * kVecBytes, tree_vector<T, OP>(L, lane * kVecBytes));
+    }
     // the elements behind the last whole vector: the first lanes of the last workgroup
     if (blockIdx.x == gridDim.x - 1 && threadIdx.x < L.count % EPV) {
         const uint64_t el = nvec * EPV + threadIdx.x;

@@ -728,11 +728,10 @@ Status plan_reduce(Plan& plan, const void* const* send, void* recv_root, uint32_
         L.nranks = nranks;
         L.root = root;
         L.elem_size = elem_size;
-        // 16 bytes per lane where every address allows it: 16-byte aligned buffers, or element types of
-        // 4 and 8 bytes (whose 128-bit accesses need 4-byte alignment only)
+        // 16 bytes per lane wherever the buffers hold whole elements (128-bit accesses work at any byte address)
         uintptr_t bits = reinterpret_cast<uintptr_t>(recv_root);
         for (uint32_t r = 0; r < nranks; ++r) bits |= reinterpret_cast<uintptr_t>(send[r]);
-        L.vector = ((bits & (kVecBytes - 1)) == 0 || (elem_size >= 4 && (bits & (elem_size - 1)) == 0)) ? 1 : 0;
+        L.vector = (bits & (elem_size - 1)) == 0 ? 1 : 0;
         const uint64_t lanes = L.vector ? std::max<uint64_t>(len / (kVecBytes / elem_size), 1) : len;
         const uint64_t tiles = (lanes + kThreads - 1) / kThreads;
         if (tiles > 0x7fffffffull) return invalid("buffer too large for one tree launch");

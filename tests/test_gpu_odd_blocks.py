@@ -172,3 +172,42 @@ def test_all_reduce_with_every_buffer_at_its_own_element_offset(dtype):
                 torch.cuda.synchronize()
                 for r in range(nranks):
                     outs[r].check(want[r], f"all_reduce dtype={dtype} N={nranks} len={length} op={op} order={order}")
+
+
+def tree_expectation(ins, dtype, op, root):
+    """The oracle's literal replay of the binomial tree towards `root`; FLOAT16 (which the reference cannot reduce)
+    as the same tree in fp32 with one rounding at the end."""
+    nranks = len(ins)
+    if dtype != orc.FLOAT16:
+        return orc.ucx_reduce(ins, dtype, op, root)[root]
+    a = [ins[(root + v) % nranks].astype(np.float32) for v in range(nranks)]
+    bit = 1
+    while bit < nranks:
+        for v in range(0, nranks - bit, 2 * bit):
+            x, y = a[v], a[v + bit]
+            with np.errstate(over="ignore"):
+                a[v] = x + y if op == orc.SUM else np.where(y > x, y, x)
+        bit *= 2
+    with np.errstate(over="ignore"):
+        return a[0].astype(np.float16)
+
+
+@pytest.mark.parametrize("dtype", [orc.FLOAT16, orc.INT8, orc.FLOAT32, orc.INT64])
+def test_reduce_to_root_with_every_buffer_at_its_own_element_offset(dtype):
+    """The rooted reduce in the reference's binomial-tree order, for rank counts with (8) and without (5, 7, 16) a
+    kernel of their own, on buffers at differing element offsets: 16 bytes per lane all the same."""
+    rng = np.random.default_rng(950 + dtype)
+    size = orc.dtype_size(dtype)
+    slots = 16 // size
+    for nranks in (5, 7, 8, 16):
+        for length in (3, 1027, (300 * 1024) // size + 7):
+            ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+            in_off = [size * ((5 * r + 1) % slots) for r in range(nranks)]
+            for op in (orc.SUM, orc.MAX):
+                for root in (0, nranks - 2):
+                    want = tree_expectation(ins, dtype, op, root)
+                    d_in = [device_in(x, in_off[r]) for r, x in enumerate(ins)]
+                    out = Guarded(length * size, size * (3 % slots))
+                    mr.reduce_to_root(d_in, out.view, length, dtype, op, root)
+                    torch.cuda.synchronize()
+                    out.check(want, f"reduce dtype={dtype} N={nranks} len={length} op={op} root={root}")
