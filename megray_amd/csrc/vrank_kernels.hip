@@ -37,11 +37,6 @@ __device__ __forceinline__ void store_w(char* p, W x) {
     __builtin_nontemporal_store(x, reinterpret_cast<W*>(p));
 }
 
-// (load_vec / store_vec: 128-bit accesses of single lanes at any byte address)
-__device__ __forceinline__ bool on_words(const void* p) {
-    return (reinterpret_cast<uintptr_t>(p) & 3u) == 0;
-}
-
 // Decodes copy `copy` of a pack launch into its endpoints.
 struct PackEnds {
     uint32_t src_rank, src_block, dst_rank, dst_block, ndst;
