@@ -76,6 +76,15 @@ struct CachedPlan {
     std::vector<KernelCall> calls;  // point into `plan`
 };
 
+// The same for the copy of a point-to-point transfer.
+struct CachedCopy {
+    const void* src;
+    void* dst;
+    size_t size;
+    Plan plan;
+    std::vector<KernelCall> calls;  // point into `plan`
+};
+
 uint64_t env_u64(const char* name, uint64_t fallback) {
     const char* text = std::getenv(name);
     if (!text || !*text) return fallback;
@@ -113,6 +122,7 @@ public:
             if (ev) (void)hipEventDestroy(ev);
         if (m_done) (void)hipEventDestroy(m_done);
         if (m_edges[0].words) (void)hipFree(m_edges[0].words);
+        if (m_p2p_words) (void)hipFree(m_p2p_words);
         if (m_edges[0].status) (void)hipHostFree(m_edges[0].status);
         give_back_static_slot(m_fixed_slot);
     }
@@ -182,7 +192,7 @@ public:
         theirs.pop_front();
         PendingP2P& s = op->is_send ? *op : *other;
         PendingP2P& r = op->is_send ? *other : *op;
-        Status st = transfer(s, r);
+        Status st = transfer(s, r, size_t(src_rank) * m_nranks + dst_rank);
         s.status = r.status = st;
         s.done = r.done = true;
         m_cv.notify_all();
@@ -423,7 +433,7 @@ private:
         EdgeSet& set = m_edges[lead.fixed];
         if (set.status && *set.status != set.status_seen) {
             set.status_seen = *set.status;
-            set_plan_error("a stream wait of an earlier collective gave up: a rank's stream did not get there in time");
+            set_plan_error("a stream wait of an earlier collective or transfer gave up: a rank's stream did not get there in time");
             return MEGRAY_UNEXPECTED_ERR;
         }
         const void* send[kMaxRanks] = {};
@@ -502,24 +512,89 @@ private:
         return MEGRAY_OK;
     }
 
+    // Counters for point-to-point transfers between ranks on different streams: two blocks per (source,
+    // destination) pair, "the sender's stream has reached the send" and "the copy is done", each holding
+    // the number of the pair's last transfer that got there.  Allocated at the first such transfer.
+    void prepare_p2p_edges() {
+        std::call_once(m_p2p_once, [&] {
+            prepare_edges();
+            if (!m_edges[0].words) return;  // events are in use (by choice, or the counters could not be allocated)
+            const size_t bytes = sizeof(EdgeWords) * 2 * m_mail.size();
+            EdgeWords* words = nullptr;
+            if (hipMalloc(reinterpret_cast<void**>(&words), bytes) != hipSuccess ||
+                hipMemset(words, 0, bytes) != hipSuccess) {
+                (void)hipGetLastError();
+                if (words) (void)hipFree(words);
+                return;
+            }
+            m_p2p_seq.assign(m_mail.size(), 0);
+            m_p2p_words = words;
+        });
+    }
+
+    // The copy itself: the library's own block copy (16 bytes per lane at any alignment), planned once per
+    // (source, destination, size) and kept for the next transfer between the same buffers; buffers the
+    // planner does not take (partly overlapping ones) go to the runtime's copy.  Called with m_mutex held.
+    Status copy_bytes(void* dst, const void* src, size_t size, hipStream_t stream) {
+        CachedCopy* cc = nullptr;
+        for (auto& c : m_copies)
+            if (c->src == src && c->dst == dst && c->size == size) cc = c.get();
+        if (!cc) {
+            auto fresh = std::make_unique<CachedCopy>();
+            fresh->src = src;
+            fresh->dst = dst;
+            fresh->size = size;
+            void* const recv[1] = {dst};
+            Status st = plan_broadcast(fresh->plan, src, recv, 1, size, 1, 0);
+            if (st == MEGRAY_OK) st = resolve(fresh->plan, MEGRAY_UINT8, MEGRAY_SUM, fresh->calls);
+            if (st != MEGRAY_OK) {
+                set_plan_error("");
+                HIP_CHECK(hipMemcpyAsync(dst, src, size, hipMemcpyDeviceToDevice, stream));
+                return MEGRAY_OK;
+            }
+            if (m_copies.size() < kPlanSlots) {
+                m_copies.push_back(std::move(fresh));
+                cc = m_copies.back().get();
+            } else {
+                m_copies[m_copy_next] = std::move(fresh);
+                cc = m_copies[m_copy_next].get();
+                m_copy_next = (m_copy_next + 1) % kPlanSlots;
+            }
+        }
+        for (const KernelCall& call : cc->calls) HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, stream));
+        return MEGRAY_OK;
+    }
+
     // Enqueue the copy of a matched send / receive pair: on the receiver's stream, after the
-    // sender's stream has reached the send, and before the sender's stream goes on.
-    Status transfer(const PendingP2P& s, const PendingP2P& r) {
+    // sender's stream has reached the send, and before the sender's stream goes on.  Between two
+    // streams the order is kept by notify / wait kernels on the pair's counters (every wait is
+    // enqueued after the kernel that satisfies it), or by events where the counters are not in use.
+    // Called with m_mutex held, so a pair's transfers are numbered in the order they are enqueued.
+    Status transfer(const PendingP2P& s, const PendingP2P& r, size_t pair) {
         if (s.size != r.size || s.device != r.device) {
             MEGRAY_ERROR("send of %zu bytes met a receive of %zu bytes", s.size, r.size);
             return MEGRAY_INVALID_USAGE;
         }
         if (!s.size) return MEGRAY_OK;
-        const size_t base = 0;
-        if (s.stream != r.stream) {
-            HIP_CHECK(hipEventRecord(event(base), s.stream));
-            HIP_CHECK(hipStreamWaitEvent(r.stream, event(base), 0));
+        if (s.stream == r.stream) return copy_bytes(r.dst, s.src, s.size, r.stream);
+        prepare_p2p_edges();
+        if (m_p2p_words) {
+            EdgeWords* reached = m_p2p_words + 2 * pair;
+            EdgeWords* copied = reached + 1;
+            const uint64_t ticket = ++m_p2p_seq[pair];
+            uint64_t* status = m_edges[0].status;
+            HIP_CHECK(edge_notify(reached, ticket, s.stream));
+            HIP_CHECK(edge_wait_done(reached, ticket, m_limit_ticks, status, r.stream));
+            MEGRAY_CHECK(copy_bytes(r.dst, s.src, s.size, r.stream));
+            HIP_CHECK(edge_notify(copied, ticket, r.stream));
+            HIP_CHECK(edge_wait_done(copied, ticket, m_limit_ticks, status, s.stream));
+            return MEGRAY_OK;
         }
-        HIP_CHECK(hipMemcpyAsync(r.dst, s.src, s.size, hipMemcpyDeviceToDevice, r.stream));
-        if (s.stream != r.stream) {
-            HIP_CHECK(hipEventRecord(event(base + 1), r.stream));
-            HIP_CHECK(hipStreamWaitEvent(s.stream, event(base + 1), 0));
-        }
+        HIP_CHECK(hipEventRecord(event(0), s.stream));
+        HIP_CHECK(hipStreamWaitEvent(r.stream, event(0), 0));
+        MEGRAY_CHECK(copy_bytes(r.dst, s.src, s.size, r.stream));
+        HIP_CHECK(hipEventRecord(event(1), r.stream));
+        HIP_CHECK(hipStreamWaitEvent(s.stream, event(1), 0));
         return MEGRAY_OK;
     }
 
@@ -560,10 +635,15 @@ private:
     [[maybe_unused]] alignas(64) char m_pad[64] = {};  // keeps what follows off the polled line
     std::vector<hipEvent_t> m_arrive;  // per rank: "my buffers are ready", recorded by the rank itself
     hipEvent_t m_done = nullptr;       // recorded by the leader behind the collective
-    std::vector<hipEvent_t> m_events;  // point-to-point transfers
+    std::vector<hipEvent_t> m_events;  // point-to-point transfers, where the counters below are not in use
+    std::once_flag m_p2p_once;
+    EdgeWords* m_p2p_words = nullptr;  // point-to-point transfers: two counter blocks per (source, destination)
+    std::vector<uint64_t> m_p2p_seq;   // per (source, destination): transfers enqueued between two streams so far
     std::vector<Mailbox> m_mail;
     std::vector<std::unique_ptr<CachedPlan>> m_plans;
     size_t m_plan_next = 0;
+    std::vector<std::unique_ptr<CachedCopy>> m_copies;  // point-to-point transfers
+    size_t m_copy_next = 0;
 };
 
 }  // namespace vrank

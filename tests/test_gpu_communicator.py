@@ -409,3 +409,42 @@ def test_back_to_back_rounds_with_fresh_data_on_rank_streams(length):
     for r in range(rounds):
         for rank in range(nranks):
             assert bits_equal(outs[r][rank], wants[r][rank]), f"round {r} rank {rank}"
+
+
+@pytest.mark.parametrize("nbytes", [13, 4096 + 3, 3 * 1024 * 1024 + 5])
+def test_ring_of_sends_back_to_back_on_rank_streams(nbytes):
+    """Four ranks, each on a stream of its own, pass blocks round a ring five times without a host synchronisation:
+    every round a rank copies fresh bytes into the SAME send buffer on its stream, sends it to the right neighbour
+    and receives from the left one inside group_start / group_end, and copies the SAME receive buffer out on its
+    stream.  A copy that started before the sender's copy-in had landed, a copy-in that overtook the previous
+    round's transfer, or a copy-out that overtook the transfer shows as a wrong round.  Buffers sit at odd byte
+    addresses; the lengths run the edge bytes only, the short copy kernel and the group copy kernel."""
+    nranks, rounds = 4, 5
+    rng = np.random.default_rng(nbytes)
+    data = [[rng.integers(0, 256, nbytes, dtype=np.uint8) for _ in range(nranks)] for _ in range(rounds)]
+    outs = [[None] * nranks for _ in range(rounds)]
+
+    def main(comm, rank, _inp, stream):
+        right, left = (rank + 1) % nranks, (rank - 1) % nranks
+        with torch.cuda.stream(stream):
+            staged = [torch.from_numpy(data[r][rank].copy()).pin_memory() for r in range(rounds)]
+            host_out = [torch.empty(nbytes, dtype=torch.uint8).pin_memory() for _ in range(rounds)]
+            src = torch.empty(nbytes + 64, dtype=torch.uint8, device="cuda:0")[1 + rank:1 + rank + nbytes]
+            dst = torch.full((nbytes + 64,), 0x5A, dtype=torch.uint8, device="cuda:0")[7 - rank:7 - rank + nbytes]
+            for r in range(rounds):
+                src.copy_(staged[r], non_blocking=True)
+                comm.group_start()
+                comm.send(src, nbytes, mr.DType.UINT8, right, stream)
+                comm.recv(dst, nbytes, mr.DType.UINT8, left, stream)
+                comm.group_end()
+                host_out[r].copy_(dst, non_blocking=True)
+            stream.synchronize()
+            for r in range(rounds):
+                outs[r][rank] = host_out[r].numpy().copy()
+        return None
+
+    for own_streams in (True, False):
+        run_test(nranks, [None] * nranks, [None] * nranks, main, own_streams=own_streams)
+        for r in range(rounds):
+            for rank in range(nranks):
+                assert bits_equal(outs[r][rank], data[r][(rank - 1) % nranks]), f"round {r} rank {rank}"
