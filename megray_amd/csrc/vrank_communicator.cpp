@@ -411,6 +411,35 @@ private:
         return nullptr;
     }
 
+    // Where a launch keeps its stream-ordering fields, if it is one that may carry them: one wavefront
+    // per workgroup and fewer than kHookMaxTiles workgroups.
+    struct HookFields {
+        EdgeHooks* hooks;
+        uint64_t* target;
+        uint64_t* ticket;
+    };
+    static bool hook_fields(Step& step, HookFields& f) {
+        switch (step.kind) {
+            case Step::kFlat:
+                if (step.flat.waves != 1 || step.flat.total_tiles >= kHookMaxTiles) return false;
+                f = {&step.flat.hooks, &step.flat.hook_target, &step.flat.hook_ticket};
+                return true;
+            case Step::kFold:
+                if (step.fold.waves != 1 || step.fold.total_tiles >= kHookMaxTiles) return false;
+                f = {&step.fold.hooks, &step.fold.hook_target, &step.fold.hook_ticket};
+                return true;
+            case Step::kTree:
+                if (step.tree.total_tiles >= kHookMaxTiles) return false;
+                f = {&step.tree.hooks, &step.tree.hook_target, &step.tree.hook_ticket};
+                return true;
+            case Step::kPack:
+                if (step.pack.waves != 1 || uint64_t(step.pack.ncopies) * step.pack.tiles_per_copy >= kHookMaxTiles) return false;
+                f = {&step.pack.hooks, &step.pack.hook_target, &step.pack.hook_ticket};
+                return true;
+        }
+        return false;
+    }
+
     // Called by the last rank to arrive; every other rank is parked or has withdrawn.
     Status launch(uint32_t leader) {
         {
@@ -481,26 +510,24 @@ private:
         m_shared_stream.store(static_cast<void*>(stream), std::memory_order_relaxed);
         m_shared_valid.store(one_stream, std::memory_order_release);
         const uint64_t ticket = m_generation.load(std::memory_order_relaxed) + 1;
-        // A short flat launch waits for the marks and publishes its completion itself: two launches
-        // less on this thread, on which every rank is waiting.
+        // A single short launch of one wavefront per workgroup waits for the marks and publishes its
+        // completion itself: two launches less on this thread, on which every rank is waiting.
         // (Only short launches: one of many tiles must not wait inside the kernel - workgroups that hold a
         // whole CU's LDS would spin on streams that may need that CU - and announcing completion costs
         // an L2 write-back per workgroup.  Those get a wait kernel before and a notify kernel after.)
-        FlatLaunch* hooked = nullptr;
-        if (set.words && !one_stream && cp->plan.steps.size() == 1 && cp->plan.steps[0].kind == Step::kFlat &&
-            cp->plan.steps[0].flat.waves == 1 && cp->plan.steps[0].flat.total_tiles < kHookMaxTiles)
-            hooked = &cp->plan.steps[0].flat;
-        if (hooked) {
-            hooked->hooks = EdgeHooks{reinterpret_cast<uint64_t*>(set.words), set.status, m_limit_ticks};
-            hooked->hook_target = wait_needed ? set.marks.load(std::memory_order_relaxed) : 0;
-            hooked->hook_ticket = ticket;
+        HookFields hooked;
+        const bool hook = set.words && !one_stream && cp->plan.steps.size() == 1 && hook_fields(cp->plan.steps[0], hooked);
+        if (hook) {
+            *hooked.hooks = EdgeHooks{reinterpret_cast<uint64_t*>(set.words), set.status, m_limit_ticks};
+            *hooked.target = wait_needed ? set.marks.load(std::memory_order_relaxed) : 0;
+            *hooked.ticket = ticket;
         } else if (wait_needed && set.words) {
             HIP_CHECK(edge_wait_arrived(set.words, set.marks.load(std::memory_order_relaxed), m_limit_ticks, set.status, stream));
         }
         for (const KernelCall& call : cp->calls) HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, stream));
         // the other ranks order their streams behind this point themselves (none has to if all share the stream)
-        if (hooked) {
-            hooked->hook_target = hooked->hook_ticket = 0;
+        if (hook) {
+            *hooked.target = *hooked.ticket = 0;
         } else if (!one_stream) {
             if (set.words) {
                 HIP_CHECK(edge_notify(set.words, ticket, stream));

@@ -371,11 +371,42 @@ __device__ __forceinline__ void fold_vector_remainder(const FoldLaunch& L, const
         store_vec(static_cast<char*>(L.out[rotate_rank(sv.out_first, 1, m, nr)]) + out_off, r);
 }
 
+// Every lane polls the same word (one request per wavefront) until it reaches `target` or the time
+// limit passes; each lane's acquire keeps its own loads behind the wait.
+__device__ __forceinline__ void hook_wait(const EdgeHooks& h, uint64_t target) {
+    const uint64_t begin = wall_clock64();
+    while (__hip_atomic_load(h.words, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < target) {
+        if (wall_clock64() - begin > h.limit_ticks) {
+            if (threadIdx.x == 0) {
+                __hip_atomic_fetch_add(h.words + 2, uint64_t(1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (h.status) __hip_atomic_fetch_add(h.status, uint64_t(1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+            return;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
+
+// After a one-wavefront workgroup's stores: count it, and let the last one publish the ticket.
+// (Only short launches do this: the release fence writes the L2 back, once per workgroup; from a few
+// hundred workgroups on that costs more than a separate notify kernel, and at 2560 workgroups it
+// alone took ten times as long as the fold.)
+__device__ __forceinline__ void hook_publish(const EdgeHooks& h, uint64_t ticket) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // this wavefront's stores before its count
+    if (threadIdx.x == 0) {
+        const uint64_t before = __hip_atomic_fetch_add(h.words + 3, uint64_t(1), __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        if (before + 1 == gridDim.x) {
+            __hip_atomic_store(h.words + 3, uint64_t(0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(h.words + 1, ticket, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
 // One wavefront per tile, for short launches.
 // K > 0: fold count known at compile time, all K loads of a lane are issued before the first use.
 // K == 0: fold count read from the launch, loads issued in groups of four.
 template <typename T, int OP, int K>
-__global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
+__device__ __forceinline__ void fold_tile(const FoldLaunch& L) {
     constexpr uint32_t EPV = kVecBytes / sizeof(T);
     const SegmentView sv = find_segment(L, blockIdx.x);
     const uint32_t local_tile = sv.local_tile, start = sv.start, out_first = sv.out_first;
@@ -432,6 +463,13 @@ __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
     } else {
         fold_element_tile<T, OP>(L, sv, nfold, local_tile, tid);
     }
+}
+
+template <typename T, int OP, int K>
+__global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
+    if (L.hook_target) hook_wait(L.hooks, L.hook_target);
+    fold_tile<T, OP, K>(L);
+    if (L.hook_ticket) hook_publish(L.hooks, L.hook_ticket);
 }
 
 // Group form of the segment fold for launches whose vector bodies are long (L.waves == kGroupWaves).
@@ -636,7 +674,7 @@ __device__ __forceinline__ u32x4 tree_vector(const TreeLaunch& L, uint64_t off) 
 }
 
 template <typename T, int OP>
-__global__ void __launch_bounds__(kThreads) fold_tree_kernel(const TreeLaunch L) {
+__device__ __forceinline__ void tree_tile(const TreeLaunch& L) {
     constexpr uint32_t EPV = kVecBytes / sizeof(T);
     const uint64_t lane = uint64_t(blockIdx.x) * kThreads + threadIdx.x;
     if (!L.vector) {
@@ -657,6 +695,13 @@ __global__ void __launch_bounds__(kThreads) fold_tree_kernel(const TreeLaunch L)
         const uint64_t el = nvec * EPV + threadIdx.x;
         static_cast<T*>(L.out)[el] = tree_element<T, OP, 0>(L, L.nranks, L.root, el);
     }
+}
+
+template <typename T, int OP>
+__global__ void __launch_bounds__(kThreads) fold_tree_kernel(const TreeLaunch L) {
+    if (L.hook_target) hook_wait(L.hooks, L.hook_target);
+    tree_tile<T, OP>(L);
+    if (L.hook_ticket) hook_publish(L.hooks, L.hook_ticket);
 }
 
 // The run tables of a flat launch are kernel arguments read through scalar loads.  Written naively
@@ -850,37 +895,6 @@ __device__ __forceinline__ void flat_tile_across_runs(const FlatLaunch& L, uint3
 #pragma unroll 1
             for (uint32_t m = 0; m < nout; ++m)
                 static_cast<T*>(L.out[rotate_rank(rout, 1, m, K)])[el - rshift] = r;
-        }
-    }
-}
-
-// Every lane polls the same word (one request per wavefront) until it reaches `target` or the time
-// limit passes; each lane's acquire keeps its own loads behind the wait.
-__device__ __forceinline__ void hook_wait(const EdgeHooks& h, uint64_t target) {
-    const uint64_t begin = wall_clock64();
-    while (__hip_atomic_load(h.words, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < target) {
-        if (wall_clock64() - begin > h.limit_ticks) {
-            if (threadIdx.x == 0) {
-                __hip_atomic_fetch_add(h.words + 2, uint64_t(1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (h.status) __hip_atomic_fetch_add(h.status, uint64_t(1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-            }
-            return;
-        }
-        __builtin_amdgcn_s_sleep(1);
-    }
-}
-
-// After a one-wavefront workgroup's stores: count it, and let the last one publish the ticket.
-// (Only short launches do this: the release fence writes the L2 back, once per workgroup; from a few
-// hundred workgroups on that costs more than a separate notify kernel, and at 2560 workgroups it
-// alone took ten times as long as the fold.)
-__device__ __forceinline__ void hook_publish(const EdgeHooks& h, uint64_t ticket) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // this wavefront's stores before its count
-    if (threadIdx.x == 0) {
-        const uint64_t before = __hip_atomic_fetch_add(h.words + 3, uint64_t(1), __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        if (before + 1 == gridDim.x) {
-            __hip_atomic_store(h.words + 3, uint64_t(0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(h.words + 1, ticket, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }

@@ -109,6 +109,7 @@ __device__ __forceinline__ void pack_vector_tile(const PackLaunch& L, const Pack
 
 // One wavefront per tile: short block copies.
 __global__ void __launch_bounds__(kThreads) pack_kernel(const PackLaunch L) {
+    if (L.hook_target) hook_wait(L.hooks, L.hook_target);
     const uint32_t copy = blockIdx.x / L.tiles_per_copy;
     const uint64_t tile = L.first_tile + (blockIdx.x - copy * L.tiles_per_copy);
     const PackEnds e = pack_ends(L, copy);
@@ -118,6 +119,7 @@ __global__ void __launch_bounds__(kThreads) pack_kernel(const PackLaunch L) {
     const PackVectors pv = pack_vectors(L, e, dst_off);
     pack_vector_tile(L, e, pv, src, dst_off, tile, tid);
     if (tile == 0) pack_edges(L, e, pv, src, dst_off, tid);
+    if (L.hook_ticket) hook_publish(L.hooks, L.hook_ticket);
 }
 
 // Group form of the pack kernel for long blocks: a workgroup of kGroupWaves

@@ -32,6 +32,18 @@ struct FoldSegment {
     uint8_t flags;
 };
 
+// Cross-stream ordering carried by a launch itself (thread-per-rank API, short launches of one wavefront
+// per workgroup): before it reads, every workgroup waits until `arrived` has reached the launch's
+// hook_target (the other ranks' streams have got to the collective); after its stores, the last workgroup
+// to finish publishes the launch's hook_ticket in `done`.  The four words are the group's counters in
+// device memory.  Every launch descriptor carries the three fields; 0 in hook_target / hook_ticket
+// (what the planner leaves there) means "do not wait" / "do not publish".
+struct EdgeHooks {
+    uint64_t* words;       // [0] arrived  [1] done  [2] timeouts  [3] workgroups finished
+    uint64_t* status;      // host-visible count of waits that gave up
+    uint64_t limit_ticks;  // a wait gives up after this many wall-clock ticks
+};
+
 // One launch of the fold kernel: every output element is a left fold, in a fixed order, over the
 // same element of `nfold` input buffers, written to `nout` output buffers.
 struct FoldLaunch {
@@ -47,16 +59,9 @@ struct FoldLaunch {
     uint32_t new_wins_ties;  // float MAX/MIN: an equal / unordered compare keeps the newcomer
     uint32_t elem_size;
     uint32_t waves;          // wavefronts per workgroup: 1, or 4 for the group form (long vector bodies)
-};
-
-// Cross-stream ordering carried by a launch itself (thread-per-rank API, short launches): before it
-// reads, every workgroup waits until `arrived` has reached FlatLaunch::hook_target (the other ranks'
-// streams have got to the collective); after its stores, the last workgroup to finish publishes
-// FlatLaunch::hook_ticket in `done`.  The four words are the group's counters in device memory.
-struct EdgeHooks {
-    uint64_t* words;       // [0] arrived  [1] done  [2] timeouts  [3] workgroups finished
-    uint64_t* status;      // host-visible count of waits that gave up
-    uint64_t limit_ticks;  // a wait gives up after this many wall-clock ticks
+    EdgeHooks hooks;         // one wavefront per workgroup only
+    uint64_t hook_target;
+    uint64_t hook_ticket;
 };
 
 constexpr uint32_t kMaxFlatRuns = 48;  // 2N chunks cut again at N-1 rank borders
@@ -112,7 +117,7 @@ constexpr uint32_t kGroupWaves = 4;
 constexpr uint32_t kGroupStride = 32;
 constexpr uint32_t kGroupMinTiles = 512;
 constexpr uint32_t kFlatGroupMinTiles = 2048;
-// Launches of the flat fold below this many tiles carry the thread-per-rank API's stream ordering
+// One-wavefront launches below this many workgroups carry the thread-per-rank API's stream ordering
 // themselves (EdgeHooks).  Beyond it the release fence every workgroup then executes costs more than
 // the two launches it saves.  Measured, 8 ranks, a stream per rank, microseconds per all_reduce with /
 // without: 16 - 128 tiles 16 - 18 / 22 - 23, 256 tiles 18 / 22.5, 384 tiles 21 - 34 / 22 - 23, 508 tiles
@@ -134,6 +139,9 @@ struct TreeLaunch {
     uint32_t total_tiles;  // kThreads lanes per tile
     uint32_t vector;       // 1: a lane takes a 16-byte vector (the last workgroup also the odd elements at the end);
                            // 0: a lane takes one element
+    EdgeHooks hooks;
+    uint64_t hook_target;
+    uint64_t hook_ticket;
 };
 
 enum PackMode : uint32_t {
@@ -160,6 +168,9 @@ struct PackLaunch {
     uint32_t groups_per_copy;  // group form: workgroups per block copy
     uint64_t first_tile;  // the launch covers tiles [first_tile, first_tile + tiles_per_copy) of every copy (blocks
                           // too long for one grid are cut into several launches; a multiple of the group span)
+    EdgeHooks hooks;      // one wavefront per workgroup only
+    uint64_t hook_target;
+    uint64_t hook_ticket;
 };
 
 // The pack kernels move 16 bytes per lane whatever the blocks' alignment.  Each copy lays its tiles out from the

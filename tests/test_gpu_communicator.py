@@ -448,3 +448,65 @@ def test_ring_of_sends_back_to_back_on_rank_streams(nbytes):
         for r in range(rounds):
             for rank in range(nranks):
                 assert bits_equal(outs[r][rank], data[r][(rank - 1) % nranks]), f"round {r} rank {rank}"
+
+
+@pytest.mark.parametrize("nranks,part", [(8, 3), (5, 1000 + 1), (8, 40 * 256), (3, 700 * 256 + 2)])
+def test_back_to_back_rounds_of_every_collective_on_rank_streams(nranks, part):
+    """Four rounds of reduce_scatter, all_gather, all_to_all, scatter, gather, broadcast and reduce, one after the
+    other on each rank's own stream with no host synchronisation: every round a rank copies fresh data into the SAME
+    send buffer on its stream before the first call and copies every result out of the SAME receive buffers on its
+    stream after the calls.  The short lengths run single launches of one wavefront per workgroup, which carry the
+    stream ordering themselves (copy, segment fold, tree and flat kernels alike); the long ones run between separate
+    wait and notify kernels."""
+    rounds, root = 4, nranks - 2
+    length = part * nranks
+    f32, npf = mr.DType.FLOAT32, np.float32
+    rng = np.random.default_rng(nranks * 1000003 + part)
+    data = [[rand_array(orc.FLOAT32, length, rng, wide=False) for _ in range(nranks)] for _ in range(rounds)]
+    names = ("reduce_scatter", "all_gather", "all_to_all", "scatter", "gather", "broadcast", "reduce")
+    sizes = {"reduce_scatter": part, "all_gather": length, "all_to_all": length, "scatter": part, "gather": length,
+             "broadcast": part, "reduce": part}
+    wants = []
+    for ins in data:
+        heads = [x[:part] for x in ins]
+        wants.append({
+            "reduce_scatter": orc.ucx_reduce_scatter(ins, orc.FLOAT32, orc.SUM),
+            "all_gather": orc.ucx_all_gather(heads, orc.FLOAT32),
+            "all_to_all": orc.ucx_all_to_all(ins, orc.FLOAT32),
+            "scatter": orc.ucx_scatter(ins, orc.FLOAT32, root),
+            "gather": orc.ucx_gather(heads, orc.FLOAT32, root),
+            "broadcast": orc.ucx_broadcast(heads, orc.FLOAT32, root),
+            "reduce": orc.ucx_reduce(heads, orc.FLOAT32, orc.MAX, root),
+        })
+    outs = [[None] * nranks for _ in range(rounds)]
+
+    def main(comm, rank, _inp, stream):
+        with torch.cuda.stream(stream):
+            staged = [torch.from_numpy(data[r][rank].view(np.uint8).copy()).pin_memory() for r in range(rounds)]
+            host = [{k: torch.empty(sizes[k] * 4, dtype=torch.uint8).pin_memory() for k in names} for _ in range(rounds)]
+            src = torch.empty(length * 4, dtype=torch.uint8, device="cuda:0")
+            dev = {k: torch.full((sizes[k] * 4,), 0x5A, dtype=torch.uint8, device="cuda:0") for k in names}
+            for r in range(rounds):
+                src.copy_(staged[r], non_blocking=True)
+                comm.reduce_scatter(src, dev["reduce_scatter"], part, f32, mr.ReduceOp.SUM, stream)
+                comm.all_gather(src, dev["all_gather"], part, f32, stream)
+                comm.all_to_all(src, dev["all_to_all"], part, f32, stream)
+                comm.scatter(src if rank == root else None, dev["scatter"], part, f32, root, stream)
+                comm.gather(src, dev["gather"] if rank == root else None, part, f32, root, stream)
+                comm.broadcast(src, dev["broadcast"], part, f32, root, stream)
+                comm.reduce(src, dev["reduce"] if rank == root else None, part, f32, mr.ReduceOp.MAX, root, stream)
+                for k in names:
+                    host[r][k].copy_(dev[k], non_blocking=True)
+            stream.synchronize()
+            for r in range(rounds):
+                outs[r][rank] = {k: host[r][k].numpy().view(npf).copy() for k in names}
+        return None
+
+    run_test(nranks, [None] * nranks, [None] * nranks, main)
+    for r in range(rounds):
+        for rank in range(nranks):
+            for k in names:
+                if k in ("gather", "reduce") and rank != root:
+                    continue
+                want = wants[r][k][rank]
+                assert bits_equal(outs[r][rank][k], want), f"round {r} rank {rank} {k}"
