@@ -72,9 +72,30 @@ struct CachedPlan {
     Call key;
     const void* send[kMaxRanks];
     void* recv[kMaxRanks];
+    uint64_t signature;  // plan_signature() of the three above: compared first
+    uint64_t last_used;  // the group's collective count when the plan was last launched
     Plan plan;
     std::vector<KernelCall> calls;  // point into `plan`
 };
+
+// A 64-bit mix of what identifies a planned collective, so that a look-up among many plans compares
+// one word per plan before it compares arguments and addresses.
+uint64_t plan_signature(const Call& c, const void* const* send, void* const* recv) {
+    uint64_t h = 0x9e3779b97f4a7c15ull;
+    const auto mix = [&h](uint64_t v) {
+        h ^= v + 0x9e3779b97f4a7c15ull + (h << 6) + (h >> 2);
+        h *= 0xff51afd7ed558ccdull;
+        h ^= h >> 32;
+    };
+    mix(uint64_t(c.kind) | uint64_t(c.dtype) << 8 | uint64_t(c.op) << 16 | uint64_t(c.root) << 24 |
+        uint64_t(c.order) << 32 | uint64_t(c.sched) << 40 | uint64_t(c.fixed) << 48);
+    mix(c.len);
+    for (uint32_t r = 0; r < kMaxRanks; ++r) {
+        mix(reinterpret_cast<uintptr_t>(send[r]));
+        mix(reinterpret_cast<uintptr_t>(recv[r]));
+    }
+    return h;
+}
 
 // The same for the copy of a point-to-point transfer.
 struct CachedCopy {
@@ -402,10 +423,10 @@ private:
         return MEGRAY_OK;
     }
 
-    CachedPlan* lookup(const Call& lead, const void* const* send, void* const* recv) {
+    CachedPlan* lookup(const Call& lead, const void* const* send, void* const* recv, uint64_t signature) {
         for (auto& cp : m_plans) {
-            if (same_collective(cp->key, lead) && std::memcmp(cp->send, send, sizeof(cp->send)) == 0 &&
-                std::memcmp(cp->recv, recv, sizeof(cp->recv)) == 0)
+            if (cp->signature == signature && same_collective(cp->key, lead) &&
+                std::memcmp(cp->send, send, sizeof(cp->send)) == 0 && std::memcmp(cp->recv, recv, sizeof(cp->recv)) == 0)
                 return cp.get();
         }
         return nullptr;
@@ -472,10 +493,12 @@ private:
             recv[r] = m_slots[r].call.recv;
         }
         // plan first: a rejected call must not leave marks or waits behind
-        CachedPlan* cp = lookup(lead, send, recv);
+        const uint64_t signature = plan_signature(lead, send, recv);
+        CachedPlan* cp = lookup(lead, send, recv, signature);
         if (!cp) {
             auto fresh = std::make_unique<CachedPlan>();
             fresh->key = lead;
+            fresh->signature = signature;
             std::memcpy(fresh->send, send, sizeof(send));
             std::memcpy(fresh->recv, recv, sizeof(recv));
             Status st = plan_collective(fresh->plan, lead.kind, send, recv, m_nranks, lead.len, lead.dtype, lead.order,
@@ -486,11 +509,15 @@ private:
                 m_plans.push_back(std::move(fresh));
                 cp = m_plans.back().get();
             } else {
-                m_plans[m_plan_next] = std::move(fresh);
-                cp = m_plans[m_plan_next].get();
-                m_plan_next = (m_plan_next + 1) % kPlanSlots;
+                // the plan that has gone unused for longest makes room
+                size_t oldest = 0;
+                for (size_t i = 1; i < m_plans.size(); ++i)
+                    if (m_plans[i]->last_used < m_plans[oldest]->last_used) oldest = i;
+                m_plans[oldest] = std::move(fresh);
+                cp = m_plans[oldest].get();
             }
         }
+        cp->last_used = ++m_plan_clock;
         // order the leader's stream behind everything already enqueued on the other ranks' streams
         hipStream_t stream = lead.stream;
         bool one_stream = true, wait_needed = false;
@@ -579,13 +606,13 @@ private:
                 HIP_CHECK(hipMemcpyAsync(dst, src, size, hipMemcpyDeviceToDevice, stream));
                 return MEGRAY_OK;
             }
-            if (m_copies.size() < kPlanSlots) {
+            if (m_copies.size() < kCopySlots) {
                 m_copies.push_back(std::move(fresh));
                 cc = m_copies.back().get();
             } else {
                 m_copies[m_copy_next] = std::move(fresh);
                 cc = m_copies[m_copy_next].get();
-                m_copy_next = (m_copy_next + 1) % kPlanSlots;
+                m_copy_next = (m_copy_next + 1) % kCopySlots;
             }
         }
         for (const KernelCall& call : cc->calls) HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, stream));
@@ -635,7 +662,10 @@ private:
     std::vector<Slot> m_slots;
     std::vector<uint64_t> m_entered;  // per rank: the generation count that ends the collective it last entered
     static constexpr int kSpinPolls = 20000;
-    static constexpr size_t kPlanSlots = 8;
+    // Plans kept per group: a training step repeats the same few dozen collectives (one per gradient bucket) in the
+    // same order, which a cache smaller than that set would miss every time.
+    static constexpr size_t kPlanSlots = 64;
+    static constexpr size_t kCopySlots = 16;
     Status m_result[2] = {MEGRAY_OK, MEGRAY_OK};
     char m_error[2][256] = {"", ""};  // text that goes with m_result
     char m_poison_text[200] = "";
@@ -668,7 +698,7 @@ private:
     std::vector<uint64_t> m_p2p_seq;   // per (source, destination): transfers enqueued between two streams so far
     std::vector<Mailbox> m_mail;
     std::vector<std::unique_ptr<CachedPlan>> m_plans;
-    size_t m_plan_next = 0;
+    uint64_t m_plan_clock = 0;
     std::vector<std::unique_ptr<CachedCopy>> m_copies;  // point-to-point transfers
     size_t m_copy_next = 0;
 };

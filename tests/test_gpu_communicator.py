@@ -510,3 +510,26 @@ def test_back_to_back_rounds_of_every_collective_on_rank_streams(nranks, part):
                     continue
                 want = wants[r][k][rank]
                 assert bits_equal(outs[r][rank][k], want), f"round {r} rank {rank} {k}"
+
+
+def test_more_distinct_collectives_than_the_plan_cache_holds():
+    """A group keeps the plans of its 64 most recently used collectives.  Seventy all_reduces of different lengths,
+    gone through twice in the same order (every call of the second pass finds its plan evicted) and then the last
+    few once more (found), all give the exact sums."""
+    nranks, longest = 4, 70
+    rng = np.random.default_rng(70)
+    ins = [rng.integers(-2 ** 31, 2 ** 31, longest, dtype=np.int64).astype(np.int32) for _ in range(nranks)]
+    total = np.sum(np.stack(ins).astype(np.int64), axis=0).astype(np.int32)  # wraps like the int32 sum
+    lengths = list(range(1, longest + 1)) * 2 + list(range(longest - 5, longest + 1))
+
+    def main(comm, rank, inp, stream):
+        with torch.cuda.stream(stream):
+            src = to_device(inp)
+            outs = [empty_device(n * 4) for n in lengths]
+            for n, dst in zip(lengths, outs):
+                comm.all_reduce(src, dst, n, mr.DType.INT32, mr.ReduceOp.SUM, stream)
+            stream.synchronize()
+            return np.concatenate([to_host(dst, np.int32) for dst in outs])
+
+    want = np.concatenate([total[:n] for n in lengths])
+    run_test(nranks, ins, [want] * nranks, main)
