@@ -23,6 +23,19 @@ def empty_device(nbytes, offset_bytes=0, fill=0xA5):
     return buf[offset_bytes:offset_bytes + nbytes]
 
 
+class Guarded:
+    """An output buffer of `nbytes` bytes at `offset_bytes` from a 256-byte boundary, with `margin` bytes of a known
+    fill on either side: `intact()` tells whether a kernel wrote outside the buffer."""
+
+    def __init__(self, nbytes, offset_bytes=0, fill=0xA5, margin=256):
+        self.fill, self.lo, self.hi = fill, margin + offset_bytes, margin + offset_bytes + nbytes
+        self.buf = torch.full((self.hi + margin,), fill, dtype=torch.uint8, device=DEV)
+        self.view = self.buf[self.lo:self.hi]
+
+    def intact(self):
+        return bool((self.buf[:self.lo] == self.fill).all().item()) and bool((self.buf[self.hi:] == self.fill).all().item())
+
+
 def to_host(view, np_dtype):
     return view.cpu().numpy().view(np_dtype)
 

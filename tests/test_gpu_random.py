@@ -11,7 +11,7 @@ torch = pytest.importorskip("torch")
 pytestmark = pytest.mark.gpu
 
 import megray_amd as mr  # noqa: E402
-from gpu_util import bits_equal, empty_device, first_mismatch, rand_array, to_device, to_host  # noqa: E402
+from gpu_util import Guarded, bits_equal, first_mismatch, rand_array, to_device, to_host  # noqa: E402
 
 REDUCE_TYPES = [orc.INT8, orc.UINT8, orc.INT32, orc.UINT32, orc.INT64, orc.UINT64, orc.FLOAT16, orc.FLOAT32, orc.FLOAT64]
 COPY_TYPES = REDUCE_TYPES + [orc.CHAR]
@@ -21,19 +21,36 @@ def same(got, want, what):
     assert bits_equal(got, want), f"{what}: first mismatch {first_mismatch(got, want)}"
 
 
+_guards = []
+
+
+def empty_device(nbytes, offset_bytes=0):
+    """An output buffer between guard bytes, which the end of the case checks."""
+    _guards.append(Guarded(nbytes, offset_bytes))
+    return _guards[-1].view
+
+
+def check_guards(what):
+    for i, g in enumerate(_guards):
+        assert g.intact(), f"{what}: output buffer {i} of the case was written outside its bounds"
+    _guards.clear()
+
+
 def draw_length(rng, nranks):
     bytes_ = int(np.exp(rng.uniform(np.log(1), np.log(6e6))))
     return max(0, bytes_ + int(rng.integers(-3, 4)))
 
 
 def offsets_for(rng, nranks, size):
-    mode = rng.integers(0, 4)
+    mode = rng.integers(0, 5)
     if mode <= 1:
         return [0] * nranks                       # aligned
     if mode == 2:
         k = int(rng.integers(1, 16 // size + 1)) * size if size < 16 else 0
         return [k % 16] * nranks                  # one common offset from a 16-byte boundary
-    return [int(rng.integers(0, 16 // size)) * size for _ in range(nranks)]  # every buffer its own
+    if mode == 3:
+        return [int(rng.integers(0, 16 // size)) * size for _ in range(nranks)]  # every buffer its own
+    return [int(rng.integers(0, 2048 // size)) * size for _ in range(nranks)]   # ... anywhere on the 1 KiB tile grid
 
 
 @pytest.mark.parametrize("seed", range(6))
@@ -48,7 +65,8 @@ def test_random_reductions(seed):
         kind = rng.choice(["all_reduce", "all_reduce", "reduce_scatter", "reduce"])
         nbytes = draw_length(rng, nranks)
         offs = offsets_for(rng, nranks, size)
-        what = f"seed={seed} case={case} {kind} dtype={dtype} N={nranks} op={op} order={order} offs={offs}"
+        outs = offs if rng.random() < 0.6 else offsets_for(rng, nranks, size)  # outputs at the inputs' offsets, or not
+        what = f"seed={seed} case={case} {kind} dtype={dtype} N={nranks} op={op} order={order} offs={offs} outs={outs}"
         if kind == "all_reduce":
             length = nbytes // size
             sched = mr.Schedule.FUSED if rng.random() < 0.7 else mr.Schedule.TWO_PHASE
@@ -56,7 +74,7 @@ def test_random_reductions(seed):
             ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
             want = orc.fold_all_reduce(ins, dtype, op, order)
             d_in = [to_device(x, offs[r]) for r, x in enumerate(ins)]
-            d_out = d_in if inplace else [empty_device(length * size, offs[r]) for r in range(nranks)]
+            d_out = d_in if inplace else [empty_device(length * size, outs[r]) for r in range(nranks)]
             mr.all_reduce(d_in, d_out, length, dtype, op, order, sched)
             torch.cuda.synchronize()
             for r in range(nranks):
@@ -66,7 +84,7 @@ def test_random_reductions(seed):
             ins = [rand_array(dtype, recvlen * nranks, rng) for _ in range(nranks)]
             want = orc.fold_reduce_scatter(ins, dtype, op, order)
             d_in = [to_device(x, offs[r]) for r, x in enumerate(ins)]
-            d_out = [empty_device(recvlen * size, offs[(r + 1) % nranks]) for r in range(nranks)]
+            d_out = [empty_device(recvlen * size, outs[r]) for r in range(nranks)]
             mr.reduce_scatter(d_in, d_out, recvlen, dtype, op, order)
             torch.cuda.synchronize()
             for r in range(nranks):
@@ -78,10 +96,11 @@ def test_random_reductions(seed):
             ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
             want = orc.fold_all_reduce(ins, dtype, op, order)[0]
             d_in = [to_device(x, offs[r]) for r, x in enumerate(ins)]
-            d_out = empty_device(length * size, offs[root])
+            d_out = empty_device(length * size, outs[root])
             mr.reduce_to_root(d_in, d_out, length, dtype, op, root, order)
             torch.cuda.synchronize()
             same(to_host(d_out, ins[0].dtype), want, f"{what} len={length} root={root}")
+        check_guards(what)
 
 
 @pytest.mark.parametrize("seed", range(3))
@@ -95,13 +114,14 @@ def test_random_copies(seed):
         kind = rng.choice(["all_gather", "all_to_all", "scatter", "gather", "broadcast"])
         block = draw_length(rng, nranks) // size // (nranks if kind != "broadcast" else 1)
         offs = offsets_for(rng, nranks, size)
+        outs = offs if rng.random() < 0.5 else offsets_for(rng, nranks, size)
         root = int(rng.integers(0, nranks))
-        what = f"seed={seed} case={case} {kind} dtype={dtype} N={nranks} block={block} offs={offs} root={root}"
+        what = f"seed={seed} case={case} {kind} dtype={dtype} N={nranks} block={block} offs={offs} outs={outs} root={root}"
         if kind == "all_gather":
             parts = [rand_array(gen, block, rng) for _ in range(nranks)]
             want = orc.ucx_all_gather(parts, dtype)
             d_in = [to_device(x, offs[r]) for r, x in enumerate(parts)]
-            d_out = [empty_device(nranks * block * size, offs[r]) for r in range(nranks)]
+            d_out = [empty_device(nranks * block * size, outs[r]) for r in range(nranks)]
             mr.all_gather(d_in, d_out, block, dtype)
             torch.cuda.synchronize()
             for r in range(nranks):
@@ -110,7 +130,7 @@ def test_random_copies(seed):
             ins = [rand_array(gen, nranks * block, rng) for _ in range(nranks)]
             want = orc.ucx_all_to_all(ins, dtype)
             d_in = [to_device(x, offs[r]) for r, x in enumerate(ins)]
-            d_out = [empty_device(nranks * block * size, offs[r]) for r in range(nranks)]
+            d_out = [empty_device(nranks * block * size, outs[r]) for r in range(nranks)]
             mr.all_to_all(d_in, d_out, block, dtype)
             torch.cuda.synchronize()
             for r in range(nranks):
@@ -119,7 +139,7 @@ def test_random_copies(seed):
             src = rand_array(gen, nranks * block, rng)
             want = orc.ucx_scatter([src if r == root else None for r in range(nranks)], dtype, root)
             d_root = to_device(src, offs[root])
-            d_out = [empty_device(block * size, offs[r]) for r in range(nranks)]
+            d_out = [empty_device(block * size, outs[r]) for r in range(nranks)]
             mr.scatter(d_root, d_out, block, dtype, root)
             torch.cuda.synchronize()
             for r in range(nranks):
@@ -128,7 +148,7 @@ def test_random_copies(seed):
             parts = [rand_array(gen, block, rng) for _ in range(nranks)]
             want = orc.ucx_gather(parts, dtype, root)[root]
             d_in = [to_device(x, offs[r]) for r, x in enumerate(parts)]
-            d_root = empty_device(nranks * block * size, offs[root])
+            d_root = empty_device(nranks * block * size, outs[root])
             mr.gather(d_in, d_root, block, dtype, root)
             torch.cuda.synchronize()
             same(to_host(d_root, parts[0].dtype), want, what)
@@ -136,8 +156,9 @@ def test_random_copies(seed):
             parts = [rand_array(gen, block, rng) for _ in range(nranks)]
             want = orc.ucx_broadcast(parts, dtype, root)
             d_root = to_device(parts[root], offs[root])
-            d_out = [empty_device(block * size, offs[r]) for r in range(nranks)]
+            d_out = [empty_device(block * size, outs[r]) for r in range(nranks)]
             mr.broadcast(d_root, d_out, block, dtype, root)
             torch.cuda.synchronize()
             for r in range(nranks):
                 same(to_host(d_out[r], parts[0].dtype), want[r], f"{what} rank={r}")
+        check_guards(what)
