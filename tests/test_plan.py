@@ -2,6 +2,8 @@
 by run, and must reproduce the oracle's literal replays bit for bit.  This checks chunking, fold
 orders, tie conventions, the head / vector-body / tail split and the multi-launch schedules
 independently of the kernels."""
+import os
+
 import numpy as np
 import pytest
 
@@ -408,3 +410,25 @@ def test_runs_whose_tiles_share_cache_lines_are_dealt_to_xcds():
     runs = vector_runs(mr.Collective.ALL_REDUCE, fake_ptrs(1 << 44, nranks, offs, stride=1 << 40),
                        fake_ptrs(1 << 46, nranks, offs, stride=1 << 40), big, mr.DType.FLOAT32)
     assert runs and all(r["deal"] == 1 for r in runs)
+
+
+def test_random_plans_keep_inside_the_buffers_under_host_sanitizers(tmp_path):
+    """tests/cpp/plan_fuzz.cpp: the host planner (pure host code) built with the address and undefined-behaviour
+    sanitizers and called with random collectives, rank counts, element sizes, lengths up to 2^33 elements and
+    buffer offsets.  Every launch descriptor of every plan must keep the kernels inside the callers' buffers, the
+    tile tables must add up, and the one-pass plans must write every output element exactly once."""
+    import shutil
+    import subprocess
+
+    gxx = shutil.which("g++")
+    if not gxx:
+        pytest.skip("no host compiler")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = str(tmp_path / "plan_fuzz")
+    build = subprocess.run([gxx, "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
+                            f"-I{root}/include", f"-I{root}/megray_amd/csrc", f"{root}/tests/cpp/plan_fuzz.cpp",
+                            f"{root}/megray_amd/csrc/vrank_plan.cpp", "-o", exe], capture_output=True, text=True, timeout=300)
+    assert build.returncode == 0, build.stderr
+    for seed in ("11", "12"):
+        run = subprocess.run([exe, "30000", seed], capture_output=True, text=True, timeout=300)
+        assert run.returncode == 0 and run.stdout.startswith("ok "), run.stdout + run.stderr
