@@ -16,7 +16,8 @@
 //
 // Rounds vary the rank count's streams (one each, all shared, mixed), the collective and its length (launches
 // that carry the ordering themselves, launches between wait and notify kernels, group launches), the
-// allocation-free entry point, rounds in which one rank's arguments are rejected, and rings of send / recv.
+// allocation-free entry point, the rooted collectives, rounds in which one rank's arguments are rejected, and rings of
+// send / recv.
 // Usage: stream_sim [rounds] [seed] [events]; prints "ok" or the first violation.
 #include <sys/mman.h>
 
@@ -317,7 +318,9 @@ hipError_t hipMemcpyAsync(void* dst, const void* src, size_t, hipMemcpyKind, hip
 namespace {
 
 struct Round {
-    int kind;                  // 0 all_reduce, 1 all_gather, 2 all_to_all, 3 reduce_scatter, 4 ring of send / recv
+    int kind;                  // 0 all_reduce, 1 all_gather, 2 all_to_all, 3 reduce_scatter, 4 ring of send / recv,
+                               // 5 broadcast, 6 reduce, 7 scatter, 8 gather
+    uint32_t root;
     size_t len;
     bool fixed;                // the allocation-free all_reduce
     int poisoned;              // rank whose arguments are rejected, or -1
@@ -364,7 +367,8 @@ int main(int argc, char** argv) {
     const size_t lengths[] = {16, 70000, 100000, 600000, 3, 1001};
     std::vector<Round> plan(rounds);
     for (Round& r : plan) {
-        r.kind = int(rng() % 5);
+        r.kind = int(rng() % 9);
+        r.root = uint32_t(rng() % nranks);
         r.len = lengths[rng() % 6];
         if (r.kind != 0) r.len = r.len / nranks + 1;
         r.fixed = r.kind == 0 && rng() % 5 == 0;
@@ -429,6 +433,10 @@ int main(int argc, char** argv) {
                     case 1: got = comm->all_gather(src, dst, round.len, dtype, ctx); break;
                     case 2: got = comm->all_to_all(src, dst, round.len, dtype, ctx); break;
                     case 3: got = comm->reduce_scatter(src, dst, round.len, dtype, MEGRAY_SUM, ctx); break;
+                    case 5: got = comm->broadcast(src, dst, round.len, dtype, round.root, ctx); break;
+                    case 6: got = comm->reduce(src, dst, round.len, dtype, MEGRAY_MAX, round.root, ctx); break;
+                    case 7: got = comm->scatter(src, dst, round.len, dtype, round.root, ctx); break;
+                    case 8: got = comm->gather(src, dst, round.len, dtype, round.root, ctx); break;
                     default:
                         if (nranks < 2) break;
                         comm->group_start();
@@ -446,8 +454,9 @@ int main(int argc, char** argv) {
                 if (round.poisoned == int(rank) ? !threw : got != MEGRAY_INVALID_USAGE) violation("a rejected call was not reported");
             } else {
                 if (threw || got != MEGRAY_OK) violation("a collective failed");
-                // the consumer: this rank's output holds the round, on this rank's stream
-                push(stream, [dst, version]() {
+                // the consumer: this rank's output (if the collective gives it one) holds the round, on this rank's stream
+                const bool has_output = (round.kind != 6 && round.kind != 8) || rank == round.root;
+                if (has_output) push(stream, [dst, version]() {
                     if (load_word(dst) != version) violation("a rank's stream went on before the collective's result was there");
                     return true;
                 });
