@@ -235,6 +235,10 @@ MRV_API int mrv_comm_init(mrv_comm* comm, const char* master_ip, int port);
 /* Fold order / schedule of this rank's communicator (MRV_ORDER_*, MRV_SCHED_*); no reference counterpart. */
 MRV_API int mrv_comm_configure(mrv_comm* comm, int order, int schedule);
 
+/* Communicator::send / recv (include/megray/communicator.h:51-57): `len` elements of `dtype` to / from rank `rank`.
+ * A send and the matching receive become one block copy between the two ranks' buffers, enqueued on the receiver's
+ * stream behind everything the sender's stream held at the send; the sender's stream goes on when the copy is done.
+ * Outside mrv_comm_group_start / _end a call returns when its counterpart has been posted and the copy is enqueued. */
 MRV_API int mrv_comm_send(mrv_comm* comm, const void* sendbuff, size_t len, int dtype, uint32_t rank,
                           void* stream);
 MRV_API int mrv_comm_recv(mrv_comm* comm, void* recvbuff, size_t len, int dtype, uint32_t rank, void* stream);
