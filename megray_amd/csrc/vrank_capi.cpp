@@ -62,6 +62,9 @@ int guarded(F&& body) {
     } catch (const std::exception& e) {
         set_error(e.what());
         return int(MEGRAY_UNEXPECTED_ERR);
+    } catch (...) {  // nothing may unwind through the C boundary
+        set_error("unknown failure");
+        return int(MEGRAY_UNEXPECTED_ERR);
     }
 }
 
