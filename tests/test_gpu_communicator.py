@@ -533,3 +533,44 @@ def test_more_distinct_collectives_than_the_plan_cache_holds():
 
     want = np.concatenate([total[:n] for n in lengths])
     run_test(nranks, ins, [want] * nranks, main)
+
+
+def test_two_groups_at_the_same_time():
+    """Two communicator groups of four ranks each, alive and busy at the same time (eight rank threads, eight streams):
+    each group keeps its own counters, plans and rendezvous, so their collectives - short ones that carry the stream
+    ordering themselves and long ones between wait and notify kernels - do not disturb each other."""
+    nranks, rounds = 4, 12
+    results = {}
+
+    def group_main(tag, length):
+        rng = np.random.default_rng(1000 + tag)
+        ins = [rand_array(orc.FLOAT32, length, rng) for _ in range(nranks)]
+        want = orc.ucx_all_reduce(ins, orc.FLOAT32, orc.SUM)
+
+        def main(comm, rank, inp, stream):
+            with torch.cuda.stream(stream):
+                staged = torch.from_numpy(inp.view(np.uint8).copy()).pin_memory()
+                src = torch.empty(length * 4, dtype=torch.uint8, device="cuda:0")
+                dst = torch.full((length * 4,), 0x5A, dtype=torch.uint8, device="cuda:0")
+                host_out = torch.empty(length * 4, dtype=torch.uint8).pin_memory()
+                for _ in range(rounds):
+                    src.copy_(staged, non_blocking=True)
+                    comm.all_reduce(src, dst, length, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream)
+                    host_out.copy_(dst, non_blocking=True)
+                stream.synchronize()
+                return host_out.numpy().view(np.float32).copy()
+
+        try:
+            run_test(nranks, ins, want, main)
+            results[tag] = "ok"
+        except BaseException as exc:  # noqa: BLE001
+            results[tag] = repr(exc)
+
+    threads = [threading.Thread(target=group_main, args=(0, 20000), daemon=True),
+               threading.Thread(target=group_main, args=(1, 300000), daemon=True)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(200)
+        assert not t.is_alive(), "a group hung"
+    assert results == {0: "ok", 1: "ok"}, results
