@@ -273,6 +273,7 @@ int mrv_plan_create(int collective, const void* const* sendbuffs, void* const* r
                 params.func = const_cast<void*>(call.kernel);
                 params.gridDim = dim3(call.grid);
                 params.blockDim = dim3(call.block);
+                params.sharedMemBytes = call.lds;
                 params.kernelParams = args;
                 hipGraphNode_t node = nullptr;
                 HIP_CHECK(hipGraphAddKernelNode(&node, p->graph, prev ? &prev : nullptr, prev ? 1 : 0, &params));
@@ -293,7 +294,7 @@ int mrv_plan_launch(const mrv_plan* plan, void* stream) {
             return MEGRAY_OK;
         }
         for (const KernelCall& call : plan->calls)
-            HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, as_stream(stream)));
+            HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, as_stream(stream), call.lds));
         return MEGRAY_OK;
     });
 }

@@ -551,7 +551,7 @@ private:
         } else if (wait_needed && set.words) {
             HIP_CHECK(edge_wait_arrived(set.words, set.marks.load(std::memory_order_relaxed), m_limit_ticks, set.status, stream));
         }
-        for (const KernelCall& call : cp->calls) HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, stream));
+        for (const KernelCall& call : cp->calls) HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, stream, call.lds));
         // the other ranks order their streams behind this point themselves (none has to if all share the stream)
         if (hook) {
             *hooked.target = *hooked.ticket = 0;
@@ -615,7 +615,7 @@ private:
                 m_copy_next = (m_copy_next + 1) % kCopySlots;
             }
         }
-        for (const KernelCall& call : cc->calls) HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, stream));
+        for (const KernelCall& call : cc->calls) HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, stream, call.lds));
         return MEGRAY_OK;
     }
 

@@ -93,7 +93,10 @@ Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCal
                     call = {flat_kernel_for(step.flat, dtype, op), group_grid(step.flat.total_tiles),
                             kThreads * kGroupWaves, &step.flat};
                 else
-                    call = {flat_kernel_for(step.flat, dtype, op), step.flat.total_tiles, kThreads, &step.flat};
+                    call = {flat_kernel_for(step.flat, dtype, op), step.flat.total_tiles, kThreads, &step.flat,
+                            // the planner leaves a launch this large at one wavefront per tile only to have it
+                            // run at a reduced occupancy
+                            step.flat.total_tiles >= kFlatOneOutMinTiles ? flat_one_out_lds(step.flat.nranks) : 0u};
                 break;
             case Step::kTree:
                 call = {tree_kernel_for(step.tree, dtype, op), step.tree.total_tiles, kThreads, &step.tree};
@@ -120,7 +123,7 @@ Status execute(const Plan& plan, DType dtype, ReduceOp op, hipStream_t stream) {
     std::vector<KernelCall> calls;
     const Status st = resolve(plan, dtype, op, calls);
     if (st != MEGRAY_OK) return st;
-    for (const KernelCall& call : calls) HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, stream));
+    for (const KernelCall& call : calls) HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, stream, call.lds));
     return MEGRAY_OK;
 }
 

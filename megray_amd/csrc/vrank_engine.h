@@ -29,6 +29,7 @@ struct KernelCall {
     uint32_t grid;
     uint32_t block;  // threads per workgroup
     const void* launch;
+    uint32_t lds = 0;  // LDS bytes reserved per workgroup on top of the kernel's own (sets the occupancy)
 };
 
 // Which collective a plan is for (the values of the C ABI's MRV_* selectors).

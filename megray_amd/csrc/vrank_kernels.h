@@ -17,8 +17,10 @@ const void* tree_kernel_for(const TreeLaunch& launch, DType dtype, ReduceOp op);
 const void* pack_kernel_for(const PackLaunch& launch);
 
 // Enqueue `kernel` over `grid` workgroups of `block` threads (one or four wavefronts) with `*launch` as
-// its only argument.
-hipError_t enqueue(const void* kernel, uint32_t grid, uint32_t block, const void* launch, hipStream_t stream);
+// its only argument.  `lds` bytes of LDS are reserved per workgroup on top of what the kernel declares (it never
+// touches them: fewer workgroups then share a CU, see flat_one_out_lds).
+hipError_t enqueue(const void* kernel, uint32_t grid, uint32_t block, const void* launch, hipStream_t stream,
+                   uint32_t lds = 0);
 
 }  // namespace vrank
 }  // namespace MegRay

@@ -244,11 +244,12 @@ const void* pack_kernel_for(const PackLaunch& L) {
                                   : reinterpret_cast<const void*>(&pack_kernel);
 }
 
-hipError_t enqueue(const void* kernel, uint32_t grid, uint32_t block, const void* launch, hipStream_t stream) {
+hipError_t enqueue(const void* kernel, uint32_t grid, uint32_t block, const void* launch, hipStream_t stream,
+                   uint32_t lds) {
     if (!kernel) return hipErrorInvalidValue;
     if (!grid) return hipSuccess;
     void* args[] = {const_cast<void*>(launch)};
-    return hipLaunchKernel(kernel, dim3(grid), dim3(block), args, 0, stream);
+    return hipLaunchKernel(kernel, dim3(grid), dim3(block), args, lds, stream);
 }
 
 }  // namespace vrank

@@ -158,11 +158,13 @@ private:
         // the inputs' offsets) also exchange the results between the wavefronts of a group
         bool unshifted = true;
         for (const Run& r : m_runs) unshifted = unshifted && r.in_begin == r.out_begin;
-        L.waves = total >= kFlatGroupMinTiles ? kGroupWaves : 1;
-        L.exchange = (L.waves == kGroupWaves && !m_tree && m_nout == m_nranks && unshifted) ? 1 : 0;
         // tiles that do not sit on the cache lines of every buffer share lines with their neighbours
         bool on_lines = lines_shared(0) && m_misalign % 128 == 0;  // flat tiles start at the buffers' first byte
         for (const Run& r : m_runs) on_lines = on_lines && lines_shared((r.in_begin - r.out_begin) * m_elem);
+        // (large one-output folds on line boundaries stay at one wavefront per tile, see flat_one_out)
+        const bool one_wave = total < kFlatGroupMinTiles || (on_lines && flat_one_out(m_nranks, m_nout, total));
+        L.waves = one_wave ? 1 : kGroupWaves;
+        L.exchange = (L.waves == kGroupWaves && !m_tree && m_nout == m_nranks && unshifted) ? 1 : 0;
         if (L.waves == kGroupWaves && !on_lines) L.exchange |= 2u;
         L.unshifted = unshifted ? 1 : 0;
         m_plan.steps.push_back(step);

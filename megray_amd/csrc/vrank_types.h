@@ -117,6 +117,23 @@ constexpr uint32_t kGroupWaves = 4;
 constexpr uint32_t kGroupStride = 32;
 constexpr uint32_t kGroupMinTiles = 512;
 constexpr uint32_t kFlatGroupMinTiles = 2048;
+// Large flat folds with ONE output (reduce_scatter, reduce, the first launch of the two-phase all_reduce), three
+// or more inputs and tiles on cache-line boundaries stay at one wavefront per tile and run at a reduced occupancy instead: a wavefront has its K
+// loads in flight at once, and what HBM needs to stay busy (bandwidth x latency, about 32 KiB per CU) is reached by
+// far fewer wavefronts than a CU can hold - the rest only queue up in the memory system and get in each other's
+// way.  The occupancy is set by LDS reserved per workgroup at launch, which the kernel never touches.  Measured on
+// MI355X, % of the HBM peak, group form / one wavefront per tile at 32, 20, 16, 13 wavefronts per CU (fp32, 2^26
+// elements per rank): 8 ranks reduce_scatter 81 / 79, 84, 87, 87 and reduce 82 / 80, 85, 87, 87; 4 ranks 80 / -, 85.5,
+// 85.5, 82 and 80 / -, 87, 84, 80; 3 ranks 80 / -, 80, 80, 80 and 82 / -, 86, 81, 77; 2 ranks 84 / -, 84, 76, 69 (two
+// loads per wavefront need every wavefront there is: left in the group form).  fp16, int8 and int64 behave like fp32;
+// below 8192 tiles per buffer the group form is level or ahead.
+constexpr uint32_t kFlatOneOutMinTiles = 8192;
+constexpr uint32_t flat_one_out_lds(uint32_t nranks) {  // LDS bytes reserved per one-wavefront workgroup
+    return nranks >= 8 ? 10240u : 8192u;                 // 16 resp. 20 wavefronts per CU (160 KiB of LDS)
+}
+constexpr bool flat_one_out(uint32_t nranks, uint32_t nout, uint64_t total_tiles) {
+    return nout == 1 && nranks >= 3 && total_tiles >= kFlatOneOutMinTiles;
+}
 // One-wavefront launches below this many workgroups carry the thread-per-rank API's stream ordering
 // themselves (EdgeHooks).  Beyond it the release fence every workgroup then executes costs more than
 // the two launches it saves.  Measured, 8 ranks, a stream per rank, microseconds per all_reduce with /

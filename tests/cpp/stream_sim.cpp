@@ -169,7 +169,7 @@ const void* flat_kernel_for(const FlatLaunch&, DType, ReduceOp) { return &g_tags
 const void* tree_kernel_for(const TreeLaunch&, DType, ReduceOp) { return &g_tags[kTagTree]; }
 const void* pack_kernel_for(const PackLaunch&) { return &g_tags[kTagPack]; }
 
-hipError_t enqueue(const void* kernel, uint32_t grid, uint32_t, const void* launch, hipStream_t stream) {
+hipError_t enqueue(const void* kernel, uint32_t grid, uint32_t, const void* launch, hipStream_t stream, uint32_t) {
     if (!kernel) return hipErrorInvalidValue;
     if (!grid) return hipSuccess;
     switch (*static_cast<const int*>(kernel)) {

@@ -262,11 +262,21 @@ def test_full_size_plan_shapes():
     assert sum(r["count"] for r in runs) == n
     assert br == bw == 8 * n * 4
     assert all(r["waves"] == 4 for r in runs)  # the group form: four wavefronts, four tiles per workgroup
-    # so do long reduce_scatter and tree launches; short launches keep one wavefront per tile
-    rs, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, sp, rp, 1 << 22, orc.FLOAT32)
+    # so do reduce_scatter and tree launches of 2048 to 8191 tiles per buffer; short launches keep one wavefront per tile
+    rs, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, sp, rp, 1 << 17, orc.FLOAT32)
     assert rs and all(r["waves"] == 4 and r["vector"] == 2 for r in rs)
-    tree, _, _ = mr.describe(mr.Collective.REDUCE, sp, rp, 1 << 22, orc.FLOAT32, root=3)
+    tree, _, _ = mr.describe(mr.Collective.REDUCE, sp, rp, 1 << 20, orc.FLOAT32, root=3)
     assert tree and all(r["waves"] == 4 and r["dir"] == 0 for r in tree)
+    # from 8192 tiles on, folds of three or more inputs into ONE output go back to one wavefront per tile (launched
+    # at a reduced occupancy); two inputs stay in the group form
+    rs, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, sp, rp, 1 << 22, orc.FLOAT32)
+    assert rs and all(r["waves"] == 1 and r["vector"] == 2 for r in rs)
+    tree, _, _ = mr.describe(mr.Collective.REDUCE, sp, rp, 1 << 22, orc.FLOAT32, root=3)
+    assert tree and all(r["waves"] == 1 and r["dir"] == 0 for r in tree)
+    two_phase, _, _ = mr.describe(mr.Collective.ALL_REDUCE, sp, rp, 1 << 24, orc.FLOAT32, schedule=mr.Schedule.TWO_PHASE)
+    assert {r["waves"] for r in two_phase if r["step"] == 0 and r["nfold"] == 8} == {1}
+    pair, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, sp[:2], rp[:2], 1 << 24, orc.FLOAT32, nranks=2)
+    assert pair and all(r["waves"] == 4 for r in pair)
     for coll, count in ((mr.Collective.ALL_REDUCE, 1 << 15), (mr.Collective.REDUCE_SCATTER, 1 << 12),
                         (mr.Collective.REDUCE, 1 << 15)):
         small, _, _ = mr.describe(coll, sp, rp, count, orc.FLOAT32)
@@ -387,7 +397,7 @@ def test_runs_whose_tiles_share_cache_lines_are_dealt_to_xcds():
     # everything on 256-byte boundaries: plain order, flat and segment kernels
     runs = vector_runs(mr.Collective.ALL_REDUCE, send, recv, big, mr.DType.FLOAT32)
     assert runs and all(r["deal"] == 0 for r in runs)
-    runs = vector_runs(mr.Collective.REDUCE_SCATTER, send, recv, big // nranks, mr.DType.FLOAT32)
+    runs = vector_runs(mr.Collective.REDUCE_SCATTER, send, recv, (1 << 20) // nranks, mr.DType.FLOAT32)  # 4096 tiles
     assert runs and all(r["deal"] == 0 for r in runs)
     five_s, five_r = send[:5], recv[:5]
     runs = vector_runs(mr.Collective.ALL_REDUCE, five_s, five_r, 5 * (1 << 20), mr.DType.FLOAT32)
