@@ -138,6 +138,53 @@ def tree_expectation(ins, dtype, op, root):
         return a[0].astype(np.float16)
 
 
+@pytest.mark.parametrize("dtype", [orc.FLOAT32, orc.FLOAT16, orc.INT8, orc.INT64])
+def test_large_folds_into_one_output_at_reduced_occupancy(dtype):
+    """reduce_scatter, reduce towards a root and the two-phase all_reduce from 8192 tiles per buffer on, tiles on
+    cache-line boundaries, three or more ranks: one wavefront per tile, launched with LDS reserved per workgroup so
+    that fewer wavefronts share a CU - eagerly, as a planned HIP graph (the reservation is part of the kernel
+    node) and with two ranks (which stay in the group form)."""
+    size = orc.dtype_size(dtype)
+    rng = np.random.default_rng(991 + dtype)
+    for nranks, tiles, waves in ((8, 8200, 1), (3, 8200, 1), (2, 8200, 4)):
+        recvlen = (tiles * 1024 // size + nranks - 1) // nranks // 128 * 128 + 128  # chunks on 128-byte boundaries
+        length = recvlen * nranks
+        ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+        d_in = [to_device(x) for x in ins]
+        parts = [empty_device(recvlen * size) for _ in range(nranks)]
+        runs, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, d_in, parts, recvlen, dtype)
+        assert runs and all(r["waves"] == waves for r in runs), "not the kernel form this test is about"
+        for op, order in ((orc.SUM, orc.ORDER_UCX), (orc.MIN, orc.ORDER_SHM)):
+            want = orc.fold_reduce_scatter(ins, dtype, op, order)
+            mr.reduce_scatter(d_in, parts, recvlen, dtype, op, order)
+            torch.cuda.synchronize()
+            for r in range(nranks):
+                assert_same(to_host(parts[r], ins[0].dtype), want[r], f"reduce_scatter dtype={dtype} N={nranks} op={op} rank={r}")
+            plan = mr.CollectivePlan(mr.Collective.REDUCE_SCATTER, d_in, parts, recvlen, dtype, op, order=order, graph=True)
+            for replay in range(2):
+                for o in parts:
+                    o.fill_(replay)
+                torch.cuda.synchronize()
+                plan.launch()
+                torch.cuda.synchronize()
+                for r in range(nranks):
+                    assert_same(to_host(parts[r], ins[0].dtype), want[r], f"planned reduce_scatter dtype={dtype} N={nranks} replay={replay}")
+            plan.close()
+        root = nranks - 1
+        out = empty_device(length * size)
+        mr.reduce_to_root(d_in, out, length, dtype, orc.MAX, root)
+        torch.cuda.synchronize()
+        assert_same(to_host(out, ins[0].dtype), tree_expectation(ins, dtype, orc.MAX, root), f"tree reduce dtype={dtype} N={nranks}")
+        mr.reduce_to_root(d_in, out, length, dtype, orc.SUM, root, orc.ORDER_RANK0)
+        torch.cuda.synchronize()
+        assert_same(to_host(out, ins[0].dtype), orc.fold_all_reduce(ins, dtype, orc.SUM, orc.ORDER_RANK0)[0],
+                    f"left-fold reduce dtype={dtype} N={nranks}")
+        got = run_all_reduce(ins, dtype, orc.SUM, orc.ORDER_UCX, mr.Schedule.TWO_PHASE)
+        want = orc.fold_all_reduce(ins, dtype, orc.SUM, orc.ORDER_UCX)
+        for r in range(nranks):
+            assert_same(got[r], want[r], f"two-phase all_reduce dtype={dtype} N={nranks} rank={r}")
+
+
 @pytest.mark.parametrize("dtype", REDUCE_TYPES)
 def test_group_form_with_one_output(dtype):
     """reduce_scatter, reduce towards a root and the two-phase all_reduce on long buffers: the
