@@ -92,11 +92,13 @@ Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCal
                 if (step.flat.waves == kGroupWaves)
                     call = {flat_kernel_for(step.flat, dtype, op), group_grid(step.flat.total_tiles),
                             kThreads * kGroupWaves, &step.flat};
-                else
-                    call = {flat_kernel_for(step.flat, dtype, op), step.flat.total_tiles, kThreads, &step.flat,
-                            // the planner leaves a launch this large at one wavefront per tile only to have it
-                            // run at a reduced occupancy
-                            step.flat.total_tiles >= kFlatOneOutMinTiles ? flat_one_out_lds(step.flat.nranks) : 0u};
+                else {
+                    call = {flat_kernel_for(step.flat, dtype, op), step.flat.total_tiles, kThreads, &step.flat};
+                    // the planner leaves a launch this large at one wavefront per tile only to have it run at a
+                    // reduced occupancy (flat_one_out)
+                    if (step.flat.total_tiles >= kFlatOneOutMinTiles)
+                        call.lds = lds_for_waves_per_cu(call.kernel, flat_one_out_waves_per_cu(step.flat.nranks));
+                }
                 break;
             case Step::kTree:
                 call = {tree_kernel_for(step.tree, dtype, op), step.tree.total_tiles, kThreads, &step.tree};

@@ -18,9 +18,13 @@ const void* pack_kernel_for(const PackLaunch& launch);
 
 // Enqueue `kernel` over `grid` workgroups of `block` threads (one or four wavefronts) with `*launch` as
 // its only argument.  `lds` bytes of LDS are reserved per workgroup on top of what the kernel declares (it never
-// touches them: fewer workgroups then share a CU, see flat_one_out_lds).
+// touches them: fewer workgroups then share a CU).
 hipError_t enqueue(const void* kernel, uint32_t grid, uint32_t block, const void* launch, hipStream_t stream,
                    uint32_t lds = 0);
+
+// LDS bytes to reserve per workgroup of `kernel`, on top of what it declares, so that at most `waves_per_cu`
+// of its one-wavefront workgroups share a CU (160 KiB of LDS each); 0 if the kernel's own LDS already sees to that.
+uint32_t lds_for_waves_per_cu(const void* kernel, uint32_t waves_per_cu);
 
 }  // namespace vrank
 }  // namespace MegRay

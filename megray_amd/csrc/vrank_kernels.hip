@@ -4,6 +4,9 @@
 // src/ucx/scatter.cpp:30-44 and src/ucx/gather.cpp:30-44) and the plain copies of the fold kernel.
 #include "vrank_fold_impl.hpp"
 
+#include <mutex>
+#include <unordered_map>
+
 namespace MegRay {
 namespace vrank {
 
@@ -242,6 +245,30 @@ const void* tree_kernel_for(const TreeLaunch&, DType dtype, ReduceOp op) {
 const void* pack_kernel_for(const PackLaunch& L) {
     return L.waves == kGroupWaves ? reinterpret_cast<const void*>(&pack_group_kernel)
                                   : reinterpret_cast<const void*>(&pack_kernel);
+}
+
+uint32_t lds_for_waves_per_cu(const void* kernel, uint32_t waves_per_cu) {
+    constexpr uint32_t kLdsPerCu = 160 * 1024;
+    if (!kernel || !waves_per_cu) return 0;
+    // what the kernel declares itself, asked of the runtime once per kernel
+    static std::mutex mutex;
+    static std::unordered_map<const void*, uint32_t> declared;
+    uint32_t own = 0;
+    {
+        std::lock_guard<std::mutex> lock(mutex);
+        auto it = declared.find(kernel);
+        if (it == declared.end()) {
+            hipFuncAttributes attr;
+            if (hipFuncGetAttributes(&attr, kernel) != hipSuccess) {
+                (void)hipGetLastError();
+                return 0;
+            }
+            it = declared.emplace(kernel, uint32_t(attr.sharedSizeBytes)).first;
+        }
+        own = it->second;
+    }
+    const uint32_t each = kLdsPerCu / waves_per_cu / 1024 * 1024;  // whole KiB: allocation granules stay out of it
+    return each > own ? each - own : 0;
 }
 
 hipError_t enqueue(const void* kernel, uint32_t grid, uint32_t block, const void* launch, hipStream_t stream,

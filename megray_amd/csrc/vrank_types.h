@@ -118,18 +118,22 @@ constexpr uint32_t kGroupStride = 32;
 constexpr uint32_t kGroupMinTiles = 512;
 constexpr uint32_t kFlatGroupMinTiles = 2048;
 // Large flat folds with ONE output (reduce_scatter, reduce, the first launch of the two-phase all_reduce), three
-// or more inputs and tiles on cache-line boundaries stay at one wavefront per tile and run at a reduced occupancy instead: a wavefront has its K
-// loads in flight at once, and what HBM needs to stay busy (bandwidth x latency, about 32 KiB per CU) is reached by
-// far fewer wavefronts than a CU can hold - the rest only queue up in the memory system and get in each other's
-// way.  The occupancy is set by LDS reserved per workgroup at launch, which the kernel never touches.  Measured on
-// MI355X, % of the HBM peak, group form / one wavefront per tile at 32, 20, 16, 13 wavefronts per CU (fp32, 2^26
-// elements per rank): 8 ranks reduce_scatter 81 / 79, 84, 87, 87 and reduce 82 / 80, 85, 87, 87; 4 ranks 80 / -, 85.5,
-// 85.5, 82 and 80 / -, 87, 84, 80; 3 ranks 80 / -, 80, 80, 80 and 82 / -, 86, 81, 77; 2 ranks 84 / -, 84, 76, 69 (two
-// loads per wavefront need every wavefront there is: left in the group form).  fp16, int8 and int64 behave like fp32;
-// below 8192 tiles per buffer the group form is level or ahead.
+// or more inputs and tiles on cache-line boundaries stay at one wavefront per tile and run at a reduced occupancy
+// instead: a wavefront has its K loads of 1 KiB in flight at once, and what HBM needs to stay busy (bandwidth x
+// latency, 32 - 64 KiB per CU) is in flight with far fewer wavefronts than a CU can hold - the rest only queue up
+// in the memory system and get in each other's way.  The occupancy is set by LDS reserved per workgroup at launch,
+// on top of what the kernel declares, which nothing ever touches (lds_for_waves_per_cu).  Measured on MI355X, % of
+// the HBM peak, fp32, 2^26 elements per rank (fp16, int8 and int64 behave alike), group form against one wavefront
+// per tile at the given wavefronts per CU:
+//   8 ranks  reduce_scatter 81 against 83 (12), 85 (10), 85 (9), 86 - 87 (8), 84 (7), 78 (6), 69 (5); reduce 82 against 87 (8)
+//   4 ranks  reduce_scatter 80 against 85.5 (13), 85.5 (11), 82 (10); reduce 80 against 87 (13), 84 (11), 80 (10)
+//   3 ranks  reduce_scatter 80 against 80 (14), 80 (12), 80 (10); reduce 82 against 86 (14), 81 (12), 77 (10)
+//   2 ranks  84 against 84 (16), 76 (13), 69 (11): two loads per wavefront need every wavefront there is; left in
+//            the group form
+// Below 8192 tiles per buffer the group form is level or ahead.
 constexpr uint32_t kFlatOneOutMinTiles = 8192;
-constexpr uint32_t flat_one_out_lds(uint32_t nranks) {  // LDS bytes reserved per one-wavefront workgroup
-    return nranks >= 8 ? 10240u : 8192u;                 // 16 resp. 20 wavefronts per CU (160 KiB of LDS)
+constexpr uint32_t flat_one_out_waves_per_cu(uint32_t nranks) {
+    return nranks >= 8 ? 8u : nranks == 4 ? 13u : 14u;
 }
 constexpr bool flat_one_out(uint32_t nranks, uint32_t nout, uint64_t total_tiles) {
     return nout == 1 && nranks >= 3 && total_tiles >= kFlatOneOutMinTiles;

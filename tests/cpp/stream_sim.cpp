@@ -197,6 +197,8 @@ hipError_t enqueue(const void* kernel, uint32_t grid, uint32_t, const void* laun
     return hipSuccess;
 }
 
+uint32_t lds_for_waves_per_cu(const void*, uint32_t) { return 0; }
+
 static uint64_t g_static_words[kStaticEdgeSlots * (sizeof(EdgeWords) / sizeof(uint64_t))];
 
 hipError_t edge_static_words(uint32_t slot, EdgeWords** words) {
