@@ -27,8 +27,9 @@ def refill(dev, arr):
     dev.copy_(torch.from_numpy(np.ascontiguousarray(arr).view(np.uint8).reshape(-1).copy()))
 
 
-# lengths: one that runs the short kernels (one wavefront per tile), one that runs the group kernels
-@pytest.mark.parametrize("length", [8 * 1000 + 8, 8 * 3000 * 256 + 8 * 5])
+# lengths: one that runs the short kernels (one wavefront per tile), one that runs the group kernels, and one whose
+# chunks lie on cache-line boundaries, so that the one-output folds run at the reduced occupancy (LDS reserved at launch)
+@pytest.mark.parametrize("length", [8 * 1000 + 8, 8 * 3000 * 256 + 8 * 5, 8 * 3000 * 256 + 8 * 32])
 def test_captured_collectives_replay_on_fresh_data(length):
     rng = np.random.default_rng(length)
     nranks = 8
