@@ -388,12 +388,15 @@ def run_other_workload(args, torch, mr):
 
 
 def other_configs(torch, mr, layout):
-    """The other benchmark configurations, twenty timed steps each after five warm-up steps: milliseconds per collective (HIP events),
+    """The other benchmark configurations, twenty timed steps each after five warm-up steps (a hundred after fifty for the
+    launches of a few hundred microseconds): milliseconds per collective (HIP events),
     GB/s on the collective's minimum bytes (which is what each of them executes) and that as a fraction of
     the HBM peak."""
     out = {}
     for w in ("c2_reduce_scatter", "c2_all_gather", "c3_max_int32", "c3_min_int64", "c5_all_to_all", "c5_sum_int8"):
-        r = time_workload(w, torch, mr, 20, 5, layout)
+        # launches of a few hundred microseconds get more steps: twenty of them are over before the clocks have settled
+        steps, warmup = (20, 5) if w.startswith("c3") else (100, 50)
+        r = time_workload(w, torch, mr, steps, warmup, layout)
         out[w] = {"workload": r["workload"], "ms": round(r["kernel_ms"] * r["launches"], 4),
                   "gbps": round(r["achieved"], 1), "frac": round(r["achieved"] / HBM_PEAK_GBPS, 4),
                   "bytes_min": r["bytes"], "traffic": r["traffic"]}

@@ -324,7 +324,10 @@ class CollectivePlan:
             self._h = ctypes.c_void_p()
 
     def __del__(self):
-        self.close()
+        try:
+            self.close()
+        except Exception:  # at interpreter shutdown the modules this needs may be gone already
+            pass
 
 
 # ---------------------------------------------------------------------------------------------
@@ -376,7 +379,10 @@ class Client:
             self._h = ctypes.c_void_p()
 
     def __del__(self):
-        self.close()
+        try:
+            self.close()
+        except Exception:  # at interpreter shutdown the modules this needs may be gone already
+            pass
 
 
 class Communicator:
@@ -454,7 +460,10 @@ class Communicator:
             self._h = ctypes.c_void_p()
 
     def __del__(self):
-        self.close()
+        try:
+            self.close()
+        except Exception:  # at interpreter shutdown the modules this needs may be gone already
+            pass
 
 
 def get_communicator(nranks, rank, backend=Backend.VRANK):
