@@ -135,6 +135,12 @@ constexpr uint32_t kFlatOneOutMinTiles = 8192;
 constexpr uint32_t flat_one_out_waves_per_cu(uint32_t nranks) {
     return nranks >= 8 ? 8u : nranks == 4 ? 13u : 14u;
 }
+// The tree kernel (reduce towards a root for rank counts the flat kernels do not have) walks its tree depth first with
+// a few loads in flight per wavefront, and likes 16 wavefronts per CU for elements of 4 and 8 bytes from 64 MiB per buffer
+// on (fp32: 5 / 7 / 12 / 16 ranks 80 / 80 / 77 / 77 -> 86 / 87 / 81 / 81 % of the HBM peak, int64 and fp64 79 -> 84 - 85; at 32 MiB
+// level, below that behind); elements of 1 and 2 bytes spend longer on their conversions and lose 10 points to any cap.
+constexpr uint32_t kTreeCapMinTiles = 65536;
+constexpr uint32_t kTreeCapWavesPerCu = 16;
 constexpr bool flat_one_out(uint32_t nranks, uint32_t nout, uint64_t total_tiles) {
     return nout == 1 && nranks >= 3 && total_tiles >= kFlatOneOutMinTiles;
 }

@@ -252,3 +252,22 @@ def test_long_ragged_launch():
     torch.cuda.synchronize()
     for r in range(nranks):
         assert torch.equal(want, ins[r]), f"in place, rank {r}"
+
+
+def test_tree_reduce_of_five_ranks_at_the_reduced_occupancy():
+    """reduce towards a root for a rank count the flat kernels do not have, 4-byte elements, 64 MiB and more per buffer:
+    the tree kernel launched with LDS reserved per workgroup (16 wavefronts per CU), ragged length, checked in full
+    against the oracle's literal replay of the reference's binomial tree (src/ucx/reduce.cpp:56-80)."""
+    nranks, root = 5, 3
+    n = 65600 * 256 + 3  # fp32 elements: 65600 tiles of 16-byte vectors and three elements behind them
+    ins = [gen(n, torch.float32, r) for r in range(nranks)]
+    out = torch.full((n + 16,), 7.0, dtype=torch.float32, device=DEV)
+    runs, _, _ = mr.describe(mr.Collective.REDUCE, ins, [out] * nranks, n, mr.DType.FLOAT32, root=root)
+    assert runs and sum(r["tiles"] for r in runs) >= 65536 and all(r["waves"] == 1 for r in runs)
+    mr.reduce_to_root(ins, out, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, root)
+    torch.cuda.synchronize()
+    host = [t.cpu().numpy() for t in ins]
+    want = orc.ucx_reduce(host, orc.FLOAT32, orc.SUM, root)[root]
+    got = out.cpu().numpy()
+    assert np.array_equal(got[:n].view(np.uint32), want.view(np.uint32))
+    assert np.all(got[n:] == 7.0), "written past the end"
