@@ -159,10 +159,14 @@ private:
         bool unshifted = true;
         for (const Run& r : m_runs) unshifted = unshifted && r.in_begin == r.out_begin;
         // tiles that do not sit on the cache lines of every buffer share lines with their neighbours
-        bool on_lines = lines_shared(0) && m_misalign % 128 == 0;  // flat tiles start at the buffers' first byte
+        const bool base_on_lines = lines_shared(0) && m_misalign % 128 == 0;  // flat tiles start at the buffers' first byte
+        bool on_lines = base_on_lines;
         for (const Run& r : m_runs) on_lines = on_lines && lines_shared((r.in_begin - r.out_begin) * m_elem);
-        // (large one-output folds on line boundaries stay at one wavefront per tile, see flat_one_out)
-        const bool one_wave = total < kFlatGroupMinTiles || (on_lines && flat_one_out(m_nranks, m_nout, total));
+        // (large one-output folds whose INPUT tiles sit on line boundaries stay at one wavefront per tile, see
+        // flat_one_out; the one output in nine streams may be shifted by a part of a line - a receive length that is no
+        // multiple of 128 bytes: 82 - 84 % of the HBM peak against 79 - 80 in the group form - but with every buffer
+        // off the lines the group form, which deals its workgroups to the XCDs, is 8 points ahead)
+        const bool one_wave = total < kFlatGroupMinTiles || (base_on_lines && flat_one_out(m_nranks, m_nout, total));
         L.waves = one_wave ? 1 : kGroupWaves;
         L.exchange = (L.waves == kGroupWaves && !m_tree && m_nout == m_nranks && unshifted) ? 1 : 0;
         if (L.waves == kGroupWaves && !on_lines) L.exchange |= 2u;

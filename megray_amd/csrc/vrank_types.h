@@ -118,7 +118,7 @@ constexpr uint32_t kGroupStride = 32;
 constexpr uint32_t kGroupMinTiles = 512;
 constexpr uint32_t kFlatGroupMinTiles = 2048;
 // Large flat folds with ONE output (reduce_scatter, reduce, the first launch of the two-phase all_reduce), three
-// or more inputs and tiles on cache-line boundaries stay at one wavefront per tile and run at a reduced occupancy
+// or more inputs and input tiles on cache-line boundaries stay at one wavefront per tile and run at a reduced occupancy
 // instead: a wavefront has its K loads of 1 KiB in flight at once, and what HBM needs to stay busy (bandwidth x
 // latency, 32 - 64 KiB per CU) is in flight with far fewer wavefronts than a CU can hold - the rest only queue up
 // in the memory system and get in each other's way.  The occupancy is set by LDS reserved per workgroup at launch,

@@ -275,6 +275,11 @@ def test_full_size_plan_shapes():
     assert tree and all(r["waves"] == 1 and r["dir"] == 0 for r in tree)
     two_phase, _, _ = mr.describe(mr.Collective.ALL_REDUCE, sp, rp, 1 << 24, orc.FLOAT32, schedule=mr.Schedule.TWO_PHASE)
     assert {r["waves"] for r in two_phase if r["step"] == 0 and r["nfold"] == 8} == {1}
+    shifted, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, sp, rp, (1 << 22) - 4, orc.FLOAT32)  # outputs off the lines
+    assert shifted and all(r["waves"] == 1 and r["vector"] == 2 for r in shifted)
+    off = [p + 16 for p in sp]  # inputs off the lines: the group form, which deals workgroups to XCDs
+    moved, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, off, [p + 16 for p in rp], 1 << 22, orc.FLOAT32)
+    assert moved and all(r["waves"] == 4 and r["deal"] == 1 for r in moved)
     pair, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, sp[:2], rp[:2], 1 << 24, orc.FLOAT32, nranks=2)
     assert pair and all(r["waves"] == 4 for r in pair)
     for coll, count in ((mr.Collective.ALL_REDUCE, 1 << 15), (mr.Collective.REDUCE_SCATTER, 1 << 12),
@@ -403,8 +408,9 @@ def test_runs_whose_tiles_share_cache_lines_are_dealt_to_xcds():
     runs = vector_runs(mr.Collective.ALL_REDUCE, five_s, five_r, 5 * (1 << 20), mr.DType.FLOAT32)
     assert runs and all(r["vector"] == 1 and r["deal"] == 0 for r in runs)
     # a receive length off the line grid shifts the outputs against the inputs
+    # (the last case is a flat launch, kept below the size from which one-output folds leave the group form)
     for dtype, recvlen in ((mr.DType.FLOAT32, big // nranks - 1), (mr.DType.FLOAT16, big // nranks - 3),
-                           (mr.DType.FLOAT32, big // nranks - 4)):
+                           (mr.DType.FLOAT32, (1 << 20) // nranks - 4)):
         runs = vector_runs(mr.Collective.REDUCE_SCATTER, send, recv, recvlen, dtype)
         dealt = [r for r in runs if r["out_first"] != 0]  # rank 0's block starts where its output does
         assert dealt and all(r["deal"] == 1 for r in dealt)
