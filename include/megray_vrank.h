@@ -232,6 +232,23 @@ MRV_API int mrv_comm_create(uint32_t nranks, uint32_t rank, int backend, mrv_com
 MRV_API void mrv_comm_destroy(mrv_comm* comm);
 /* Communicator::init(master_ip, port) (src/core/communicator.cpp:17-21). */
 MRV_API int mrv_comm_init(mrv_comm* comm, const char* master_ip, int port);
+/*
+ * Communicator::init(BcastCallback) (include/megray/communicator.h:49, src/core/communicator.cpp:23-25): the group
+ * is formed through a broadcast the CALLER supplies instead of the bootstrap server, the way the reference's NCCL
+ * backend hands its unique id to one (src/nccl/communicator.cpp:54-64).  Every rank calls this from its own thread;
+ * `broadcast(data, len, user)` must leave rank 0's `len` bytes of `data` in every rank's `data` before it returns
+ * (rank 0 passes its own bytes in, the others receive).  `len` is 16 for this backend (the group's id).
+ */
+typedef void (*mrv_bcast_fn)(char* data, size_t len, void* user);
+MRV_API int mrv_comm_init_callback(mrv_comm* comm, mrv_bcast_fn broadcast, void* user);
+/*
+ * No counterpart in the reference (whose ranks block the host at every step and cannot run ahead of a peer).
+ * Here a rank's stream waits for its peers' streams on the device, and such a wait gives up after
+ * MEGRAY_VRANK_WAIT_LIMIT_MS (default 10 000).  A wait that gives up poisons its group: the kernels behind it
+ * store nothing, and every later call of the group returns MEGRAY_UNEXPECTED_ERR.  This call asks now: it waits
+ * for `stream`, reads the group's counters back and returns MEGRAY_OK or, for good, MEGRAY_UNEXPECTED_ERR.
+ */
+MRV_API int mrv_comm_check(mrv_comm* comm, void* stream);
 /* Fold order / schedule of this rank's communicator (MRV_ORDER_*, MRV_SCHED_*); no reference counterpart. */
 MRV_API int mrv_comm_configure(mrv_comm* comm, int order, int schedule);
 
@@ -262,11 +279,16 @@ MRV_API int mrv_comm_all_reduce(mrv_comm* comm, const void* sendbuff, void* recv
  * communicator group.  It calls no hipMalloc / hipFree / hipHostMalloc / hipEventCreate.
  *   - at most 32 groups per process can use it at the same time; the 33rd gets
  *     MEGRAY_INVALID_USAGE ("every counter block of the static array is in use") on every rank;
- *   - a group's first call clears its block (one synchronous 64-byte hipMemset): a block keeps what
+ *   - a group's first call clears its block (a 64-byte fill on the null stream, waited for): a block keeps what
  *     the last group that held it left there;
  *   - every rank of a group must make this same call (mixing it with mrv_comm_all_reduce in one
  *     collective is rejected like any other mismatch); a group's collectives follow one another, so
- *     its block is never used by two calls at once, and groups do not share blocks.
+ *     its block is never used by two calls at once, and groups do not share blocks;
+ *   - a stream wait that gives up (see mrv_comm_check) stops the kernels behind it from storing, as everywhere;
+ *     but with no pinned host word to report to, the host finds out by reading the block back: a synchronous
+ *     64-byte copy behind `stream` once half the wait limit has passed since the last one (never under stream
+ *     capture), so the first call that fails comes up to one and a half limits after the wait gave up, not at
+ *     the very next call; mrv_comm_check and the group's teardown read it as well.
  */
 MRV_API int mrv_comm_all_reduce_no_alloc(mrv_comm* comm, const void* sendbuff, void* recvbuff, size_t len,
                                          int dtype, int op, void* stream);

@@ -22,6 +22,9 @@ class PlanRun(ctypes.Structure):
     ]
 
 
+# void (*mrv_bcast_fn)(char* data, size_t len, void* user)
+BCAST_FN = ctypes.CFUNCTYPE(None, ctypes.POINTER(ctypes.c_char), ctypes.c_size_t, ctypes.c_void_p)
+
 _lib = None
 
 
@@ -76,6 +79,8 @@ def load():
     L.mrv_comm_destroy.argtypes = [vp]
     L.mrv_comm_destroy.restype = None
     L.mrv_comm_init.argtypes = [vp, ctypes.c_char_p, i32]
+    L.mrv_comm_init_callback.argtypes = [vp, BCAST_FN, vp]
+    L.mrv_comm_check.argtypes = [vp, vp]
     L.mrv_comm_configure.argtypes = [vp, i32, i32]
     L.mrv_comm_send.argtypes = [vp, vp, sz, i32, u32, vp]
     L.mrv_comm_recv.argtypes = [vp, vp, sz, i32, u32, vp]
@@ -98,7 +103,7 @@ def load():
     L.mrv_client_broadcast.argtypes = [vp, vp, vp, sz, u32]
     L.mrv_client_allgather.argtypes = [vp, vp, vp, sz]
     for name in ("mrv_reduce_to_root", "mrv_get_free_port", "mrv_create_server", "mrv_comm_create",
-                 "mrv_comm_init", "mrv_comm_configure", "mrv_comm_send", "mrv_comm_recv", "mrv_comm_scatter",
+                 "mrv_comm_init", "mrv_comm_init_callback", "mrv_comm_check", "mrv_comm_configure", "mrv_comm_send", "mrv_comm_recv", "mrv_comm_scatter",
                  "mrv_comm_gather", "mrv_comm_all_to_all", "mrv_comm_all_gather", "mrv_comm_all_reduce",
                  "mrv_comm_all_reduce_no_alloc",
                  "mrv_comm_reduce_scatter", "mrv_comm_broadcast", "mrv_comm_reduce", "mrv_comm_group_start",

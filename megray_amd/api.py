@@ -401,6 +401,23 @@ class Communicator:
     def init(self, master_ip, port):
         _check(_lib.load().mrv_comm_init(self._h, master_ip.encode(), port))
 
+    def init_callback(self, broadcast):
+        """Communicator::init(BcastCallback) (include/megray/communicator.h:49): form the group through the
+        caller's own broadcast instead of the bootstrap server.  `broadcast(data: bytearray) -> bytes-like` is
+        called once on this rank's thread with this rank's bytes (meaningful on rank 0 only) and returns rank 0's."""
+        def trampoline(data, length, _user):
+            mine = ctypes.string_at(data, length)
+            got = bytes(broadcast(bytearray(mine)))
+            if len(got) != length:
+                raise ValueError(f"the broadcast returned {len(got)} bytes, {length} were handed in")
+            ctypes.memmove(data, got, length)
+        fn = _lib.BCAST_FN(trampoline)
+        _check(_lib.load().mrv_comm_init_callback(self._h, fn, None))
+
+    def check(self, stream=None):
+        """Raises if a stream wait of this rank's group has given up (mrv_comm_check; synchronous)."""
+        _check(_lib.load().mrv_comm_check(self._h, _stream(stream)))
+
     def configure(self, order=FoldOrder.UCX, schedule=Schedule.FUSED):
         _check(_lib.load().mrv_comm_configure(self._h, int(order), int(schedule)))
 

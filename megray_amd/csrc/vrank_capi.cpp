@@ -481,8 +481,8 @@ int mrv_probe_bounded_wait(uint64_t limit_us, void* stream, uint64_t* gave_up) {
         Status st = MEGRAY_OK;
         EdgeWords host{};
         // nothing ever counts itself in: the wait can only end by giving up
-        if (hipMemset(words, 0, sizeof(EdgeWords)) != hipSuccess ||
-            edge_wait_arrived(words, 1, limit_us * uint64_t(khz) / 1000, nullptr, as_stream(stream)) != hipSuccess ||
+        if (hipMemsetAsync(words, 0, sizeof(EdgeWords), as_stream(stream)) != hipSuccess ||
+            edge_wait_arrived(words, words, 1, limit_us * uint64_t(khz) / 1000, nullptr, as_stream(stream)) != hipSuccess ||
             hipStreamSynchronize(as_stream(stream)) != hipSuccess ||
             hipMemcpy(&host, words, sizeof(host), hipMemcpyDeviceToHost) != hipSuccess) {
             (void)hipGetLastError();
@@ -564,6 +564,23 @@ int mrv_comm_init(mrv_comm* comm, const char* master_ip, int port) {
         need(comm, "comm is null");
         need(master_ip, "master_ip is null");
         return comm->comm->init(master_ip, port);
+    });
+}
+
+int mrv_comm_init_callback(mrv_comm* comm, mrv_bcast_fn broadcast, void* user) {
+    return guarded([&] {
+        need(comm, "comm is null");
+        need(reinterpret_cast<const void*>(broadcast), "broadcast is null");
+        return comm->comm->init([broadcast, user](char* data, size_t len) { broadcast(data, len, user); });
+    });
+}
+
+int mrv_comm_check(mrv_comm* comm, void* stream) {
+    return guarded([&] {
+        need(comm, "comm is null");
+        auto* vr = dynamic_cast<VRankCommunicator*>(comm->comm.get());
+        if (!vr) MEGRAY_THROW("not a vrank communicator");
+        return vr->check(HipContext::make(as_stream(stream)));
     });
 }
 

@@ -106,6 +106,15 @@ struct CachedCopy {
     std::vector<KernelCall> calls;  // point into `plan`
 };
 
+// Zeroes counters in device memory and returns when they ARE zero.  (hipMemset on device memory may return before
+// the fill has run, and streams created non-blocking are not ordered behind the null stream it runs on: a rank's
+// first arrive kernel could otherwise be wiped out by the clear that was meant to precede it.)
+hipError_t clear_words(void* words, size_t bytes) {
+    hipError_t err = hipMemsetAsync(words, 0, bytes, nullptr);
+    if (err == hipSuccess) err = hipStreamSynchronize(nullptr);
+    return err;
+}
+
 uint64_t env_u64(const char* name, uint64_t fallback) {
     const char* text = std::getenv(name);
     if (!text || !*text) return fallback;
@@ -136,8 +145,22 @@ public:
               m_mail(size_t(nranks) * nranks) {}
 
     ~Group() {
+        // The counters belong to the device the group worked on, which need not be the one current in the thread
+        // that lets go of the last rank object (a finaliser thread, interpreter shutdown): switch to it for the
+        // synchronisation and the frees, and back afterwards.
+        int before = -1;
+        const bool switched = m_device >= 0 && hipGetDevice(&before) == hipSuccess && before != m_device &&
+                              hipSetDevice(m_device) == hipSuccess;
+        bool drained = true;
         // wait kernels of the last collectives may still be polling the counters
-        if (m_edges[0].words || m_edges[1].words) (void)hipDeviceSynchronize();
+        if (m_edges[0].words || m_edges[1].words) drained = hipDeviceSynchronize() == hipSuccess;
+        if (drained && m_edges[1].words && !m_dead.load(std::memory_order_relaxed)) {
+            uint64_t timeouts = 0, at = 0;
+            if (edge_read_timeouts(m_edges[1].words, nullptr, &timeouts, &at) == hipSuccess && timeouts)
+                MEGRAY_ERROR("a communicator group is torn down whose stream waits gave up (%llu of them, the first "
+                             "waiting for %llu): results after that point were not written",
+                             static_cast<unsigned long long>(timeouts), static_cast<unsigned long long>(at));
+        }
         for (hipEvent_t ev : m_events) (void)hipEventDestroy(ev);
         for (hipEvent_t ev : m_arrive)
             if (ev) (void)hipEventDestroy(ev);
@@ -145,7 +168,10 @@ public:
         if (m_edges[0].words) (void)hipFree(m_edges[0].words);
         if (m_p2p_words) (void)hipFree(m_p2p_words);
         if (m_edges[0].status) (void)hipHostFree(m_edges[0].status);
-        give_back_static_slot(m_fixed_slot);
+        // a block some kernel may still be polling is not handed to another group
+        if (drained) give_back_static_slot(m_fixed_slot);
+        (void)hipGetLastError();
+        if (switched) (void)hipSetDevice(before);
     }
 
     // Groups are found by the 128-bit id rank 0 drew and the bootstrap broadcast.
@@ -213,7 +239,8 @@ public:
         theirs.pop_front();
         PendingP2P& s = op->is_send ? *op : *other;
         PendingP2P& r = op->is_send ? *other : *op;
-        Status st = transfer(s, r, size_t(src_rank) * m_nranks + dst_rank);
+        Status st = check_alive(m_edges[0], r.stream);
+        if (st == MEGRAY_OK) st = transfer(s, r, size_t(src_rank) * m_nranks + dst_rank);
         s.status = r.status = st;
         s.done = r.done = true;
         m_cv.notify_all();
@@ -225,7 +252,27 @@ public:
         return op->status;
     }
 
+    // Reads the counters back now (after `stream` has drained): has any stream wait of the group given up?
+    Status check(hipStream_t stream) {
+        for (EdgeSet& set : m_edges) {
+            if (m_dead.load(std::memory_order_acquire) || !set.words) continue;
+            uint64_t gave_up = 0, at = 0;
+            HIP_CHECK(edge_read_timeouts(set.words, stream, &gave_up, &at));
+            if (gave_up) declare_dead(at);
+        }
+        if (!m_dead.load(std::memory_order_acquire)) return MEGRAY_OK;
+        set_plan_error(m_dead_text);
+        return MEGRAY_UNEXPECTED_ERR;
+    }
+
 private:
+    // Counters of the edge kernels.  [0]: allocated at the first collective (null: the events below are
+    // used instead).  [1]: a block of the library's static device array, for the allocation-free entry point.
+    struct EdgeSet {
+        EdgeWords* words = nullptr;
+        uint64_t* status = nullptr;  // pinned host memory: [0] waits that gave up, [1] what the last one waited for
+        std::atomic<uint64_t> marks{0};  // arrive kernels enqueued so far = value `arrived` reaches when all have run
+    };
     struct Mailbox {
         std::deque<std::shared_ptr<PendingP2P>> sends, recvs;
     };
@@ -343,7 +390,9 @@ private:
         }
         // a wait gives up after this long (wall-clock ticks): long enough for any stream to drain,
         // short enough that a lost mark does not hold a wavefront for ever
-        m_limit_ticks = env_u64("MEGRAY_VRANK_WAIT_LIMIT_MS", 10000) * uint64_t(khz);
+        const uint64_t ms = env_u64("MEGRAY_VRANK_WAIT_LIMIT_MS", 10000);
+        m_limit_ms.store(ms, std::memory_order_relaxed);
+        m_limit_ticks = ms * uint64_t(khz);
         return true;
     }
 
@@ -355,15 +404,16 @@ private:
             uint64_t* status = nullptr;
             bool ok = wait_limit();
             ok = ok && hipMalloc(reinterpret_cast<void**>(&words), sizeof(EdgeWords)) == hipSuccess;
-            ok = ok && hipMemset(words, 0, sizeof(EdgeWords)) == hipSuccess;
-            ok = ok && hipHostMalloc(reinterpret_cast<void**>(&status), sizeof(uint64_t), hipHostMallocDefault) == hipSuccess;
+            ok = ok && clear_words(words, sizeof(EdgeWords)) == hipSuccess;
+            ok = ok && hipHostMalloc(reinterpret_cast<void**>(&status), 2 * sizeof(uint64_t), hipHostMallocDefault) == hipSuccess;
             if (!ok) {
                 (void)hipGetLastError();
                 if (words) (void)hipFree(words);
                 if (status) (void)hipHostFree(status);
                 return;
             }
-            *status = 0;
+            status[0] = status[1] = 0;
+            (void)hipGetDevice(&m_device);
             m_edges[0].status = status;
             m_edges[0].words = words;
         });
@@ -384,11 +434,14 @@ private:
             }
             EdgeWords* words = nullptr;
             if (edge_static_words(uint32_t(m_fixed_slot), &words) != hipSuccess ||
-                hipMemset(words, 0, sizeof(EdgeWords)) != hipSuccess) {
+                clear_words(words, sizeof(EdgeWords)) != hipSuccess) {
                 (void)hipGetLastError();
                 m_fixed_error = "the static counter array could not be reached on this device";
                 return;
             }
+            (void)hipGetDevice(&m_device);
+            m_fixed_checked = std::chrono::steady_clock::now();
+            m_fixed_period = std::chrono::milliseconds(m_limit_ms.load(std::memory_order_relaxed) / 2);
             m_edges[1].words = words;
         });
     }
@@ -416,7 +469,7 @@ private:
     Status await_done(hipStream_t stream, uint64_t ticket, bool fixed) {
         const EdgeSet& set = m_edges[fixed];
         if (set.words) {
-            HIP_CHECK(edge_wait_done(set.words, ticket, m_limit_ticks, set.status, stream));
+            HIP_CHECK(edge_wait_done(set.words, set.words, ticket, m_limit_ticks, set.status, stream));
             return MEGRAY_OK;
         }
         HIP_CHECK(hipStreamWaitEvent(stream, m_done, 0));
@@ -461,6 +514,63 @@ private:
         return false;
     }
 
+    // Tells a launch where the group's poison is (EdgeHooks::words; the wait / publish fields stay as they are).
+    void guard(Step& step, const EdgeSet& set) {
+        const EdgeHooks hooks{reinterpret_cast<uint64_t*>(set.words), set.status, m_limit_ticks};
+        switch (step.kind) {
+            case Step::kFlat:
+                step.flat.hooks = hooks;
+                step.flat.exchange = set.words ? step.flat.exchange | kFlatGuarded : step.flat.exchange & ~kFlatGuarded;
+                break;
+            case Step::kFold: step.fold.hooks = hooks; break;
+            case Step::kTree: step.tree.hooks = hooks; break;
+            case Step::kPack: step.pack.hooks = hooks; break;
+        }
+    }
+
+    // A stream wait of the group that gave up poisons the group for good: the kernels behind it store nothing
+    // (they test the poison in device memory), and from the moment the host knows, every call of the group -
+    // collective or transfer, on every rank - fails with MEGRAY_UNEXPECTED_ERR.  The host knows through the two
+    // words of pinned memory the waits report to; a group that only ever used the allocation-free entry point has
+    // none, and reads the poison back from its counter block instead: a wait cannot give up sooner than the limit
+    // after it was enqueued, so the block is read (a synchronous copy behind `stream`, not under stream capture)
+    // when half the limit has passed since the last read, and when the group is torn down.
+    Status check_alive(EdgeSet& set, hipStream_t stream) {
+        if (!m_dead.load(std::memory_order_acquire)) {
+            uint64_t gave_up = 0, at = 0;
+            if (set.status) {
+                gave_up = __atomic_load_n(&set.status[0], __ATOMIC_ACQUIRE);
+                at = set.status[1];
+            } else if (&set == &m_edges[1] && set.words && m_limit_ticks) {
+                const auto now = std::chrono::steady_clock::now();
+                if (now - m_fixed_checked >= m_fixed_period) {
+                    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+                    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) (void)hipGetLastError();
+                    if (capturing == hipStreamCaptureStatusNone) {
+                        m_fixed_checked = now;
+                        HIP_CHECK(edge_read_timeouts(set.words, stream, &gave_up, &at));
+                    }
+                }
+            }
+            if (!gave_up) return MEGRAY_OK;
+            declare_dead(at);
+        }
+        set_plan_error(m_dead_text);
+        return MEGRAY_UNEXPECTED_ERR;
+    }
+
+    void declare_dead(uint64_t at) {
+        std::lock_guard<std::mutex> lock(m_poison_mutex);
+        if (m_dead.load(std::memory_order_relaxed)) return;
+        std::snprintf(m_dead_text, sizeof(m_dead_text),
+                      "a stream wait of this group gave up after %llu ms (it was waiting for count / ticket %llu: a "
+                      "rank's stream did not get there in time); what followed it was not written, and the group "
+                      "takes no further calls",
+                      static_cast<unsigned long long>(m_limit_ms.load(std::memory_order_relaxed)),
+                      static_cast<unsigned long long>(at));
+        m_dead.store(true, std::memory_order_release);
+    }
+
     // Called by the last rank to arrive; every other rank is parked or has withdrawn.
     Status launch(uint32_t leader) {
         {
@@ -481,11 +591,7 @@ private:
             }
         }
         EdgeSet& set = m_edges[lead.fixed];
-        if (set.status && *set.status != set.status_seen) {
-            set.status_seen = *set.status;
-            set_plan_error("a stream wait of an earlier collective or transfer gave up: a rank's stream did not get there in time");
-            return MEGRAY_UNEXPECTED_ERR;
-        }
+        MEGRAY_CHECK(check_alive(set, lead.stream));
         const void* send[kMaxRanks] = {};
         void* recv[kMaxRanks] = {};
         for (uint32_t r = 0; r < m_nranks; ++r) {
@@ -537,6 +643,9 @@ private:
         m_shared_stream.store(static_cast<void*>(stream), std::memory_order_relaxed);
         m_shared_valid.store(one_stream, std::memory_order_release);
         const uint64_t ticket = m_generation.load(std::memory_order_relaxed) + 1;
+        // every launch of the group knows where the group's poison is (null while the group has no counters:
+        // without them nothing ever waits)
+        for (Step& step : cp->plan.steps) guard(step, set);
         // A single short launch of one wavefront per workgroup waits for the marks and publishes its
         // completion itself: two launches less on this thread, on which every rank is waiting.
         // (Only short launches: one of many tiles must not wait inside the kernel - workgroups that hold a
@@ -545,11 +654,10 @@ private:
         HookFields hooked;
         const bool hook = set.words && !one_stream && cp->plan.steps.size() == 1 && hook_fields(cp->plan.steps[0], hooked);
         if (hook) {
-            *hooked.hooks = EdgeHooks{reinterpret_cast<uint64_t*>(set.words), set.status, m_limit_ticks};
             *hooked.target = wait_needed ? set.marks.load(std::memory_order_relaxed) : 0;
             *hooked.ticket = ticket;
         } else if (wait_needed && set.words) {
-            HIP_CHECK(edge_wait_arrived(set.words, set.marks.load(std::memory_order_relaxed), m_limit_ticks, set.status, stream));
+            HIP_CHECK(edge_wait_arrived(set.words, set.words, set.marks.load(std::memory_order_relaxed), m_limit_ticks, set.status, stream));
         }
         for (const KernelCall& call : cp->calls) HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, stream, call.lds));
         // the other ranks order their streams behind this point themselves (none has to if all share the stream)
@@ -557,7 +665,7 @@ private:
             *hooked.target = *hooked.ticket = 0;
         } else if (!one_stream) {
             if (set.words) {
-                HIP_CHECK(edge_notify(set.words, ticket, stream));
+                HIP_CHECK(edge_notify(set.words, set.words, ticket, stream));
             } else {
                 if (!m_done) HIP_CHECK(hipEventCreateWithFlags(&m_done, hipEventDisableTiming));
                 HIP_CHECK(hipEventRecord(m_done, stream));
@@ -576,7 +684,7 @@ private:
             const size_t bytes = sizeof(EdgeWords) * 2 * m_mail.size();
             EdgeWords* words = nullptr;
             if (hipMalloc(reinterpret_cast<void**>(&words), bytes) != hipSuccess ||
-                hipMemset(words, 0, bytes) != hipSuccess) {
+                clear_words(words, bytes) != hipSuccess) {
                 (void)hipGetLastError();
                 if (words) (void)hipFree(words);
                 return;
@@ -615,6 +723,7 @@ private:
                 m_copy_next = (m_copy_next + 1) % kCopySlots;
             }
         }
+        for (Step& step : cc->plan.steps) guard(step, m_edges[0]);
         for (const KernelCall& call : cc->calls) HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, stream, call.lds));
         return MEGRAY_OK;
     }
@@ -637,11 +746,12 @@ private:
             EdgeWords* copied = reached + 1;
             const uint64_t ticket = ++m_p2p_seq[pair];
             uint64_t* status = m_edges[0].status;
-            HIP_CHECK(edge_notify(reached, ticket, s.stream));
-            HIP_CHECK(edge_wait_done(reached, ticket, m_limit_ticks, status, r.stream));
+            EdgeWords* group = m_edges[0].words;
+            HIP_CHECK(edge_notify(reached, group, ticket, s.stream));
+            HIP_CHECK(edge_wait_done(reached, group, ticket, m_limit_ticks, status, r.stream));
             MEGRAY_CHECK(copy_bytes(r.dst, s.src, s.size, r.stream));
-            HIP_CHECK(edge_notify(copied, ticket, r.stream));
-            HIP_CHECK(edge_wait_done(copied, ticket, m_limit_ticks, status, s.stream));
+            HIP_CHECK(edge_notify(copied, group, ticket, r.stream));
+            HIP_CHECK(edge_wait_done(copied, group, ticket, m_limit_ticks, status, s.stream));
             return MEGRAY_OK;
         }
         HIP_CHECK(hipEventRecord(event(0), s.stream));
@@ -673,19 +783,17 @@ private:
     std::atomic<void*> m_shared_stream{nullptr};  // the stream of the last collective, ...
     std::atomic<bool> m_shared_valid{false};      // ... if every rank passed that same one
     std::once_flag m_edges_once;
-    // Counters of the edge kernels.  [0]: allocated at the first collective (null: the events below are
-    // used instead).  [1]: a block of the library's static device array, for the allocation-free entry point.
-    struct EdgeSet {
-        EdgeWords* words = nullptr;
-        uint64_t* status = nullptr;  // host memory: waits that gave up
-        uint64_t status_seen = 0;
-        std::atomic<uint64_t> marks{0};  // arrive kernels enqueued so far = value `arrived` reaches when all have run
-    };
     EdgeSet m_edges[2];
     std::once_flag m_fixed_once;
     int m_fixed_slot = -1;
     const char* m_fixed_error = "";
     std::atomic<uint64_t> m_limit_ticks{0};
+    std::atomic<uint64_t> m_limit_ms{0};
+    int m_device = -1;                  // the device the counters live on
+    std::atomic<bool> m_dead{false};    // a stream wait gave up: the group takes no further calls
+    char m_dead_text[320] = "";
+    std::chrono::steady_clock::time_point m_fixed_checked{};  // when the static counter block was last read back
+    std::chrono::steady_clock::duration m_fixed_period{};
     std::atomic<uint32_t> m_sleepers{0};
     alignas(64) std::atomic<uint32_t> m_arrived{0};     // ranks that have deposited their call
     alignas(64) std::atomic<uint64_t> m_generation{0};  // collectives released so far; parked ranks poll it
@@ -830,6 +938,11 @@ Status VRankCommunicator::all_reduce(const void* sendbuff, void* recvbuff, size_
 Status VRankCommunicator::all_reduce_no_alloc(const void* sendbuff, void* recvbuff, size_t len, DType dtype,
                                               ReduceOp op, std::shared_ptr<Context> ctx) {
     VRANK_COLLECTIVE_ON(true, kCollAllReduce, len, dtype, op, 0, reduce_elem_size(dtype); check_reduce_op(op));
+}
+
+Status VRankCommunicator::check(std::shared_ptr<Context> ctx) {
+    MEGRAY_ASSERT(m_group != nullptr, "communicator used before init()");
+    return m_group->check(stream_of(ctx));
 }
 
 Status VRankCommunicator::reduce_scatter(const void* sendbuff, void* recvbuff, size_t recvlen, DType dtype,

@@ -51,6 +51,13 @@ public:
     // the same call.
     Status all_reduce_no_alloc(const void* src, void* dst, size_t count, DType dtype, ReduceOp op, ContextPtr ctx);
 
+    // Not part of the reference API: has a stream wait of this rank's group given up?  Synchronous: waits for the
+    // context's stream, reads the group's counters back, and returns MEGRAY_UNEXPECTED_ERR (for good) if one
+    // has.  Collectives report the same on their own - the call after the one that gave up, or, for a group
+    // that only ever used all_reduce_no_alloc (which has no host-visible word to report to), within one and a
+    // half wait limits; this asks now.
+    Status check(ContextPtr ctx);
+
     // Not part of the reference API: which reference loop's combination order all_reduce /
     // reduce_scatter / reduce reproduce (default: the ucx ring), and how all_reduce is laid out in
     // launches (default: fused).  Every rank of a group must choose the same.

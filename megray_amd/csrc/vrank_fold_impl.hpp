@@ -372,19 +372,38 @@ __device__ __forceinline__ void fold_vector_remainder(const FoldLaunch& L, const
 }
 
 // Every lane polls the same word (one request per wavefront) until it reaches `target` or the time
-// limit passes; each lane's acquire keeps its own loads behind the wait.
-__device__ __forceinline__ void hook_wait(const EdgeHooks& h, uint64_t target) {
+// limit passes; each lane's acquire keeps its own loads behind the wait.  false: the group is poisoned
+// (a wait gave up before, or this one does now) and the kernel must not store.
+__device__ __forceinline__ bool hook_wait(const EdgeHooks& h, uint64_t target) {
     const uint64_t begin = wall_clock64();
     while (__hip_atomic_load(h.words, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < target) {
+        if (__hip_atomic_load(h.words + 2, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT)) return false;
         if (wall_clock64() - begin > h.limit_ticks) {
             if (threadIdx.x == 0) {
-                __hip_atomic_fetch_add(h.words + 2, uint64_t(1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (h.status) __hip_atomic_fetch_add(h.status, uint64_t(1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                if (__hip_atomic_fetch_add(h.words + 2, uint64_t(1), __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == 0)
+                    __hip_atomic_store(h.words + 4, target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (h.status) {
+                    __hip_atomic_store(h.status + 1, target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    __hip_atomic_fetch_add(h.status, uint64_t(1), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+                }
             }
-            return;
+            return false;
         }
         __builtin_amdgcn_s_sleep(1);
     }
+    return __hip_atomic_load(h.words + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0;
+}
+
+// The poison of the group a launch belongs to (0 for launches outside a group).  Issued early, tested
+// before the first store: the load rides along with the tile loads and costs the kernel no round trip.
+__device__ __forceinline__ uint64_t hook_poison(const EdgeHooks& h) {
+    return h.words ? __hip_atomic_load(h.words + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : uint64_t(0);
+}
+
+// What the one-wavefront kernels do first: wait if the launch says so, and find out whether they may store.
+__device__ __forceinline__ bool hook_enter(const EdgeHooks& h, uint64_t target) {
+    if (target) return hook_wait(h, target);
+    return hook_poison(h) == 0;
 }
 
 // After a one-wavefront workgroup's stores: count it, and let the last one publish the ticket.
@@ -467,7 +486,7 @@ __device__ __forceinline__ void fold_tile(const FoldLaunch& L) {
 
 template <typename T, int OP, int K>
 __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
-    if (L.hook_target) hook_wait(L.hooks, L.hook_target);
+    if (!hook_enter(L.hooks, L.hook_target)) return;
     fold_tile<T, OP, K>(L);
     if (L.hook_ticket) hook_publish(L.hooks, L.hook_ticket);
 }
@@ -495,8 +514,11 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
     const uint32_t nfold = K > 0 ? uint32_t(K) : L.nfold;
     const uint32_t nout = L.nout;
     const bool new_wins = L.new_wins_ties != 0;
+    // A launch of a communicator group stores nothing once the group is poisoned (the test masks stores only: the
+    // wavefronts of a workgroup may see the poison rise at different moments and must all reach the barriers).
+    const bool live = hook_poison(L.hooks) == 0;
     if (!sv.vector) {
-        if (wave == 0) fold_element_tile<T, OP>(L, sv, nfold, sv.local_tile, tid);
+        if (wave == 0 && live) fold_element_tile<T, OP>(L, sv, nfold, sv.local_tile, tid);
         return;
     }
     const uint64_t nvec = sv.count / EPV;
@@ -555,11 +577,11 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
         }
     }
     // the segment's incomplete last group of vectors belongs to whoever owns its index
-    if (mine == whole_groups && nvec % kThreads)
+    if (mine == whole_groups && nvec % kThreads && live)
         fold_vector_remainder<T, OP>(L, sv, nfold, mine * kThreads, nvec % kThreads, tid);
 
     if (nout == 1) {
-        if (have)
+        if (have && live)
             store_tile_any(static_cast<char*>(L.out[sv.out_first]) + out_base + mine * kGroupBytes, tid, acc.finish());
         return;
     }
@@ -568,7 +590,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
     __syncthreads();
     for (uint32_t m = 0; m < nout; ++m) {
         const uint32_t k = (wave + m) % W;
-        if (folded[k])
+        if (folded[k] && live)
             store_tile_any(static_cast<char*>(L.out[rotate_rank(sv.out_first, 1, m, nr)]) + out_base +
                                    (first + uint64_t(k) * kGroupStride) * kGroupBytes,
                            tid, result[k][tid]);
@@ -699,7 +721,7 @@ __device__ __forceinline__ void tree_tile(const TreeLaunch& L) {
 
 template <typename T, int OP>
 __global__ void __launch_bounds__(kThreads) fold_tree_kernel(const TreeLaunch L) {
-    if (L.hook_target) hook_wait(L.hooks, L.hook_target);
+    if (!hook_enter(L.hooks, L.hook_target)) return;
     tree_tile<T, OP>(L);
     if (L.hook_ticket) hook_publish(L.hooks, L.hook_ticket);
 }
@@ -966,7 +988,9 @@ __device__ __forceinline__ void flat_tile(const FlatLaunch& L, uint32_t tile, ui
 // so that the tree's K live accumulators do not cost the left fold any registers.
 template <typename T, int OP, int K, bool TREE>
 __global__ void __launch_bounds__(kThreads) fold_flat_kernel(const FlatLaunch L) {
-    if (L.hook_target) hook_wait(L.hooks, L.hook_target);
+    if ((L.hook_target != 0) | ((L.exchange & kFlatGuarded) != 0)) {
+        if (!hook_enter(L.hooks, L.hook_target)) return;
+    }
     flat_tile<T, OP, K, TREE>(L, blockIdx.x, threadIdx.x);
     if (L.hook_ticket) hook_publish(L.hooks, L.hook_ticket);
 }
@@ -1013,6 +1037,9 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
         else
             x[r] = u32x4{0u, 0u, 0u, 0u};  // never folded: such a tile goes element by element
     }
+    // A launch of a communicator group stores nothing once the group is poisoned.  The wavefronts of a workgroup
+    // may see the poison rise at different moments, so it only ever masks stores and never skips a barrier.
+    const bool live = (L.exchange & kFlatGuarded) == 0 || hook_poison(L.hooks) == 0;
     // while the loads are in flight: which run does this wavefront's own tile lie in?
     TileRun tr;
     {
@@ -1039,11 +1066,13 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
         }
         if (exchange) {
             result[wave][tid] = res;
-        } else {
+        } else if (live) {
             const uint64_t out_off = uint64_t(mine) * (kThreads * kVecBytes) - out_shift * sizeof(T);
             for (uint32_t m = 0; m < L.nout; ++m)
                 store_tile_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, K)]) + out_off, tid, res);
         }
+    } else if (!live) {
+        // nothing is stored
     } else if ((uint64_t(mine) + 1) * TILE <= L.count) {
         // inside the buffers but across run borders: from the staged vectors, stored by this wavefront
         LaneRun lr;
@@ -1058,7 +1087,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
 #pragma unroll
         for (int m = 0; m < K; ++m) {
             const uint32_t k = (wave + m) % W;
-            if (folded[k]) {
+            if (folded[k] && live) {
                 const uint64_t tile = uint64_t(first) + k * kGroupStride;
                 store_tile_vec(static_cast<char*>(L.out[m]) + tile * (kThreads * kVecBytes), tid, result[k][tid]);
             }

@@ -4,8 +4,11 @@
 // src/ucx/scatter.cpp:30-44 and src/ucx/gather.cpp:30-44) and the plain copies of the fold kernel.
 #include "vrank_fold_impl.hpp"
 
+#include <cstring>
 #include <mutex>
 #include <unordered_map>
+
+#include "megray/debug.h"
 
 namespace MegRay {
 namespace vrank {
@@ -112,7 +115,7 @@ __device__ __forceinline__ void pack_vector_tile(const PackLaunch& L, const Pack
 
 // One wavefront per tile: short block copies.
 __global__ void __launch_bounds__(kThreads) pack_kernel(const PackLaunch L) {
-    if (L.hook_target) hook_wait(L.hooks, L.hook_target);
+    if (!hook_enter(L.hooks, L.hook_target)) return;
     const uint32_t copy = blockIdx.x / L.tiles_per_copy;
     const uint64_t tile = L.first_tile + (blockIdx.x - copy * L.tiles_per_copy);
     const PackEnds e = pack_ends(L, copy);
@@ -155,7 +158,9 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
         }
     }
     const uint64_t first = L.first_tile + uint64_t(group / kGroupStride) * (W * kGroupStride) + group % kGroupStride;
-    if (first == 0 && wave == 0) pack_edges(L, e, pv, src, dst_off, tid);
+    // A launch of a communicator group stores nothing once the group is poisoned (stores are masked, barriers kept).
+    const bool live = hook_poison(L.hooks) == 0;
+    if (first == 0 && wave == 0 && live) pack_edges(L, e, pv, src, dst_off, tid);
 
     // tile t holds vectors [t * kThreads - pad, ...): whole if all of them exist
     const uint64_t mine = first + wave * kGroupStride;
@@ -165,10 +170,10 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
     u32x4 x = {0u, 0u, 0u, 0u};
     if (whole)
         x = load_tile_any(src + tile_off(mine), tid);
-    else
+    else if (live)
         pack_vector_tile(L, e, pv, src, dst_off, mine, tid);  // a partial tile at either end: copied to every destination here
     if (e.ndst == 1) {
-        if (whole) store_tile_any(static_cast<char*>(L.out[e.dst_rank]) + dst_off + tile_off(mine), tid, x);
+        if (whole && live) store_tile_any(static_cast<char*>(L.out[e.dst_rank]) + dst_off + tile_off(mine), tid, x);
         return;
     }
     stage[wave][tid] = x;
@@ -176,7 +181,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
     __syncthreads();
     for (uint32_t m = 0; m < e.ndst; ++m) {
         const uint32_t k = (wave + m) % W;
-        if (staged[k])
+        if (staged[k] && live)
             store_tile_any(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + tile_off(first + uint64_t(k) * kGroupStride),
                             tid, stage[k][tid]);
     }
@@ -247,27 +252,77 @@ const void* pack_kernel_for(const PackLaunch& L) {
                                   : reinterpret_cast<const void*>(&pack_kernel);
 }
 
+namespace {
+
+// What the occupancy caps assume of the device in use, asked of the runtime once per device: the LDS a CU
+// holds, and whether the device is the part the caps were measured on (gfx950).  On any other part the
+// caps are left out (a launch at full occupancy is always correct, the cap is a tuning of MI355X).
+struct DeviceTraits {
+    bool known = false;
+    bool tuned = false;      // gfx950: the measured occupancy tables apply
+    uint32_t lds_per_cu = 0;
+};
+
+DeviceTraits device_traits() {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mutex;
+    static DeviceTraits traits[kMaxDevices];
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+        (void)hipGetLastError();
+        return {};
+    }
+    std::lock_guard<std::mutex> lock(mutex);
+    DeviceTraits& t = traits[device];
+    if (!t.known) {
+        hipDeviceProp_t prop;
+        int lds = 0;
+        if (hipGetDeviceProperties(&prop, device) != hipSuccess ||
+            hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, device) != hipSuccess) {
+            (void)hipGetLastError();
+            return {};
+        }
+        t.known = true;
+        t.tuned = std::strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+        t.lds_per_cu = lds > 0 ? uint32_t(lds) : 0;
+        if (!t.tuned)
+            MEGRAY_WARN("device %d is %s, not gfx950: launches keep their full occupancy (the caps were measured on MI355X)",
+                        device, prop.gcnArchName);
+    }
+    return t;
+}
+
+}  // namespace
+
 uint32_t lds_for_waves_per_cu(const void* kernel, uint32_t waves_per_cu) {
-    constexpr uint32_t kLdsPerCu = 160 * 1024;
     if (!kernel || !waves_per_cu) return 0;
+    const DeviceTraits traits = device_traits();
+    if (!traits.known || !traits.tuned || !traits.lds_per_cu) return 0;
     // what the kernel declares itself, asked of the runtime once per kernel
     static std::mutex mutex;
     static std::unordered_map<const void*, uint32_t> declared;
+    static bool complained = false;
     uint32_t own = 0;
     {
         std::lock_guard<std::mutex> lock(mutex);
         auto it = declared.find(kernel);
         if (it == declared.end()) {
             hipFuncAttributes attr;
-            if (hipFuncGetAttributes(&attr, kernel) != hipSuccess) {
+            const hipError_t err = hipFuncGetAttributes(&attr, kernel);
+            if (err != hipSuccess) {
                 (void)hipGetLastError();
+                if (!complained) {
+                    complained = true;
+                    MEGRAY_WARN("hipFuncGetAttributes failed (%s): large one-output folds run at full occupancy, "
+                                "a few points of the HBM peak slower", hipGetErrorString(err));
+                }
                 return 0;
             }
             it = declared.emplace(kernel, uint32_t(attr.sharedSizeBytes)).first;
         }
         own = it->second;
     }
-    const uint32_t each = kLdsPerCu / waves_per_cu / 1024 * 1024;  // whole KiB: allocation granules stay out of it
+    const uint32_t each = traits.lds_per_cu / waves_per_cu / 1024 * 1024;  // whole KiB: allocation granules stay out of it
     return each > own ? each - own : 0;
 }
 

@@ -35,12 +35,18 @@ struct FoldSegment {
 // Cross-stream ordering carried by a launch itself (thread-per-rank API, short launches of one wavefront
 // per workgroup): before it reads, every workgroup waits until `arrived` has reached the launch's
 // hook_target (the other ranks' streams have got to the collective); after its stores, the last workgroup
-// to finish publishes the launch's hook_ticket in `done`.  The four words are the group's counters in
+// to finish publishes the launch's hook_ticket in `done`.  The words are the group's counters in
 // device memory.  Every launch descriptor carries the three fields; 0 in hook_target / hook_ticket
 // (what the planner leaves there) means "do not wait" / "do not publish".
+//
+// `words`, where the communicator sets it (every launch it makes for a group, hooked or not), also tells the
+// kernel where the group's poison is: a stream wait of the group that gave up has raised words[2], and a
+// kernel that finds it raised returns before its first store - what it would combine was not ready.
+// Launches that do not come from a communicator group (the flat entry points) leave `words` null.
 struct EdgeHooks {
-    uint64_t* words;       // [0] arrived  [1] done  [2] timeouts  [3] workgroups finished
-    uint64_t* status;      // host-visible count of waits that gave up
+    uint64_t* words;       // [0] arrived  [1] done  [2] timeouts (not 0: poisoned)  [3] workgroups finished
+                           // [4] what the first wait that gave up was waiting for
+    uint64_t* status;      // host-visible: [0] waits that gave up, [1] what the last of them was waiting for
     uint64_t limit_ticks;  // a wait gives up after this many wall-clock ticks
 };
 
@@ -63,6 +69,8 @@ struct FoldLaunch {
     uint64_t hook_target;
     uint64_t hook_ticket;
 };
+
+constexpr uint32_t kFlatGuarded = 4;  // FlatLaunch::exchange
 
 constexpr uint32_t kMaxFlatRuns = 48;  // 2N chunks cut again at N-1 rank borders
 
@@ -99,7 +107,10 @@ struct FlatLaunch {
     uint32_t tree;  // 1: combine in binomial-tree order towards rank `start` instead of a left fold
     uint32_t waves;     // wavefronts per workgroup: 1, or kGroupWaves for the group form (launches of many tiles)
     uint32_t exchange;  // group form: bit 0 = every rank is an output at the inputs' offsets, results are exchanged too;
-                        // bit 1 = tiles share cache lines with their neighbours, deal runs of workgroups to XCDs
+                        // bit 1 = tiles share cache lines with their neighbours, deal runs of workgroups to XCDs;
+                        // either form: bit 2 (kFlatGuarded) = the launch belongs to a communicator group, hooks.words
+                        // is set and the group's poison is tested before anything is stored (the flag sits here, in
+                        // the line of scalars every wavefront reads anyway; `hooks` lies several cache lines further)
     uint32_t unshifted; // 1 = every run's outputs sit at the inputs' offsets (shift == 0 throughout)
     // run i covers elements [end[i - 1], end[i]) (from 0 for the first); unused entries are 0
     uint64_t end[kMaxFlatRuns];

@@ -18,7 +18,10 @@
 // that carry the ordering themselves, launches between wait and notify kernels, group launches), the
 // allocation-free entry point, the rooted collectives, rounds in which one rank's arguments are rejected, and rings of
 // send / recv.
-// Usage: stream_sim [rounds] [seed] [events]; prints "ok" or the first violation.
+// Usage: stream_sim [rounds] [seed] [events | fixed]; prints "ok" or the first violation.
+//   events: the ordering by event record / stream-wait-event instead of counters
+//   fixed:  every round is the allocation-free all_reduce, and no round may allocate (hipMalloc, hipHostMalloc,
+//           hipEventCreate are counted)
 #include <sys/mman.h>
 
 #include <atomic>
@@ -215,7 +218,7 @@ hipError_t edge_arrive(EdgeWords* words, hipStream_t stream) {
     return hipSuccess;
 }
 
-hipError_t edge_notify(EdgeWords* words, uint64_t ticket, hipStream_t stream) {
+hipError_t edge_notify(EdgeWords* words, EdgeWords*, uint64_t ticket, hipStream_t stream) {
     push(stream, [words, ticket]() {
         store_word(&words->done, ticket);
         return true;
@@ -223,13 +226,19 @@ hipError_t edge_notify(EdgeWords* words, uint64_t ticket, hipStream_t stream) {
     return hipSuccess;
 }
 
-hipError_t edge_wait_arrived(EdgeWords* words, uint64_t target, uint64_t, uint64_t*, hipStream_t stream) {
+hipError_t edge_wait_arrived(EdgeWords* words, EdgeWords*, uint64_t target, uint64_t, uint64_t*, hipStream_t stream) {
     push(stream, [words, target]() { return load_word(&words->arrived) >= target; });
     return hipSuccess;
 }
 
-hipError_t edge_wait_done(EdgeWords* words, uint64_t ticket, uint64_t, uint64_t*, hipStream_t stream) {
+hipError_t edge_wait_done(EdgeWords* words, EdgeWords*, uint64_t ticket, uint64_t, uint64_t*, hipStream_t stream) {
     push(stream, [words, ticket]() { return load_word(&words->done) >= ticket; });
+    return hipSuccess;
+}
+
+// simulated waits never give up
+hipError_t edge_read_timeouts(const EdgeWords*, hipStream_t, uint64_t* timeouts, uint64_t* gave_up_at) {
+    *timeouts = *gave_up_at = 0;
     return hipSuccess;
 }
 
@@ -253,9 +262,16 @@ hipError_t hipDeviceGetAttribute(int* value, hipDeviceAttribute_t, int) {
     *value = 100000;
     return hipSuccess;
 }
+hipError_t hipSetDevice(int) { return hipSuccess; }
+hipError_t hipStreamIsCapturing(hipStream_t, hipStreamCaptureStatus* status) {
+    *status = hipStreamCaptureStatusNone;
+    return hipSuccess;
+}
 hipError_t hipGetLastError(void) { return hipSuccess; }
 const char* hipGetErrorString(hipError_t) { return "simulated"; }
+std::atomic<int> g_allocations{0};  // hipMalloc, hipHostMalloc, hipEventCreate*: what the allocation-free path must not call
 hipError_t hipMalloc(void** p, size_t n) {
+    g_allocations.fetch_add(1);
     *p = std::calloc(1, n);
     return *p ? hipSuccess : hipErrorOutOfMemory;
 }
@@ -269,11 +285,17 @@ hipError_t hipMemset(void* p, int v, size_t n) {
     std::memset(p, v, n);
     return hipSuccess;
 }
+hipError_t hipMemsetAsync(void* p, int v, size_t n, hipStream_t) {
+    std::memset(p, v, n);  // only ever used on counters nothing else touches yet
+    return hipSuccess;
+}
+hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
 hipError_t hipDeviceSynchronize(void) {
     drain();
     return hipSuccess;
 }
 hipError_t hipEventCreateWithFlags(hipEvent_t* ev, unsigned) {
+    g_allocations.fetch_add(1);
     *ev = reinterpret_cast<hipEvent_t>(new SimEvent);
     return hipSuccess;
 }
@@ -353,6 +375,7 @@ int main(int argc, char** argv) {
     const int rounds = argc > 1 ? std::atoi(argv[1]) : 2000;
     const uint64_t seed = argc > 2 ? std::strtoull(argv[2], nullptr, 10) : 7;
     if (argc > 3 && std::strcmp(argv[3], "events") == 0) setenv("MEGRAY_VRANK_EDGES", "events", 1);
+    const bool only_fixed = argc > 3 && std::strcmp(argv[3], "fixed") == 0;
     std::mt19937_64 rng(seed);
     const uint32_t nranks = 2 + uint32_t(rng() % 7);
 
@@ -373,7 +396,11 @@ int main(int argc, char** argv) {
         r.root = uint32_t(rng() % nranks);
         r.len = lengths[rng() % 6];
         if (r.kind != 0) r.len = r.len / nranks + 1;
-        r.fixed = r.kind == 0 && rng() % 5 == 0;
+        if (only_fixed) {
+            r.kind = 0;
+            r.len = lengths[rng() % 6];
+        }
+        r.fixed = r.kind == 0 && (only_fixed || rng() % 5 == 0);
         r.poisoned = (r.kind == 0 && rng() % 10 == 0) ? int(rng() % nranks) : -1;
         r.stream.resize(nranks);
         const int mode = int(rng() % 3);
@@ -481,6 +508,7 @@ int main(int argc, char** argv) {
     g_stop.store(true);
     exec.join();
     if (failures.load()) return 1;
+    if (only_fixed && g_allocations.load()) violation("the allocation-free entry point allocated (hipMalloc, hipHostMalloc or hipEventCreate)");
     std::printf("ok %d rounds, %u ranks\n", rounds, nranks);
     return 0;
 }

@@ -11,7 +11,9 @@
 #include <cstdlib>
 #include <cstring>
 #include <functional>
+#include <condition_variable>
 #include <limits>
+#include <mutex>
 #include <string>
 #include <thread>
 #include <vector>
@@ -257,6 +259,54 @@ void test_all_reduce() {  // test/test_opr.cpp:286-359
     }
 }
 
+// Communicator::init(BcastCallback) (include/megray/communicator.h:49, src/core/communicator.cpp:23-25): the group is
+// formed through the caller's own broadcast - here a buffer in host memory that rank 0 fills and the others copy, the
+// way the reference's NCCL backend hands its unique id to the callback (src/nccl/communicator.cpp:54-64) - with no
+// bootstrap server anywhere; then an AllReduce as in test/test_opr.cpp:286-330.
+void test_init_with_callback() {
+    const int nranks = 4;
+    const size_t len = 1000;
+    std::vector<std::vector<float>> in(nranks, std::vector<float>(len)), out(nranks, std::vector<float>(len));
+    for (size_t j = 0; j < len; j++) {
+        float sum = 0;
+        for (int i = 0; i < nranks; i++) in[i][j] = 0.25f * float((i + 1) * (j % 97 + 1));
+        for (int i = 0; i < nranks; i++) sum += in[i][j];  // ranks 0..N-1; these values add exactly in any order
+        for (int i = 0; i < nranks; i++) out[i][j] = sum;
+    }
+    std::mutex m;
+    std::condition_variable cv;
+    std::vector<char> id;
+    std::vector<std::shared_ptr<Communicator>> comms(nranks);
+    std::vector<std::vector<float>> got(nranks, std::vector<float>(len));
+    for (int i = 0; i < nranks; i++) comms[i] = MegRay::get_communicator(nranks, i, MegRay::MEGRAY_VRANK);
+    std::vector<std::thread> threads;
+    for (int i = 0; i < nranks; i++)
+        threads.emplace_back([&, i] {
+            REQUIRE(hipSetDevice(0) == hipSuccess);
+            const MegRay::Status st = comms[i]->init([&, i](char* data, size_t bytes) {
+                std::unique_lock<std::mutex> lock(m);
+                if (i == 0) {
+                    id.assign(data, data + bytes);
+                    cv.notify_all();
+                } else {
+                    cv.wait(lock, [&] { return !id.empty(); });
+                    REQUIRE(id.size() == bytes);
+                    std::memcpy(data, id.data(), bytes);
+                }
+            });
+            REQUIRE(st == MegRay::MEGRAY_OK);
+            hipStream_t stream;
+            auto ctx = make_context(&stream);
+            void* in_ptr = upload(in[i]);
+            void* out_ptr = dev_alloc(len * sizeof(float));
+            REQUIRE(comms[i]->all_reduce(in_ptr, out_ptr, len, MegRay::MEGRAY_FLOAT32, MegRay::MEGRAY_SUM, ctx) == 0);
+            download(got[i], out_ptr, stream);
+        });
+    for (auto& t : threads) t.join();
+    for (int i = 0; i < nranks; i++) REQUIRE(std::memcmp(got[i].data(), out[i].data(), len * sizeof(float)) == 0);
+    std::printf("ok   InitCallback\n");
+}
+
 void test_reduce_scatter() {  // test/test_opr.cpp:361-438
     const int nranks = 3;
     const size_t recvlen = 10;
@@ -380,6 +430,7 @@ int main() {
         return 2;
     }
     test_init();
+    test_init_with_callback();
     test_send_recv();
     test_scatter_gather();
     test_all_to_all();

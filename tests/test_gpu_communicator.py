@@ -375,6 +375,136 @@ def test_a_stream_wait_that_nothing_satisfies_gives_up_at_its_limit():
         assert elapsed_us < limit_us + 500000, (limit_us, elapsed_us)
 
 
+def test_init_through_the_callers_own_broadcast():
+    """Communicator::init(BcastCallback) (include/megray/communicator.h:49, src/core/communicator.cpp:23-25): no
+    bootstrap server; the group is formed through a broadcast the caller supplies (here a slot in host memory that
+    rank 0 fills and the others wait for), the way the reference's NCCL backend passes its unique id through the
+    callback (src/nccl/communicator.cpp:54-64).  Then an all_reduce of seeded data against the oracle."""
+    nranks, n = 5, 4099
+    rng = np.random.default_rng(606)
+    data = [rand_array(orc.FLOAT32, n, rng, wide=False) for _ in range(nranks)]
+    want = orc.ucx_all_reduce(data, orc.FLOAT32, orc.SUM)
+    comms = [mr.get_communicator(nranks, r, mr.Backend.VRANK) for r in range(nranks)]
+    slot, filled = {}, threading.Event()
+    results, errors, seen = [None] * nranks, [], [None] * nranks
+
+    def rank_main(rank):
+        try:
+            torch.cuda.set_device(0)
+
+            def broadcast(mine):
+                if rank == 0:
+                    slot["id"] = bytes(mine)
+                    filled.set()
+                else:
+                    assert filled.wait(60), "rank 0 never broadcast"
+                seen[rank] = slot["id"]
+                return slot["id"]
+
+            comms[rank].init_callback(broadcast)
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                src, dst = to_device(data[rank]), empty_device(n * 4)
+                comms[rank].all_reduce(src, dst, n, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream)
+                stream.synchronize()
+                results[rank] = to_host(dst, np.float32)
+        except BaseException as exc:  # noqa: BLE001
+            errors.append((rank, repr(exc)))
+
+    threads = [threading.Thread(target=rank_main, args=(r,), daemon=True) for r in range(nranks)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(120)
+        assert not t.is_alive(), "a rank hung"
+    assert not errors, errors
+    assert len(seen[0]) == 16 and any(seen[0]) and all(s == seen[0] for s in seen)  # one 128-bit id, rank 0's
+    for r in range(nranks):
+        assert bits_equal(results[r], want[r])
+    for c in comms:
+        c.close()
+
+
+@pytest.mark.parametrize("entry", ["all_reduce", "all_reduce_no_alloc"])
+@pytest.mark.parametrize("length", [3000, 1 << 20])
+def test_a_stream_wait_that_gives_up_poisons_its_group(entry, length, monkeypatch):
+    """A rank whose stream does not get to the collective within the wait limit: forced from the host with a limit of
+    150 ms and a rank whose stream is kept busy with a second of its own work before the call.  Every kernel ends
+    normally.  What must hold: the collective that could not wait long enough stores NOTHING (its inputs were not
+    ready), the streams behind it are let go at once rather than each waiting out its own limit, and from then on
+    every call of the group fails with MEGRAY_UNEXPECTED_ERR and says why - at the very next call for groups whose
+    counters report to pinned host memory, after mrv_comm_check or within one and a half limits for a group that
+    only uses the allocation-free entry point.  The lengths take the short launch that waits inside the fold kernel
+    and the group launch between wait and notify kernels."""
+    import time
+    monkeypatch.setenv("MEGRAY_VRANK_WAIT_LIMIT_MS", "150")
+    nranks, fill = 2, 0x3C
+    rng = np.random.default_rng(length)
+    data = [rand_array(orc.FLOAT32, length, rng, wide=False) for _ in range(nranks)]
+    want = orc.ucx_all_reduce(data, orc.FLOAT32, orc.SUM)
+    port = mr.get_free_port()
+    mr.create_server(nranks, port)
+    comms = [mr.get_communicator(nranks, r, mr.Backend.VRANK) for r in range(nranks)]
+    ballast = torch.ones(1 << 28, dtype=torch.float32, device="cuda:0")  # 1 GiB: ~0.6 ms per pass over it
+    first, late, after, errors = [None] * nranks, [None] * nranks, [[] for _ in range(nranks)], []
+    barrier = threading.Barrier(nranks)
+
+    def rank_main(rank):
+        try:
+            torch.cuda.set_device(0)
+            comm = comms[rank]
+            comm.init("localhost", port)
+            call = getattr(comm, entry)
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                src = to_device(data[rank])
+                dst = empty_device(length * 4, fill=fill)
+                call(src, dst, length, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream)  # a healthy collective first
+                stream.synchronize()
+                first[rank] = to_host(dst, np.float32)
+                dst.fill_(fill)
+                stream.synchronize()
+                barrier.wait(60)
+                if rank == 1:  # about a second of work in front of this rank's call
+                    for _ in range(1500):
+                        ballast.mul_(1.0)
+                call(src, dst, length, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream)  # enqueued all the same: returns OK
+                t0 = time.perf_counter()
+                stream.synchronize()
+                waited = time.perf_counter() - t0
+                late[rank] = (to_host(dst, np.uint8).copy(), waited)
+                barrier.wait(60)
+                if entry == "all_reduce_no_alloc":
+                    with pytest.raises(mr.MegRayError) as info:
+                        comm.check(stream)
+                    after[rank].append((info.value.status, info.value.message))
+                for _ in range(2):  # and it stays that way
+                    with pytest.raises(mr.MegRayError) as info:
+                        call(src, dst, length, mr.DType.FLOAT32, mr.ReduceOp.SUM, stream)
+                    after[rank].append((info.value.status, info.value.message))
+                stream.synchronize()
+        except BaseException as exc:  # noqa: BLE001
+            errors.append((rank, repr(exc)))
+            barrier.abort()
+
+    threads = [threading.Thread(target=rank_main, args=(r,), daemon=True) for r in range(nranks)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(180)
+        assert not t.is_alive(), "a rank hung"
+    assert not errors, errors
+    for r in range(nranks):
+        assert bits_equal(first[r], want[r])
+        untouched, waited = late[r]
+        assert bool((untouched == fill).all()), f"rank {r}: the collective that could not wait stored something"
+        assert waited < 5.0, f"rank {r} waited {waited:.1f} s"
+        for status, message in after[r]:
+            assert status == mr.Status.UNEXPECTED_ERR and "gave up" in message, (status, message)
+    for c in comms:
+        c.close()
+
+
 @pytest.mark.parametrize("length", [3000, 70000, 100000, (1 << 19) + 11])
 def test_back_to_back_rounds_with_fresh_data_on_rank_streams(length):
     """Five all_reduces back to back, every round with different inputs that each rank copies into the SAME device

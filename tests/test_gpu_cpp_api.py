@@ -14,8 +14,9 @@ BIN = os.path.join(ROOT, "tests", "cpp", "test_vrank_opr")
 
 @pytest.mark.parametrize("edges", ["default", "events"])
 def test_cpp_api_thread_per_rank(edges):
-    """`edges`: how the ranks' streams are ordered against each other - stream memory operations where the
-    device has them (default), or events (MEGRAY_VRANK_EDGES=events, also the fallback)."""
+    """`edges`: how the ranks' streams are ordered against each other - one-wavefront arrive / wait / notify
+    kernels on counters in device memory (default), or events (MEGRAY_VRANK_EDGES=events, also the fallback
+    when the counters cannot be allocated)."""
     if not os.path.exists(BIN):
         from megray_amd import build
         build.build_cpp_test()
@@ -27,6 +28,6 @@ def test_cpp_api_thread_per_rank(edges):
     print(proc.stderr)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert "all passed" in proc.stdout
-    for case in ("Init", "SendRecv", "Scatter", "Gather", "AllToAll", "AllGather", "AllReduce op=0",
+    for case in ("Init", "InitCallback", "SendRecv", "Scatter", "Gather", "AllToAll", "AllGather", "AllReduce op=0",
                  "AllReduce op=1", "AllReduce op=2", "ReduceScatter op=0", "Broadcast", "Reduce op=0", "Errors"):
         assert f"ok   {case}" in proc.stdout

@@ -105,4 +105,4 @@ def test_ten_mib_row_agrees_with_an_event_timing(tmp_path):
     out = run_cli("-d", str(nranks), "-f", "all_reduce", "-s", str(nbytes), "-w", "100", "-i", "500")
     own = parse_tables(out)["all_reduce_sum"][1][0]
     print(f"performance tool, a stream per rank: {own[4]:.0f} GB/s ({own[1]:.1f} us per call)")
-    assert own[4] > 0.45 * event_gbps
+    assert own[4] > 0.6 * event_gbps

@@ -85,6 +85,43 @@ def test_no_alloc_all_reduce_matches_all_reduce_two_calls_in_a_row():
         c.close()
 
 
+def test_no_alloc_leaves_the_device_memory_as_it_finds_it():
+    """What the entry point is for: between a group's first call through it and its last, the free device memory
+    does not change (no hipMalloc, no hipFree).  Buffers are allocated and the kernels loaded (by another group)
+    beforehand; the calls take the short launch and the one between wait and notify kernels, a stream per rank.
+    (Host-side allocations the free-memory figure cannot see - pinned memory, events - are counted on the simulated
+    streams of tests/test_stream_sim.py, mode "fixed".)"""
+    nranks = 4
+    lengths = [777, (1 << 19) + 5]
+    rng = np.random.default_rng(99)
+    inputs = [[rng.integers(-1000, 1000, n).astype(np.int32) for _ in range(nranks)] for n in lengths]
+    warm, comms = make_group(nranks), make_group(nranks)
+    bufs = [[(to_device(inputs[i][r]), empty_device(n * 4)) for i, n in enumerate(lengths)] for r in range(nranks)]
+    streams = [torch.cuda.Stream() for _ in range(nranks)]
+    free = {}
+
+    def run(group, rank, rounds):
+        for _ in range(rounds):
+            for i, n in enumerate(lengths):
+                src, dst = bufs[rank][i]
+                group[rank].all_reduce_no_alloc(src, dst, n, mr.DType.INT32, mr.ReduceOp.SUM, streams[rank])
+        streams[rank].synchronize()
+
+    run_ranks(nranks, lambda rank: run(warm, rank, 1))
+    torch.cuda.synchronize()
+    free["before"] = torch.cuda.mem_get_info()[0]
+    run_ranks(nranks, lambda rank: run(comms, rank, 3))
+    torch.cuda.synchronize()
+    free["after"] = torch.cuda.mem_get_info()[0]
+    assert free["after"] == free["before"], free
+    for i, n in enumerate(lengths):
+        want = sum(x.astype(np.int64) for x in inputs[i]).astype(np.int32)
+        for r in range(nranks):
+            assert np.array_equal(to_host(bufs[r][i][1], np.int32), want)
+    for c in warm + comms:
+        c.close()
+
+
 def test_no_alloc_rejects_a_mixed_collective_and_runs_out_of_blocks_cleanly():
     nranks = 2
     groups = [make_group(nranks) for _ in range(33)]
