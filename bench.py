@@ -12,6 +12,8 @@ with all buffers already resident in HBM.  Prints ONE JSON line:
   comm_api_us   the same all_reduce at 4 KiB .. 1 MiB per rank through MegRay::Communicator::all_reduce,
              one thread per rank (the reference's test/performance.cpp:103-137 harness shape), every
              rank on a stream of its own and all ranks on one stream: microseconds per collective
+  comm_api_large  the headline shape through the same API and harness on random inputs: 8 ranks x 10 MiB / 128 MiB /
+             1 GiB, buffers each rank allocates itself or placed by the library, a stream per rank or one shared
   small_msg_us  the same sizes through the flat C ABI (one caller, one stream)
   other_configs the other benchmark configurations (reduce_scatter / all_gather fp16, MAX int32,
              MIN int64, all_to_all uint8, SUM int8), each timed with HIP events
@@ -70,7 +72,7 @@ def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--log2n", type=int, default=28, help="elements per rank = 2^log2n")
     ap.add_argument("--ranks", type=int, default=8)
     ap.add_argument("--schedule", default="fused", choices=["fused", "two_phase", "ring"])
@@ -96,12 +98,12 @@ LAYOUT_TEXT = {
 }
 
 
-def alloc_buffers(torch, mr, specs, layout):
+def alloc_buffers(torch, mr, specs, layout, collective=None, written=None):
     """Tensors for (numel, dtype) pairs in HBM.  "placed": views into one allocation at the distances the
-    library recommends for buffers that a collective walks through in step; "separate": one torch allocation
-    each, wherever the caching allocator puts them."""
+    library recommends for buffers that a collective walks through in step (`collective` and `written` tell it
+    what the buffers are for); "separate": one torch allocation each, wherever the caching allocator puts them."""
     if layout == "placed":
-        return mr.place_tensors(torch, specs, "cuda:0")
+        return mr.place_tensors(torch, specs, "cuda:0", collective, written)
     return [torch.empty(numel, dtype=dtype, device="cuda:0") for numel, dtype in specs]
 
 
@@ -218,9 +220,48 @@ def comm_api_sweep():
             if proc.returncode != 0:
                 raise SystemExit(f"bench: {' '.join(cmd)} failed:\n{proc.stdout}\n{proc.stderr}")
             rows = [json.loads(line) for line in tmp.read().splitlines() if line.strip()]
-        out[mode] = {str(r["bufsize"]): {"avg_us": round(r["avg_us"], 2), "median_us": round(r["median_us"], 2),
-                                          "p99_us": round(r["p99_us"], 2)} for r in rows}
+        keys = ("avg_us", "host_us", "median_us", "p90_us", "p99_us", "p999_us", "max_us")
+        out[mode] = {str(r["bufsize"]): dict({k: round(r[k], 2) for k in keys},
+                                             drain_ms=round(r["drain_us"] / 1e3, 2), sleeps=r["sleeps"]) for r in rows}
     out["harness"] = "megray_performance -d 8 -f all_reduce -w 200 -i 2000 (thread per rank, MegRay::Communicator API)"
+    out["columns"] = ("avg_us: wall time of the 2000 calls including the final stream sync, per call; host_us: the same "
+                      "without the final sync (what a call costs the calling thread); median / p90 / p99 / p999 / max: of "
+                      "the time between consecutive call returns on rank 0; drain_ms: the final sync (how far the device "
+                      "was behind); sleeps: times a rank slept on the condition variable while waiting for the others")
+    return out
+
+
+def comm_api_large():
+    """The headline shape through the drop-in boundary itself: MegRay::Communicator::all_reduce, one thread per rank
+    (the reference's harness, test/performance.cpp:85-137), inputs from the counter generator (-R), 8 ranks x
+    {10 MiB, 128 MiB, 1 GiB} fp32 SUM.  Four set-ups: buffers each rank allocates itself with hipMalloc (-M, what
+    test/performance.cpp:108-110 does) or laid out by the library in one allocation, and a stream per rank (as in
+    the reference) or one shared stream (-S).  Per size: microseconds per collective (wall clock of all timed calls
+    including the final sync), GB/s on the collective's minimum bytes 2 * N * bufsize, and that over the HBM peak.
+    Runs as child processes before this process touches the GPU."""
+    exe = os.path.join(ROOT, "megray_amd", "apps", "megray_performance")
+    if not os.path.exists(exe):
+        raise SystemExit("bench: megray_amd/apps/megray_performance is not built (python -m megray_amd.build)")
+    out = {}
+    for buffers, bflag in (("own_hipMalloc", ["-M"]), ("placed", [])):
+        for streams, sflag in (("own_streams", []), ("shared_stream", ["-S"])):
+            rows = []
+            for sizes, warm, iters in (("10485760", 100, 500), ("134217728,1073741824", 10, 30)):
+                with tempfile.NamedTemporaryFile("r", suffix=".jsonl") as tmp:
+                    cmd = [exe, "-d", "8", "-f", "all_reduce", "-s", sizes, "-w", str(warm), "-i", str(iters), "-R",
+                           "-J", tmp.name] + bflag + sflag
+                    proc = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+                    if proc.returncode != 0:
+                        raise SystemExit(f"bench: {' '.join(cmd)} failed:\n{proc.stdout}\n{proc.stderr}")
+                    rows += [json.loads(line) for line in tmp.read().splitlines() if line.strip()]
+            entry = {}
+            for r in rows:
+                gbps = 2 * 8 * r["bufsize"] / r["avg_us"] / 1e3
+                entry[str(r["bufsize"])] = {"avg_us": round(r["avg_us"], 2), "iters": r["iters"], "gbps": round(gbps, 1),
+                                            "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+            out[f"{buffers}/{streams}"] = entry
+    out["harness"] = ("megray_performance -d 8 -f all_reduce -R [-M] [-S]: thread per rank through "
+                      "MegRay::Communicator::all_reduce, random inputs, 100 + 500 calls at 10 MiB, 10 + 30 at 128 MiB and 1 GiB")
     return out
 
 
@@ -298,10 +339,11 @@ def time_workload(w, torch, mr, steps, warmup, layout="placed"):
     st = torch.cuda.current_stream()
     n8 = 8
 
-    def buffers(n_in, n_out, dtype, count_in=n8, count_out=n8):
+    def buffers(n_in, n_out, dtype, count_in=n8, count_out=n8, collective=None):
         """count_in inputs of n_in elements (filled) and count_out outputs of n_out elements."""
         from megray_amd import synth
-        bufs = alloc_buffers(torch, mr, [(n_in, dtype)] * count_in + [(n_out, dtype)] * count_out, layout)
+        bufs = alloc_buffers(torch, mr, [(n_in, dtype)] * count_in + [(n_out, dtype)] * count_out, layout, collective,
+                             [0] * count_in + [1] * count_out)
         for rank, t in enumerate(bufs[:count_in]):
             synth.fill_torch(dtype, n_in, rank, "normal" if dtype.is_floating_point else "uniform", device=dev, out=t)
         return bufs[:count_in], bufs[count_in:]
@@ -320,7 +362,7 @@ def time_workload(w, torch, mr, steps, warmup, layout="placed"):
         text, dt = "reduce_scatter SUM fp16 (fp32 accumulate), 8 ranks x 2^26 elements in, 2^23 out", "f16"
     elif w == "c2_all_gather":
         sendlen = 1 << 23
-        src, dst = buffers(sendlen, n8 * sendlen, torch.float16)
+        src, dst = buffers(sendlen, n8 * sendlen, torch.float16, collective=mr.Collective.ALL_GATHER)
         step = lambda: mr.all_gather(src, dst, sendlen, mr.DType.FLOAT16, stream=st)  # noqa: E731
         desc = (mr.Collective.ALL_GATHER, src, dst, sendlen, mr.DType.FLOAT16)
         text, dt = "all_gather fp16, 8 ranks x 2^23 elements in, 2^26 out", "f16"
@@ -412,6 +454,7 @@ def main():
     headline = args.workload == "all_reduce"
     # the thread-per-rank leg runs in a child process, before this process touches the GPU
     comm_api = comm_api_sweep() if headline and not args.no_comm else None
+    comm_large = comm_api_large() if headline and not args.no_comm and args.log2n == 28 else None
 
     import numpy as np
     import torch
@@ -504,9 +547,10 @@ def main():
     if not args.no_others:  # the same launches on buffers placed the other way, for the record
         other = "separate" if args.layout == "placed" else "placed"
         ins, outs = make_buffers(torch, mr, nranks, n, other)
-        _, other_ms = timed(ins, outs, 5, 2)
-        result["other_layout"] = {"layout": LAYOUT_TEXT[other], "ms_per_step": round(other_ms / 5, 4),
-                                  "pct_of_peak": round(100.0 * bmin / (other_ms / 5 * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2)}
+        _, other_ms = timed(ins, outs, args.steps, args.warmup)  # timed like the headline
+        result["other_layout"] = {"layout": LAYOUT_TEXT[other], "steps": args.steps, "warmup": args.warmup,
+                                  "ms_per_step": round(other_ms / args.steps, 4),
+                                  "pct_of_peak": round(100.0 * bmin / (other_ms / args.steps * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2)}
         del ins, outs
         torch.cuda.empty_cache()
     props = torch.cuda.get_device_properties(0)
@@ -517,6 +561,8 @@ def main():
         result["small_msg_us"] = small_message_sweep(torch, mr)
     if comm_api is not None:
         result["comm_api_us"] = comm_api
+    if comm_large is not None:
+        result["comm_api_large"] = comm_large
     if not args.no_others:
         result["other_configs"] = other_configs(torch, mr, args.layout)
     if not args.no_cpu:

@@ -249,6 +249,13 @@ MRV_API int mrv_comm_init_callback(mrv_comm* comm, mrv_bcast_fn broadcast, void*
  * for `stream`, reads the group's counters back and returns MEGRAY_OK or, for good, MEGRAY_UNEXPECTED_ERR.
  */
 MRV_API int mrv_comm_check(mrv_comm* comm, void* stream);
+/*
+ * Diagnostic, no counterpart in the reference: counts kept by this rank's group since it was formed (any pointer may
+ * be null).  *collectives: collectives launched; *plans_built: how many of them had to be planned rather than found in
+ * the group's plan cache; *sleeps: times a rank waiting for the others stopped polling and slept on a condition
+ * variable.
+ */
+MRV_API int mrv_comm_stats(mrv_comm* comm, uint64_t* collectives, uint64_t* plans_built, uint64_t* sleeps);
 /* Fold order / schedule of this rank's communicator (MRV_ORDER_*, MRV_SCHED_*); no reference counterpart. */
 MRV_API int mrv_comm_configure(mrv_comm* comm, int order, int schedule);
 
@@ -328,6 +335,19 @@ MRV_API int mrv_probe_bounded_wait(uint64_t limit_us, void* stream, uint64_t* ga
 MRV_API int mrv_rank_buffers_layout(int count, const size_t* bytes, size_t* offsets, size_t* total);
 MRV_API int mrv_rank_buffers_alloc(int count, const size_t* bytes, void** ptrs, void** base);
 MRV_API int mrv_rank_buffers_free(void* base);
+/*
+ * The same for callers that know what the buffers are for (no counterpart in the reference either).  The best
+ * distance depends on it: the buffers an all_gather stores every rank's block into (one read stream, N write
+ * streams) are served best a multiple of 128 MiB PLUS 32 MiB apart (all_gather of 8 x 16 MiB fp16: 79 % of the HBM
+ * peak with the outputs 128 MiB apart, 84 % at 160 MiB), where the folds and the pairwise copies lose one to two
+ * points at such distances and a broadcast does not care.  `collective` is one of the MRV_* selectors (or -1: no
+ * particular use, as above); written[i] != 0 marks the buffers the collective writes (null: none).  For every
+ * collective but MRV_ALL_GATHER the result is that of the calls above.
+ */
+MRV_API int mrv_rank_buffers_layout_for(int collective, int count, const size_t* bytes, const unsigned char* written,
+                                        size_t* offsets, size_t* total);
+MRV_API int mrv_rank_buffers_alloc_for(int collective, int count, const size_t* bytes, const unsigned char* written,
+                                       void** ptrs, void** base);
 MRV_API int mrv_comm_group_start(mrv_comm* comm);
 MRV_API int mrv_comm_group_end(mrv_comm* comm);
 

@@ -73,6 +73,10 @@ def load():
     L.mrv_rank_buffers_layout.argtypes = [i32, ctypes.POINTER(sz), ctypes.POINTER(sz), ctypes.POINTER(sz)]
     L.mrv_rank_buffers_alloc.argtypes = [i32, ctypes.POINTER(sz), ctypes.POINTER(vp), ctypes.POINTER(vp)]
     L.mrv_rank_buffers_free.argtypes = [vp]
+    u8p = ctypes.POINTER(ctypes.c_ubyte)
+    L.mrv_rank_buffers_layout_for.argtypes = [i32, i32, ctypes.POINTER(sz), u8p, ctypes.POINTER(sz), ctypes.POINTER(sz)]
+    L.mrv_rank_buffers_alloc_for.argtypes = [i32, i32, ctypes.POINTER(sz), u8p, ctypes.POINTER(vp), ctypes.POINTER(vp)]
+    L.mrv_rank_buffers_layout_for.restype = L.mrv_rank_buffers_alloc_for.restype = i32
     L.mrv_get_free_port.argtypes = []
     L.mrv_create_server.argtypes = [u32, i32]
     L.mrv_comm_create.argtypes = [u32, u32, i32, ctypes.POINTER(vp)]
@@ -81,6 +85,8 @@ def load():
     L.mrv_comm_init.argtypes = [vp, ctypes.c_char_p, i32]
     L.mrv_comm_init_callback.argtypes = [vp, BCAST_FN, vp]
     L.mrv_comm_check.argtypes = [vp, vp]
+    u64p = ctypes.POINTER(ctypes.c_uint64)
+    L.mrv_comm_stats.argtypes = [vp, u64p, u64p, u64p]
     L.mrv_comm_configure.argtypes = [vp, i32, i32]
     L.mrv_comm_send.argtypes = [vp, vp, sz, i32, u32, vp]
     L.mrv_comm_recv.argtypes = [vp, vp, sz, i32, u32, vp]
@@ -103,7 +109,7 @@ def load():
     L.mrv_client_broadcast.argtypes = [vp, vp, vp, sz, u32]
     L.mrv_client_allgather.argtypes = [vp, vp, vp, sz]
     for name in ("mrv_reduce_to_root", "mrv_get_free_port", "mrv_create_server", "mrv_comm_create",
-                 "mrv_comm_init", "mrv_comm_init_callback", "mrv_comm_check", "mrv_comm_configure", "mrv_comm_send", "mrv_comm_recv", "mrv_comm_scatter",
+                 "mrv_comm_init", "mrv_comm_init_callback", "mrv_comm_check", "mrv_comm_stats", "mrv_comm_configure", "mrv_comm_send", "mrv_comm_recv", "mrv_comm_scatter",
                  "mrv_comm_gather", "mrv_comm_all_to_all", "mrv_comm_all_gather", "mrv_comm_all_reduce",
                  "mrv_comm_all_reduce_no_alloc",
                  "mrv_comm_reduce_scatter", "mrv_comm_broadcast", "mrv_comm_reduce", "mrv_comm_group_start",

@@ -200,15 +200,28 @@ def probe_bounded_wait(limit_us, stream=None):
     return gave_up.value
 
 
-def rank_buffers_layout(sizes):
+def _written_array(written, count):
+    if written is None:
+        return None
+    if len(written) != count:
+        raise MegRayError(Status.INVALID_ARGUMENT, f"{count} buffers but {len(written)} written flags")
+    return (ctypes.c_ubyte * max(count, 1))(*[1 if w else 0 for w in written])
+
+
+def rank_buffers_layout(sizes, collective=None, written=None):
     """-> (offsets, total): where buffers of `sizes` bytes go inside one allocation so that a collective over them is
-    served well by the memory system (buffers of 8 MiB and more an odd multiple of 128 MiB apart).
-    mrv_rank_buffers_layout; needs no GPU."""
+    served well by the memory system (buffers of 8 MiB and more an odd multiple of 128 MiB apart; with
+    `collective` ALL_GATHER the buffers flagged in `written` a multiple of 128 MiB plus 32 MiB apart).
+    mrv_rank_buffers_layout / mrv_rank_buffers_layout_for; needs no GPU."""
     count = len(sizes)
     arr = (ctypes.c_size_t * max(count, 1))(*[int(b) for b in sizes])
     offs = (ctypes.c_size_t * max(count, 1))()
     total = ctypes.c_size_t(0)
-    _check(_lib.load().mrv_rank_buffers_layout(count, arr, offs, ctypes.byref(total)))
+    if collective is None:
+        _check(_lib.load().mrv_rank_buffers_layout(count, arr, offs, ctypes.byref(total)))
+    else:
+        _check(_lib.load().mrv_rank_buffers_layout_for(int(collective), count, arr, _written_array(written, count), offs,
+                                                       ctypes.byref(total)))
     return list(offs)[:count], total.value
 
 
@@ -216,12 +229,16 @@ class RankBuffers:
     """Buffers of `sizes` bytes in one device allocation, placed by mrv_rank_buffers_alloc; `.ptrs` are their
     addresses.  free() (or the end of a with block) releases the allocation."""
 
-    def __init__(self, sizes):
+    def __init__(self, sizes, collective=None, written=None):
         count = len(sizes)
         arr = (ctypes.c_size_t * max(count, 1))(*[int(b) for b in sizes])
         ptrs = (ctypes.c_void_p * max(count, 1))()
         base = ctypes.c_void_p(None)
-        _check(_lib.load().mrv_rank_buffers_alloc(count, arr, ptrs, ctypes.byref(base)))
+        if collective is None:
+            _check(_lib.load().mrv_rank_buffers_alloc(count, arr, ptrs, ctypes.byref(base)))
+        else:
+            _check(_lib.load().mrv_rank_buffers_alloc_for(int(collective), count, arr, _written_array(written, count),
+                                                          ptrs, ctypes.byref(base)))
         self.ptrs = [int(p or 0) for p in ptrs][:count]
         self.sizes = [int(b) for b in sizes]
         self._base = base
@@ -244,12 +261,12 @@ class RankBuffers:
             pass
 
 
-def place_tensors(torch, specs, device="cuda"):
+def place_tensors(torch, specs, device="cuda", collective=None, written=None):
     """Tensors of the given (numel, dtype) pairs as views into ONE torch allocation, placed by rank_buffers_layout:
-    the way to hand torch-owned memory to a collective in the placement the library recommends.  The views keep the
-    allocation alive."""
+    the way to hand torch-owned memory to a collective in the placement the library recommends (`collective` and
+    `written` as for rank_buffers_layout).  The views keep the allocation alive."""
     sizes = [int(numel) * torch.empty((), dtype=dtype).element_size() for numel, dtype in specs]
-    offsets, total = rank_buffers_layout(sizes)
+    offsets, total = rank_buffers_layout(sizes, collective, written)
     align = 2 << 20
     arena = torch.empty(total + align, dtype=torch.uint8, device=device)
     skew = (-arena.data_ptr()) % align
@@ -417,6 +434,12 @@ class Communicator:
     def check(self, stream=None):
         """Raises if a stream wait of this rank's group has given up (mrv_comm_check; synchronous)."""
         _check(_lib.load().mrv_comm_check(self._h, _stream(stream)))
+
+    def stats(self):
+        """{"collectives", "plans_built", "sleeps"} of this rank's group since it was formed (mrv_comm_stats)."""
+        c, p, s = ctypes.c_uint64(0), ctypes.c_uint64(0), ctypes.c_uint64(0)
+        _check(_lib.load().mrv_comm_stats(self._h, ctypes.byref(c), ctypes.byref(p), ctypes.byref(s)))
+        return {"collectives": c.value, "plans_built": p.value, "sleeps": s.value}
 
     def configure(self, order=FoldOrder.UCX, schedule=Schedule.FUSED):
         _check(_lib.load().mrv_comm_configure(self._h, int(order), int(schedule)))

@@ -24,6 +24,7 @@
 
 #include "megray.h"
 #include "megray_vrank.h"
+#include "vrank_communicator.h"
 
 namespace {
 
@@ -44,6 +45,7 @@ struct Arguments {
     hipStream_t shared_stream = nullptr;  // -S: every rank enqueues on this one stream
     bool share = false;
     std::string json_path;  // -J: per-size results as JSON lines, with the spread of the per-call times
+    bool random_fill = false;      // -R: inputs from the counter generator instead of zeros
     bool own_allocations = false;  // -M: every rank hipMallocs its own buffers, as the reference's harness does
     std::vector<void*> placed;     // otherwise: in buffers of ranks 0..N-1, then out buffers, in one allocation
 };
@@ -51,14 +53,19 @@ struct Arguments {
 // What rank 0's thread measured for one buffer size.
 struct Timing {
     double avg_us = 0;     // wall time of all iterations including the final stream sync, per iteration
-    double median_us = 0;  // of the time from one call's return to the next call's return
-    double p99_us = 0;
+    double host_us = 0;    // the same without the final sync: what the calls cost the host, per iteration
+    double drain_us = 0;   // the final stream sync: how far the device was behind the host when the last call returned
+    // of the time from one call's return to the next call's return
+    double median_us = 0, p90_us = 0, p99_us = 0, p999_us = 0, max_us = 0;
+    uint64_t sleeps = 0;       // times a rank of the group went to sleep while waiting for the others (all iterations)
+    uint64_t plans_built = 0;  // collectives that had to be planned (the rest came from the plan cache)
 };
 
 using Kernel = std::function<void(std::shared_ptr<MegRay::Communicator>, void*, void*, std::shared_ptr<MegRay::Context>)>;
 
 struct Func {
     std::string name;
+    int collective;  // MRV_* selector for the placement of the buffers (-1: none in particular)
     // buffer sizes per rank as multiples of bufsize (N = ranks), and HBM bytes moved per collective
     std::function<size_t(size_t, size_t)> in_bytes, out_bytes, hbm_bytes;
     std::function<Kernel(const Arguments&, int)> make;
@@ -72,6 +79,21 @@ struct Func {
             std::exit(1);                                                                  \
         }                                                                                  \
     } while (0)
+
+// Inputs for -R: element i of rank r is uniform in [-1, 1), a pure function of (seed + r, i): the splitmix64 finaliser
+// of ((seed + r) xor golden * i) + golden, its top 24 bits as float(u) * 2^-23 - 1.  All-zero buffers (what the
+// reference's harness leaves in its buffers, test/performance.cpp:111) run a few points of the HBM peak faster
+// than data.
+__global__ void fill_uniform_kernel(float* p, uint64_t n, uint64_t key) {
+    const uint64_t golden = 0x9E3779B97F4A7C15ull;
+    for (uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += uint64_t(gridDim.x) * blockDim.x) {
+        uint64_t z = (key ^ (i * golden)) + golden;
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        z ^= z >> 31;
+        p[i] = float(z >> 40) * (1.0f / 8388608.0f) - 1.0f;
+    }
+}
 
 double now_us() {
     return std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now().time_since_epoch()).count();
@@ -93,7 +115,16 @@ void worker(const Func& func, Arguments args, int dev, int port, Timing* res) {
         in_ptr = args.placed[size_t(dev)];
         out_ptr = args.placed[size_t(args.n_devs + dev)];
     }
-    CHECK_HIP(hipMemset(in_ptr, 0, args.in_bufsize));
+    if (args.random_fill) {
+        const uint64_t n = args.in_bufsize / 4;
+        const uint64_t seed = 0x4D656752ull;  // "MegR"
+        if (n) hipLaunchKernelGGL(fill_uniform_kernel, dim3(unsigned(std::min<uint64_t>((n + 255) / 256, 65536))), dim3(256), 0,
+                                  stream, static_cast<float*>(in_ptr), n, seed + uint64_t(dev));
+        CHECK_HIP(hipGetLastError());
+        CHECK_HIP(hipStreamSynchronize(stream));
+    } else {
+        CHECK_HIP(hipMemset(in_ptr, 0, args.in_bufsize));
+    }
     Kernel kernel = func.make(args, dev);
     for (int i = 0; i < args.warmup_iters; i++) kernel(comm, in_ptr, out_ptr, context);
     CHECK_HIP(hipStreamSynchronize(stream));
@@ -105,6 +136,7 @@ void worker(const Func& func, Arguments args, int dev, int port, Timing* res) {
         kernel(comm, in_ptr, out_ptr, context);
         if (dev == 0) stamps.push_back(now_us());
     }
+    const double t_issued = now_us();
     CHECK_HIP(hipStreamSynchronize(stream));
     const double t1 = now_us();
     if (args.own_allocations) {
@@ -116,9 +148,20 @@ void worker(const Func& func, Arguments args, int dev, int port, Timing* res) {
         std::vector<double> gaps;
         for (size_t i = 1; i < stamps.size(); ++i) gaps.push_back(stamps[i] - stamps[i - 1]);
         std::sort(gaps.begin(), gaps.end());
+        const auto at = [&](double q) { return gaps[std::min(gaps.size() - 1, size_t(double(gaps.size()) * q))]; };
         res->avg_us = (t1 - t0) / args.iters;
-        res->median_us = gaps[gaps.size() / 2];
-        res->p99_us = gaps[std::min(gaps.size() - 1, size_t(double(gaps.size()) * 0.99))];
+        res->host_us = (t_issued - t0) / args.iters;
+        res->drain_us = t1 - t_issued;
+        res->median_us = at(0.5);
+        res->p90_us = at(0.9);
+        res->p99_us = at(0.99);
+        res->p999_us = at(0.999);
+        res->max_us = gaps.back();
+        if (auto* vr = dynamic_cast<MegRay::VRankCommunicator*>(comm.get())) {
+            const auto st = vr->stats();
+            res->sleeps = st.sleeps;
+            res->plans_built = st.plans_built;
+        }
     }
 }
 
@@ -138,8 +181,11 @@ Timing run_test(const Func& func, Arguments args) {
         }
         args.placed.resize(2 * n);
         CHECK_HIP(hipSetDevice(0));
-        if (mrv_rank_buffers_alloc(int(2 * n), sizes.data(), args.placed.data(), &base) != 0) {
-            std::fprintf(stderr, "mrv_rank_buffers_alloc: %s\n", mrv_last_error());
+        std::vector<unsigned char> written(2 * n, 0);
+        for (size_t i = 0; i < n; ++i) written[n + i] = 1;
+        if (mrv_rank_buffers_alloc_for(func.collective, int(2 * n), sizes.data(), written.data(), args.placed.data(),
+                                       &base) != 0) {
+            std::fprintf(stderr, "mrv_rank_buffers_alloc_for: %s\n", mrv_last_error());
             std::exit(1);
         }
     }
@@ -156,49 +202,49 @@ std::vector<Func> all_funcs() {
     auto one = [](size_t b, size_t) { return b; };
     auto all = [](size_t b, size_t n) { return b * n; };
     std::vector<Func> f;
-    f.push_back({"send_recv", one, one, [](size_t b, size_t) { return 2 * b; }, [=](A a, int dev) -> Kernel {
+    f.push_back({"send_recv", -1, one, one, [](size_t b, size_t) { return 2 * b; }, [=](A a, int dev) -> Kernel {
                      return [=](auto comm, void* in, void* out, auto ctx) {
                          if (dev == a.send_dev) comm->send(in, a.bufsize / 4, f32, a.recv_dev, ctx);
                          if (dev == a.recv_dev) comm->recv(out, a.bufsize / 4, f32, a.send_dev, ctx);
                      };
                  }});
-    f.push_back({"all_reduce_sum", one, one, [](size_t b, size_t n) { return 2 * n * b; }, [=](A a, int) -> Kernel {
+    f.push_back({"all_reduce_sum", MRV_ALL_REDUCE, one, one, [](size_t b, size_t n) { return 2 * n * b; }, [=](A a, int) -> Kernel {
                      return [=](auto comm, void* in, void* out, auto ctx) {
                          comm->all_reduce(in, out, a.bufsize / 4, f32, MegRay::MEGRAY_SUM, ctx);
                      };
                  }});
-    f.push_back({"scatter", all, one, [](size_t b, size_t n) { return 2 * n * b; }, [=](A a, int) -> Kernel {
+    f.push_back({"scatter", MRV_SCATTER, all, one, [](size_t b, size_t n) { return 2 * n * b; }, [=](A a, int) -> Kernel {
                      return [=](auto comm, void* in, void* out, auto ctx) {
                          comm->scatter(in, out, a.bufsize / 4, f32, 0, ctx);
                      };
                  }});
-    f.push_back({"gather", one, all, [](size_t b, size_t n) { return 2 * n * b; }, [=](A a, int) -> Kernel {
+    f.push_back({"gather", MRV_GATHER, one, all, [](size_t b, size_t n) { return 2 * n * b; }, [=](A a, int) -> Kernel {
                      return [=](auto comm, void* in, void* out, auto ctx) {
                          comm->gather(in, out, a.bufsize / 4, f32, 0, ctx);
                      };
                  }});
-    f.push_back({"all_to_all", all, all, [](size_t b, size_t n) { return 2 * n * n * b; }, [=](A a, int) -> Kernel {
+    f.push_back({"all_to_all", MRV_ALL_TO_ALL, all, all, [](size_t b, size_t n) { return 2 * n * n * b; }, [=](A a, int) -> Kernel {
                      return [=](auto comm, void* in, void* out, auto ctx) {
                          comm->all_to_all(in, out, a.bufsize / 4, f32, ctx);
                      };
                  }});
-    f.push_back({"all_gather", one, all, [](size_t b, size_t n) { return n * b + n * n * b; }, [=](A a, int) -> Kernel {
+    f.push_back({"all_gather", MRV_ALL_GATHER, one, all, [](size_t b, size_t n) { return n * b + n * n * b; }, [=](A a, int) -> Kernel {
                      return [=](auto comm, void* in, void* out, auto ctx) {
                          comm->all_gather(in, out, a.bufsize / 4, f32, ctx);
                      };
                  }});
-    f.push_back({"reduce_scatter_sum", all, one, [](size_t b, size_t n) { return n * n * b + n * b; },
+    f.push_back({"reduce_scatter_sum", MRV_REDUCE_SCATTER, all, one, [](size_t b, size_t n) { return n * n * b + n * b; },
                  [=](A a, int) -> Kernel {
                      return [=](auto comm, void* in, void* out, auto ctx) {
                          comm->reduce_scatter(in, out, a.bufsize / 4, f32, MegRay::MEGRAY_SUM, ctx);
                      };
                  }});
-    f.push_back({"broadcast", one, one, [](size_t b, size_t n) { return b + n * b; }, [=](A a, int) -> Kernel {
+    f.push_back({"broadcast", MRV_BROADCAST, one, one, [](size_t b, size_t n) { return b + n * b; }, [=](A a, int) -> Kernel {
                      return [=](auto comm, void* in, void* out, auto ctx) {
                          comm->broadcast(in, out, a.bufsize / 4, f32, 0, ctx);
                      };
                  }});
-    f.push_back({"reduce_sum", one, one, [](size_t b, size_t n) { return n * b + b; }, [=](A a, int) -> Kernel {
+    f.push_back({"reduce_sum", MRV_REDUCE, one, one, [](size_t b, size_t n) { return n * b + b; }, [=](A a, int) -> Kernel {
                      return [=](auto comm, void* in, void* out, auto ctx) {
                          comm->reduce(in, out, a.bufsize / 4, f32, MegRay::MEGRAY_SUM, 0, ctx);
                      };
@@ -221,11 +267,14 @@ void show_help(const char* argv0) {
                  "      -s[int,..]  packet size(s) in bytes per rank (default: 8, 1 KiB, 512 KiB, 1 MiB, 10 MiB)\n"
                  "      -w[int]     warm-up iterations (default 100)\n"
                  "      -i[int]     timed iterations (default 100)\n"
-                 "      -J[path]    also append one JSON line per size to this file: avg, median and 99th percentile\n"
-                 "                  of the per-call time on rank 0 (not in the reference's harness)\n"
+                 "      -J[path]    also append one JSON line per size to this file: average, median, 90 / 99 / 99.9th\n"
+                 "                  percentile and maximum of the per-call time on rank 0, the final stream sync, and the\n"
+                 "                  group's sleep and planning counts (not in the reference's harness)\n"
+                 "      -R          fill the inputs with uniform random fp32 in [-1, 1) from a counter generator (seed + rank)\n"
+                 "                  instead of zeros; the table is the same\n"
                  "      -M          every rank allocates its own buffers with hipMalloc, as the reference's harness\n"
-                 "                  does; without it all buffers lie in one allocation, placed by the library\n"
-                 "                  (mrv_rank_buffers_alloc: large buffers an odd multiple of 128 MiB apart)\n"
+                 "                  does; without it all buffers lie in one allocation, placed by the library for the\n"
+                 "                  collective at hand (mrv_rank_buffers_alloc_for)\n"
                  "      -S          all ranks enqueue on ONE stream (not in the reference's harness: its ranks\n"
                  "                  are devices); without it every rank has a stream of its own\n"
                  "      -A -B       send/recv: sending node rank / dev (default 0 / 0)\n"
@@ -244,11 +293,12 @@ void print(T value) {
 int main(int argc, char* argv[]) {
     Arguments args;
     int ch;
-    while ((ch = getopt(argc, argv, "hSMd:I:P:n:r:e:f:s:w:i:A:B:C:D:J:")) != EOF) {
+    while ((ch = getopt(argc, argv, "hSMRd:I:P:n:r:e:f:s:w:i:A:B:C:D:J:")) != EOF) {
         switch (ch) {
             case 'h': show_help(argv[0]); return 0;
             case 'S': args.share = true; break;
             case 'M': args.own_allocations = true; break;
+            case 'R': args.random_fill = true; break;
             case 'J': args.json_path = optarg; break;
             case 'd': args.n_devs = std::atoi(optarg); break;
             case 'I': args.master_ip = optarg; break;
@@ -327,8 +377,13 @@ int main(int argc, char* argv[]) {
             if (json.is_open()) {
                 json << "{\"func\": \"" << func.name << "\", \"ranks\": " << args.n_devs << ", \"bufsize\": " << size
                      << ", \"streams\": \"" << (args.share ? "shared" : "own") << "\", \"iters\": " << args.iters
-                     << ", \"avg_us\": " << timing.avg_us << ", \"median_us\": " << timing.median_us
-                     << ", \"p99_us\": " << timing.p99_us << "}" << std::endl;
+                     << ", \"fill\": \"" << (args.random_fill ? "random" : "zeros") << "\", \"buffers\": \""
+                     << (args.own_allocations ? "own" : "placed") << "\", \"avg_us\": " << timing.avg_us
+                     << ", \"host_us\": " << timing.host_us << ", \"drain_us\": " << timing.drain_us
+                     << ", \"median_us\": " << timing.median_us << ", \"p90_us\": " << timing.p90_us
+                     << ", \"p99_us\": " << timing.p99_us << ", \"p999_us\": " << timing.p999_us
+                     << ", \"max_us\": " << timing.max_us << ", \"sleeps\": " << timing.sleeps
+                     << ", \"plans_built\": " << timing.plans_built << "}" << std::endl;
             }
             double hbm = func.hbm_bytes(run.bufsize, args.n_devs) / avg_us / 1000.0;
             print(size);

@@ -133,9 +133,10 @@ PERF_BIN = os.path.join(HERE, "apps", "megray_performance")
 
 def build_performance():
     """Compile the performance CLI (the MegRay benchmark harness for this backend)."""
-    cmd = [HIPCC, "-std=c++17", "-O2", "-x", "c++", "-D__HIP_PLATFORM_AMD__=1", f"-I{os.path.join(ROOT, 'include')}",
-           f"-I{ROCM}/include", PERF_SRC, "-o", PERF_BIN, f"-L{HERE}", "-lmegray_vrank", f"-L{ROCM}/lib",
-           "-lamdhip64", "-pthread", "-Wl,-rpath,$ORIGIN/..", f"-Wl,-rpath,{ROCM}/lib"]
+    # compiled as HIP: the tool has one kernel of its own (the random fill of -R)
+    cmd = [HIPCC, "-std=c++17", "-O2", "-x", "hip", "-ffp-contract=off"] + DEVICE_FLAGS + [
+           f"-I{os.path.join(ROOT, 'include')}", f"-I{CSRC}", PERF_SRC, "-o", PERF_BIN, f"-L{HERE}", "-lmegray_vrank",
+           "-pthread", "-Wl,-rpath,$ORIGIN/..", f"-Wl,-rpath,{ROCM}/lib"]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"building {PERF_SRC} failed:\n{proc.stdout}\n{proc.stderr}")

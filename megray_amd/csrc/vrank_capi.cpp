@@ -494,35 +494,63 @@ int mrv_probe_bounded_wait(uint64_t limit_us, void* stream, uint64_t* gave_up) {
     });
 }
 
+namespace {
+
+PlacementUse placement_use(int collective) {
+    if (collective < 0) return kPlaceAny;
+    if (collective > MRV_REDUCE) MEGRAY_THROW("unknown collective");
+    return collective == MRV_ALL_GATHER ? kPlaceOneToAll : kPlaceAny;
+}
+
+Status layout_buffers(int collective, int count, const size_t* bytes, const unsigned char* written, size_t* offsets,
+                      size_t* total) {
+    if (count < 0) MEGRAY_THROW("negative buffer count");
+    need(total, "total is null");
+    if (count > 0) {
+        need(bytes, "bytes is null");
+        need(offsets, "offsets is null");
+    }
+    if (!placement_layout(count, bytes, offsets, total, placement_use(collective), written))
+        MEGRAY_THROW("the buffers do not fit the address space");
+    return MEGRAY_OK;
+}
+
+Status alloc_buffers(int collective, int count, const size_t* bytes, const unsigned char* written, void** ptrs,
+                     void** base) {
+    if (count <= 0) MEGRAY_THROW("no buffers asked for");
+    need(bytes, "bytes is null");
+    need(ptrs, "ptrs is null");
+    need(base, "base is null");
+    *base = nullptr;
+    std::vector<size_t> offsets(static_cast<size_t>(count));
+    size_t total = 0;
+    if (!placement_layout(count, bytes, offsets.data(), &total, placement_use(collective), written))
+        MEGRAY_THROW("the buffers do not fit the address space");
+    void* p = nullptr;
+    HIP_CHECK(hipMalloc(&p, total ? total : 1));
+    *base = p;
+    for (int i = 0; i < count; ++i) ptrs[i] = static_cast<char*>(p) + offsets[size_t(i)];
+    return MEGRAY_OK;
+}
+
+}  // namespace
+
 int mrv_rank_buffers_layout(int count, const size_t* bytes, size_t* offsets, size_t* total) {
-    return guarded([&] {
-        if (count < 0) MEGRAY_THROW("negative buffer count");
-        need(total, "total is null");
-        if (count > 0) {
-            need(bytes, "bytes is null");
-            need(offsets, "offsets is null");
-        }
-        if (!placement_layout(count, bytes, offsets, total)) MEGRAY_THROW("the buffers do not fit the address space");
-        return MEGRAY_OK;
-    });
+    return guarded([&] { return layout_buffers(-1, count, bytes, nullptr, offsets, total); });
+}
+
+int mrv_rank_buffers_layout_for(int collective, int count, const size_t* bytes, const unsigned char* written,
+                                size_t* offsets, size_t* total) {
+    return guarded([&] { return layout_buffers(collective, count, bytes, written, offsets, total); });
 }
 
 int mrv_rank_buffers_alloc(int count, const size_t* bytes, void** ptrs, void** base) {
-    return guarded([&] {
-        if (count <= 0) MEGRAY_THROW("no buffers asked for");
-        need(bytes, "bytes is null");
-        need(ptrs, "ptrs is null");
-        need(base, "base is null");
-        *base = nullptr;
-        std::vector<size_t> offsets(static_cast<size_t>(count));
-        size_t total = 0;
-        if (!placement_layout(count, bytes, offsets.data(), &total)) MEGRAY_THROW("the buffers do not fit the address space");
-        void* p = nullptr;
-        HIP_CHECK(hipMalloc(&p, total));
-        for (int i = 0; i < count; ++i) ptrs[i] = static_cast<char*>(p) + offsets[size_t(i)];
-        *base = p;
-        return MEGRAY_OK;
-    });
+    return guarded([&] { return alloc_buffers(-1, count, bytes, nullptr, ptrs, base); });
+}
+
+int mrv_rank_buffers_alloc_for(int collective, int count, const size_t* bytes, const unsigned char* written,
+                               void** ptrs, void** base) {
+    return guarded([&] { return alloc_buffers(collective, count, bytes, written, ptrs, base); });
 }
 
 int mrv_rank_buffers_free(void* base) {
@@ -581,6 +609,19 @@ int mrv_comm_check(mrv_comm* comm, void* stream) {
         auto* vr = dynamic_cast<VRankCommunicator*>(comm->comm.get());
         if (!vr) MEGRAY_THROW("not a vrank communicator");
         return vr->check(HipContext::make(as_stream(stream)));
+    });
+}
+
+int mrv_comm_stats(mrv_comm* comm, uint64_t* collectives, uint64_t* plans_built, uint64_t* sleeps) {
+    return guarded([&] {
+        need(comm, "comm is null");
+        auto* vr = dynamic_cast<VRankCommunicator*>(comm->comm.get());
+        if (!vr) MEGRAY_THROW("not a vrank communicator");
+        const VRankCommunicator::Stats st = vr->stats();
+        if (collectives) *collectives = st.collectives;
+        if (plans_built) *plans_built = st.plans_built;
+        if (sleeps) *sleeps = st.sleeps;
+        return MEGRAY_OK;
     });
 }
 

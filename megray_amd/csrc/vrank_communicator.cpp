@@ -252,6 +252,12 @@ public:
         return op->status;
     }
 
+    void stats(uint64_t out[3]) const {
+        out[0] = m_stat_collectives.load(std::memory_order_relaxed);
+        out[1] = m_stat_plans.load(std::memory_order_relaxed);
+        out[2] = m_stat_sleeps.load(std::memory_order_relaxed);
+    }
+
     // Reads the counters back now (after `stream` has drained): has any stream wait of the group given up?
     Status check(hipStream_t stream) {
         for (EdgeSet& set : m_edges) {
@@ -369,6 +375,7 @@ private:
     }
 
     void sleep_until_past(uint64_t need) {
+        m_stat_sleeps.fetch_add(1, std::memory_order_relaxed);
         std::unique_lock<std::mutex> lock(m_mutex);
         m_sleepers.fetch_add(1, std::memory_order_seq_cst);
         m_cv.wait(lock, [&] { return m_generation.load(std::memory_order_seq_cst) >= need; });
@@ -493,6 +500,8 @@ private:
         uint64_t* ticket;
     };
     static bool hook_fields(Step& step, HookFields& f) {
+        // MEGRAY_VRANK_HOOK_MAX_TILES in the environment moves the border (0: no launch carries the ordering)
+        static const uint64_t kHookMaxTiles = env_u64("MEGRAY_VRANK_HOOK_MAX_TILES", vrank::kHookMaxTiles);
         switch (step.kind) {
             case Step::kFlat:
                 if (step.flat.waves != 1 || step.flat.total_tiles >= kHookMaxTiles) return false;
@@ -601,7 +610,9 @@ private:
         // plan first: a rejected call must not leave marks or waits behind
         const uint64_t signature = plan_signature(lead, send, recv);
         CachedPlan* cp = lookup(lead, send, recv, signature);
+        m_stat_collectives.fetch_add(1, std::memory_order_relaxed);
         if (!cp) {
+            m_stat_plans.fetch_add(1, std::memory_order_relaxed);
             auto fresh = std::make_unique<CachedPlan>();
             fresh->key = lead;
             fresh->signature = signature;
@@ -795,6 +806,7 @@ private:
     std::chrono::steady_clock::time_point m_fixed_checked{};  // when the static counter block was last read back
     std::chrono::steady_clock::duration m_fixed_period{};
     std::atomic<uint32_t> m_sleepers{0};
+    std::atomic<uint64_t> m_stat_collectives{0}, m_stat_plans{0}, m_stat_sleeps{0};
     alignas(64) std::atomic<uint32_t> m_arrived{0};     // ranks that have deposited their call
     alignas(64) std::atomic<uint64_t> m_generation{0};  // collectives released so far; parked ranks poll it
     [[maybe_unused]] alignas(64) char m_pad[64] = {};  // keeps what follows off the polled line
@@ -938,6 +950,12 @@ Status VRankCommunicator::all_reduce(const void* sendbuff, void* recvbuff, size_
 Status VRankCommunicator::all_reduce_no_alloc(const void* sendbuff, void* recvbuff, size_t len, DType dtype,
                                               ReduceOp op, std::shared_ptr<Context> ctx) {
     VRANK_COLLECTIVE_ON(true, kCollAllReduce, len, dtype, op, 0, reduce_elem_size(dtype); check_reduce_op(op));
+}
+
+VRankCommunicator::Stats VRankCommunicator::stats() const {
+    uint64_t v[3] = {0, 0, 0};
+    if (m_group) m_group->stats(v);
+    return {v[0], v[1], v[2]};
 }
 
 Status VRankCommunicator::check(std::shared_ptr<Context> ctx) {

@@ -58,6 +58,15 @@ public:
     // half wait limits; this asks now.
     Status check(ContextPtr ctx);
 
+    // Not part of the reference API: counts kept by this rank's group since it was formed, for benchmarks and
+    // diagnosis.  collectives: collectives launched; plans_built: of those, how many had to be planned (the others
+    // found their plan in the group's cache); sleeps: times a rank that was waiting for the others gave up polling
+    // and went to sleep on a condition variable (a wake-up costs tens of microseconds).
+    struct Stats {
+        uint64_t collectives, plans_built, sleeps;
+    };
+    Stats stats() const;
+
     // Not part of the reference API: which reference loop's combination order all_reduce /
     // reduce_scatter / reduce reproduce (default: the ucx ring), and how all_reduce is laid out in
     // launches (default: fused).  Every rank of a group must choose the same.

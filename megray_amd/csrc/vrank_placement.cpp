@@ -18,8 +18,13 @@ bool round_up(size_t value, size_t unit, size_t* out) {
 
 }  // namespace
 
-size_t placement_pitch(size_t bytes) {
+size_t placement_pitch(size_t bytes, bool written_one_to_all) {
     size_t pitch = 0;
+    if (bytes >= kSpreadFrom && written_one_to_all) {
+        const size_t units = bytes / kSpreadUnit + (bytes % kSpreadUnit != 0);
+        if (units > (SIZE_MAX - kWrittenShift) / kSpreadUnit) return 0;
+        return units * kSpreadUnit + kWrittenShift;
+    }
     if (bytes >= kSpreadFrom) {
         size_t units = bytes / kSpreadUnit + (bytes % kSpreadUnit != 0);
         units |= 1;  // odd: buffer i starts at i * units * 128 MiB, which differs in bits 27 and up for every i < 32
@@ -31,10 +36,11 @@ size_t placement_pitch(size_t bytes) {
     return pitch;
 }
 
-bool placement_layout(int count, const size_t* bytes, size_t* offsets, size_t* total) {
+bool placement_layout(int count, const size_t* bytes, size_t* offsets, size_t* total, PlacementUse use,
+                      const unsigned char* written) {
     size_t at = 0, end = 0;
     for (int i = 0; i < count; ++i) {
-        const size_t pitch = placement_pitch(bytes[i]);
+        const size_t pitch = placement_pitch(bytes[i], use == kPlaceOneToAll && written && written[i]);
         size_t own = 0;  // the last buffer needs its own pages only, not the distance to a next one
         if (bytes[i] >= kLargePage && !round_up(at, kLargePage, &at)) return false;  // after smaller buffers
         if (pitch == 0 || pitch > SIZE_MAX - at || !round_up(bytes[i] ? bytes[i] : 1, kPage, &own)) return false;

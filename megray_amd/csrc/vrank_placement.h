@@ -21,13 +21,32 @@ namespace vrank {
 
 constexpr size_t kSpreadUnit = size_t(128) << 20;  // distances between spread buffers are odd multiples of this
 constexpr size_t kSpreadFrom = size_t(8) << 20;    // smaller buffers stay close together (they live in the caches)
+// The buffers an all_gather WRITES (every rank's block is read once and stored into every rank's buffer: eight
+// write streams to one read stream, each walking through eight blocks) are served best a multiple of 128 MiB PLUS
+// 32 MiB apart:
+// all_gather of 8 x 16 MiB fp16 into 128 MiB buffers 79.4 % of the HBM peak with the outputs 128 MiB apart, 82.9 /
+// 84.2 / 84.0 / 83.9 / 82.7 / 83.2 / 80.4 / 84.3 at 128 MiB + 8 / 16 / 32 / 48 / 64 / 96 / 128 / 160 MiB; into 512 MiB
+// buffers 82.1 % at 512 MiB and 84.9 - 85.4 at + 16 ... + 96 MiB, 82.5 at + 128.  The all_reduce family loses one to two
+// points at such distances (8 x 1 GiB 84.0 -> 83.5, 8 x 128 MiB 84.8 -> 82.6, whether all buffers or only the outputs
+// move), and a broadcast (one block into every buffer) reads 84 - 85 % either way, so the distance depends on what the
+// buffers are for.
+constexpr size_t kWrittenShift = size_t(32) << 20;
 
-// Distance from the start of a buffer of `bytes` bytes to the start of the next one.
-size_t placement_pitch(size_t bytes);
+// What the buffers handed to placement_layout are for.
+enum PlacementUse : int {
+    kPlaceAny = 0,        // folds and pairwise copies: everything an odd multiple of 128 MiB apart
+    kPlaceOneToAll = 1,   // all_gather: the buffers marked as written lie 128 MiB * k + 32 MiB apart
+};
 
-// offsets[i] of buffer i (bytes[i] long) from a common base, *total = bytes to allocate.
+// Distance from the start of a buffer of `bytes` bytes to the start of the next one (`written_one_to_all`: the
+// buffer is one of those an all_gather stores every rank's block into).
+size_t placement_pitch(size_t bytes, bool written_one_to_all = false);
+
+// offsets[i] of buffer i (bytes[i] long) from a common base, *total = bytes to allocate.  `written` (may be null:
+// nothing is) marks the buffers the collective writes; it matters for kPlaceOneToAll only.
 // false if the sum does not fit a size_t.
-bool placement_layout(int count, const size_t* bytes, size_t* offsets, size_t* total);
+bool placement_layout(int count, const size_t* bytes, size_t* offsets, size_t* total, PlacementUse use = kPlaceAny,
+                      const unsigned char* written = nullptr);
 
 }  // namespace vrank
 }  // namespace MegRay

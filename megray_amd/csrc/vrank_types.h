@@ -156,11 +156,13 @@ constexpr bool flat_one_out(uint32_t nranks, uint32_t nout, uint64_t total_tiles
     return nout == 1 && nranks >= 3 && total_tiles >= kFlatOneOutMinTiles;
 }
 // One-wavefront launches below this many workgroups carry the thread-per-rank API's stream ordering
-// themselves (EdgeHooks).  Beyond it the release fence every workgroup then executes costs more than
-// the two launches it saves.  Measured, 8 ranks, a stream per rank, microseconds per all_reduce with /
-// without: 16 - 128 tiles 16 - 18 / 22 - 23, 256 tiles 18 / 22.5, 384 tiles 21 - 34 / 22 - 23, 508 tiles
-// 30 / 22, 1024 tiles 42 / 24.
-constexpr uint32_t kHookMaxTiles = 288;
+// themselves (EdgeHooks).  Beyond it the release fence every workgroup then executes (it writes the L2 back)
+// costs the DEVICE more than the two launches it saves the host: the calls still return quickly, but the
+// device falls behind them.  Measured, 8 ranks, a stream per rank, 2000 all_reduces back to back, microseconds
+// per all_reduce INCLUDING the final stream synchronisation (and what the calls alone cost the host), with /
+// without: 4 tiles 16 (16) / 21, 64 tiles 16 (15) / 21, 128 tiles 19 (16) / 19.5, 192 tiles 20 - 23 (16) / 21,
+// 256 tiles 27 - 29 (15) / 19 - 21, 384 tiles 27 - 45 (15) / 21, 512 tiles 36 - 41 (16) / 20.5.
+constexpr uint32_t kHookMaxTiles = 136;
 constexpr uint32_t group_grid(uint32_t total_tiles) {
     return (total_tiles + kGroupWaves * kGroupStride - 1) / (kGroupWaves * kGroupStride) * kGroupStride;
 }

@@ -386,10 +386,10 @@ int main(int argc, char** argv) {
     }
     std::thread exec(executor, seed ^ 0x5bd1e995);
 
-    // lengths (int32 elements): launches that carry the stream ordering themselves (1 and 274 tiles), a short
+    // lengths (int32 elements): launches that carry the stream ordering themselves (1 and 118 tiles), a short
     // launch between wait and notify kernels (391 tiles), the group form (2344 tiles), and off-grid lengths
     // that go through the general kernels
-    const size_t lengths[] = {16, 70000, 100000, 600000, 3, 1001};
+    const size_t lengths[] = {16, 30000, 100000, 600000, 3, 1001};
     std::vector<Round> plan(rounds);
     for (Round& r : plan) {
         r.kind = int(rng() % 9);

@@ -505,14 +505,14 @@ def test_a_stream_wait_that_gives_up_poisons_its_group(entry, length, monkeypatc
         c.close()
 
 
-@pytest.mark.parametrize("length", [3000, 70000, 100000, (1 << 19) + 11])
+@pytest.mark.parametrize("length", [3000, 30000, 70000, 100000, (1 << 19) + 11])
 def test_back_to_back_rounds_with_fresh_data_on_rank_streams(length):
     """Five all_reduces back to back, every round with different inputs that each rank copies into the SAME device
     buffer on its own stream right before the call, and with the result copied out of the SAME device buffer on
     that stream right after, no host synchronisation in between.  A collective that started before some rank's
     copy-in had landed, or a copy-in that overtook the previous collective's reads, or a copy-out that overtook
     the collective's writes, shows as a wrong round.  The lengths run the short kernel that carries the stream
-    ordering itself (12 and 274 tiles), the short kernel between separate wait / notify kernels (391 tiles) and the
+    ordering itself (12 and 118 tiles), the short kernel between separate wait / notify kernels (274 and 391 tiles) and the
     group kernel between them (2049 tiles)."""
     nranks, rounds = 8, 5
     rng = np.random.default_rng(length)

@@ -106,3 +106,25 @@ def test_ten_mib_row_agrees_with_an_event_timing(tmp_path):
     own = parse_tables(out)["all_reduce_sum"][1][0]
     print(f"performance tool, a stream per rank: {own[4]:.0f} GB/s ({own[1]:.1f} us per call)")
     assert own[4] > 0.6 * event_gbps
+
+
+def test_random_fill_own_buffers_and_the_spread_record(tmp_path):
+    """-R fills the inputs from the counter generator, -M lets every rank hipMalloc its own buffers (what the reference's
+    harness does, test/performance.cpp:108-110); the table keeps the reference's columns either way, and -J records
+    how the per-call times spread, how far the device was behind at the end and how often a rank went to sleep."""
+    log = tmp_path / "spread.jsonl"
+    out = run_cli("-d", "8", "-f", "all_reduce", "-s", "65536,4194304", "-w", "50", "-i", "300", "-R", "-M", "-J", str(log))
+    cols, rows = parse_tables(out)["all_reduce_sum"]
+    assert cols[:4] == ["bufsize", "time(us)", "speed(GB/s)", "iters"] and [int(r[0]) for r in rows] == [65536, 4194304]
+    records = [json.loads(line) for line in log.read_text().splitlines()]
+    assert [r["bufsize"] for r in records] == [65536, 4194304]
+    for r in records:
+        assert r["fill"] == "random" and r["buffers"] == "own" and r["streams"] == "own" and r["iters"] == 300
+        assert 0 < r["median_us"] <= r["p90_us"] <= r["p99_us"] <= r["p999_us"] <= r["max_us"]
+        assert r["host_us"] <= r["avg_us"] and r["drain_us"] >= 0
+        assert r["avg_us"] * 300 == pytest.approx(r["host_us"] * 300 + r["drain_us"], rel=1e-4)  # six printed digits
+        assert r["plans_built"] == 1  # 350 collectives on the same buffers: planned once
+    zeros = tmp_path / "zeros.jsonl"
+    run_cli("-d", "2", "-f", "all_reduce", "-s", "4096", "-w", "5", "-i", "20", "-J", str(zeros))
+    r = json.loads(zeros.read_text().splitlines()[0])
+    assert r["fill"] == "zeros" and r["buffers"] == "placed"

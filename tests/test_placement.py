@@ -26,6 +26,34 @@ def test_large_buffers_lie_an_odd_multiple_of_128_mib_apart():
         assert offsets[-1] + size <= total < offsets[-1] + size + 4096
 
 
+def test_buffers_an_all_gather_writes_lie_32_mib_off_the_128_mib_grid():
+    """all_gather stores every rank's block into every rank's buffer: the written buffers go a multiple of
+    128 MiB plus 32 MiB apart (what eight write streams against one read stream are served best at), the buffers
+    that are read keep the odd multiple of 128 MiB; every other collective is laid out as without the hint."""
+    shift = 32 * MIB
+    for coll in (mr.Collective.ALL_GATHER,):
+        for small, large in ((16 * MIB, 128 * MIB), (64 * MIB, 512 * MIB), (9 * MIB, 72 * MIB + 4096)):
+            sizes, written = [small] * 8 + [large] * 8, [0] * 8 + [1] * 8
+            offsets, total = mr.rank_buffers_layout(sizes, coll, written)
+            read_pitch, write_pitch = offsets[1] - offsets[0], offsets[9] - offsets[8]
+            assert read_pitch % UNIT == 0 and (read_pitch // UNIT) % 2 == 1
+            assert write_pitch % UNIT == shift and large <= write_pitch - shift < large + UNIT, (large, write_pitch)
+            assert offsets[8:] == [offsets[8] + i * write_pitch for i in range(8)]
+            spans = sorted(zip(offsets, sizes))
+            assert all(a + n <= b for (a, n), (b, _) in zip(spans, spans[1:])) and spans[-1][0] + spans[-1][1] <= total
+        # small written buffers live in the caches and stay close together
+        assert mr.rank_buffers_layout([4096] * 4, coll, [1] * 4) == mr.rank_buffers_layout([4096] * 4)
+    sizes = [1 << 27] * 16
+    for coll in (mr.Collective.ALL_REDUCE, mr.Collective.REDUCE_SCATTER, mr.Collective.ALL_TO_ALL, mr.Collective.SCATTER,
+                 mr.Collective.GATHER, mr.Collective.BROADCAST, mr.Collective.REDUCE, mr.Collective.REDUCE2):
+        assert mr.rank_buffers_layout(sizes, coll, [0] * 8 + [1] * 8) == mr.rank_buffers_layout(sizes)
+    assert mr.rank_buffers_layout(sizes, mr.Collective.ALL_GATHER, None) == mr.rank_buffers_layout(sizes)  # nothing marked
+    with pytest.raises(mr.MegRayError, match="unknown collective"):
+        mr.rank_buffers_layout(sizes, 99, [0] * 16)
+    with pytest.raises(mr.MegRayError, match="written flags"):
+        mr.rank_buffers_layout(sizes, mr.Collective.ALL_GATHER, [1] * 3)
+
+
 def test_small_buffers_stay_close_together():
     offsets, total = mr.rank_buffers_layout([4096] * 16)
     assert offsets == [i * 4096 for i in range(16)] and total == 16 * 4096
