@@ -1027,15 +1027,24 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
     const uint32_t mine = first + wave * kGroupStride;
     const bool exchange = (L.exchange & 1u) != 0;
 
-    // tile k of the group is first + k * kGroupStride; it is loaded if it lies inside the buffers
-    u32x4 x[K];
-#pragma unroll
-    for (int r = 0; r < K; ++r) {
+    // tile k of the group is first + k * kGroupStride; it is loaded if it lies inside the buffers.
+    // A wavefront keeps kGroupLoadsInFlight loads in flight: load r + 2 is issued when load r has arrived (its
+    // address is made to depend on it).  The memory system serves a workgroup's accesses better spread over time
+    // than all at once, the more so the worse the caller's buffers lie relative to each other (see kGroupLoadsInFlight).
+    constexpr int D = K < int(kGroupLoadsInFlight) ? K : int(kGroupLoadsInFlight);
+    const auto load_input = [&](int r, uint32_t lane) -> u32x4 {
         const uint64_t tile = uint64_t(first) + ((wave + r) % W) * kGroupStride;
         if ((tile + 1) * TILE <= L.count)
-            x[r] = load_tile_vec(static_cast<const char*>(L.in[r]) + tile * (kThreads * kVecBytes), tid);
-        else
-            x[r] = u32x4{0u, 0u, 0u, 0u};  // never folded: such a tile goes element by element
+            return load_tile_vec(static_cast<const char*>(L.in[r]) + tile * (kThreads * kVecBytes), lane);
+        return u32x4{0u, 0u, 0u, 0u};  // never folded: such a tile goes element by element
+    };
+    const bool paced = (L.exchange & kFlatPaced) != 0;
+    u32x4 x[K];
+#pragma unroll
+    for (int r = 0; r < D; ++r) x[r] = load_input(r, tid);
+    if (!paced) {  // short launches: everything at once, their time is latency
+#pragma unroll
+        for (int r = D; r < K; ++r) x[r] = load_input(r, tid);
     }
     // A launch of a communicator group stores nothing once the group is poisoned.  The wavefronts of a workgroup
     // may see the poison rise at different moments, so it only ever masks stores and never skips a barrier.
@@ -1051,7 +1060,14 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
     const int dir = meta_dir(tr.meta);
     const uint64_t out_shift = tr.shift;
 #pragma unroll
-    for (int r = 0; r < K; ++r) stage[(wave + r) % W][r][tid] = x[r];
+    for (int r = 0; r < K; ++r) {
+        if (paced && r + D < K) {
+            uint32_t lane = tid;
+            asm volatile("" : "+v"(lane) : "v"(x[r]));  // the next load's address waits for x[r]
+            x[r + D] = load_input(r + D, lane);
+        }
+        stage[(wave + r) % W][r][tid] = x[r];
+    }
     __syncthreads();
 
     if (run >= 0) {
@@ -1091,6 +1107,8 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
                 const uint64_t tile = uint64_t(first) + k * kGroupStride;
                 store_tile_vec(static_cast<char*>(L.out[m]) + tile * (kThreads * kVecBytes), tid, result[k][tid]);
             }
+            // ... and kGroupStoresInFlight stores in flight
+            if (paced && (m + 1) % int(kGroupStoresInFlight) == 0 && m + 1 < K) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
     }
 }

@@ -71,6 +71,7 @@ struct FoldLaunch {
 };
 
 constexpr uint32_t kFlatGuarded = 4;  // FlatLaunch::exchange
+constexpr uint32_t kFlatPaced = 8;    // FlatLaunch::exchange, group form: a wavefront keeps two loads and two stores in flight
 
 constexpr uint32_t kMaxFlatRuns = 48;  // 2N chunks cut again at N-1 rank borders
 
@@ -108,6 +109,7 @@ struct FlatLaunch {
     uint32_t waves;     // wavefronts per workgroup: 1, or kGroupWaves for the group form (launches of many tiles)
     uint32_t exchange;  // group form: bit 0 = every rank is an output at the inputs' offsets, results are exchanged too;
                         // bit 1 = tiles share cache lines with their neighbours, deal runs of workgroups to XCDs;
+                        // bit 3 (kFlatPaced) = a wavefront keeps kGroupLoadsInFlight loads / stores in flight instead of all;
                         // either form: bit 2 (kFlatGuarded) = the launch belongs to a communicator group, hooks.words
                         // is set and the group's poison is tested before anything is stored (the flag sits here, in
                         // the line of scalars every wavefront reads anyway; `hooks` lies several cache lines further)
@@ -126,6 +128,18 @@ struct FlatLaunch {
 // and 2 or 4 ranks cross between 2 and 4 MiB as well), the segment and pack kernels from 512.
 constexpr uint32_t kGroupWaves = 4;
 constexpr uint32_t kGroupStride = 32;
+// A wavefront of the flat group kernel has this many loads in flight, and (where every rank is an output) this many
+// stores: two each.  With all eight at once a workgroup puts 32 loads, then 32 stores, on the memory system within a
+// few hundred cycles, to the same offsets of buffers whose addresses may differ in a few high bits only; spaced out,
+// the same accesses are served faster, and the worse the buffers lie the more it gains.  Measured on MI355X, bare
+// kernel of the same shape, 8 x 1 GiB fp32 in, 8 x 1 GiB out, % of the HBM peak, all at once -> two in flight:
+// sixteen buffers of one allocation 1 GiB apart 76.3 -> 80.1, 1 GiB + 128 MiB apart 82.1 -> 84.0, sixteen separate
+// allocations (inputs first) 76.3 -> 79.1, (each rank's input next to its output) 81.7 -> 82.9.  One in flight loses
+// 6 points, three or four gain half as much; two stores with four or eight loads gain 1; fewer workgroups per CU on
+// top of it lose.  Short launches, whose time is latency, keep everything in flight at once: the planner sets
+// kFlatPaced per launch (paced_launch in vrank_plan.cpp).
+constexpr uint32_t kGroupLoadsInFlight = 2;
+constexpr uint32_t kGroupStoresInFlight = 2;
 constexpr uint32_t kGroupMinTiles = 512;
 constexpr uint32_t kFlatGroupMinTiles = 2048;
 // Large flat folds with ONE output (reduce_scatter, reduce, the first launch of the two-phase all_reduce), three

@@ -78,6 +78,33 @@ def test_all_reduce_group_form(dtype):
 
 
 @pytest.mark.parametrize("dtype", REDUCE_TYPES)
+def test_all_reduce_group_form_with_paced_accesses(dtype, monkeypatch):
+    """Long group launches keep two loads and two stores per wavefront in flight instead of all of them (the planner
+    switches it on from a few GiB; MEGRAY_VRANK_PACE=always forces it here at sizes the oracle handles): same results,
+    bit for bit, ragged lengths, every order, out of place and in place."""
+    monkeypatch.setenv("MEGRAY_VRANK_PACE", "always")
+    size = orc.dtype_size(dtype)
+    rng = np.random.default_rng(1077 + dtype)
+    for nranks, tiles in ((3, 4500), (4, 4301), (8, 5051)):
+        length = (tiles * 1024 + 1024 - 16 * (nranks - 1)) // size - 3
+        ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+        for op, order in ((orc.SUM, orc.ORDER_UCX), (orc.MAX, orc.ORDER_SHM), (orc.MIN, orc.ORDER_RANK0)):
+            want = orc.fold_all_reduce(ins, dtype, op, order)
+            for inplace in (False, True):
+                got = run_all_reduce(ins, dtype, op, order, mr.Schedule.FUSED, inplace=inplace)
+                for r in range(nranks):
+                    assert_same(got[r], want[r], f"paced group form dtype={dtype} N={nranks} len={length} op={op} "
+                                                 f"order={order} inplace={inplace} rank={r}")
+    monkeypatch.setenv("MEGRAY_VRANK_PACE", "never")
+    nranks, length = 8, 5051 * 1024 // size + 5
+    ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+    got = run_all_reduce(ins, dtype, orc.SUM, orc.ORDER_UCX, mr.Schedule.FUSED)
+    want = orc.fold_all_reduce(ins, dtype, orc.SUM, orc.ORDER_UCX)
+    for r in range(nranks):
+        assert_same(got[r], want[r], f"unpaced group form dtype={dtype} rank={r}")
+
+
+@pytest.mark.parametrize("dtype", REDUCE_TYPES)
 def test_segment_group_form(dtype):
     """The general fold kernel with long vector bodies (512 groups of 64 vectors and more) runs in its
     group form: rank counts without a flat kernel (5 and 16: the fold count is read from the launch and
