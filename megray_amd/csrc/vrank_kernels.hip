@@ -184,6 +184,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
         if (staged[k] && live)
             store_tile_any(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + tile_off(first + uint64_t(k) * kGroupStride),
                             tid, stage[k][tid]);
+        if (L.paced) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // one store in flight per wavefront
     }
 }
 

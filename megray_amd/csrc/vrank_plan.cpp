@@ -617,6 +617,29 @@ Status plan_all_gather(Plan& plan, const void* const* send, void* const* recv, u
 
 namespace {
 
+// Should the group pack kernel of an all_gather issue a wavefront's N stores one at a time (PackLaunch::paced)?
+// Measured on MI355X, uint8 blocks of 16 / 32 / 64 MiB, % of the HBM peak, all stores at once -> one at a time:
+//   8 ranks, separate allocations                      80.5 - 81.2 -> 83.1 / 82.8 - 83.0 -> 84.2 - 84.5 / 81.3 - 82.5 -> 84.8
+//   8 ranks, outputs placed 128 MiB k + 32 MiB apart   83.4 -> 83.8 - 84.0 / 85.4 -> 84.6 / 84.9 -> 84.7
+//   4 ranks, separate allocations                      78.8 - 79.2 -> 79.1 / 80.8 - 82.1 -> 81.6 - 82.0 / 83.8 - 84.4 -> 83.1 - 83.5
+//   4 ranks, placed                                    81.4 - 81.7 -> 79.7 / 84.4 -> 82.3 / 84.0 - 84.7 -> 83.5
+// and a broadcast loses 3 points at 32 MiB either way.  So: eight ranks and more, a GiB and more written, outputs that
+// do not lie 32 MiB-aligned distances apart that differ in address bits 25 - 31 (what vrank_placement.h gives them).
+bool paced_gather(const void* const* out, uint32_t nranks, uint64_t block_bytes) {
+    if (pace_override() >= 0) return pace_override() == 1;
+    if (nranks < 8 || block_bytes * nranks * nranks < (uint64_t(1) << 30)) return false;
+    constexpr uintptr_t kUnit = uintptr_t(32) << 20;
+    bool placed = true;
+    uint64_t keys[2] = {0, 0};
+    for (uint32_t r = 0; r < nranks && placed; ++r) {
+        const uintptr_t a = reinterpret_cast<uintptr_t>(out[r]);
+        const uint32_t key = uint32_t((a / kUnit) % 128);
+        placed = (a % kUnit) == (reinterpret_cast<uintptr_t>(out[0]) % kUnit) && !(keys[key / 64] >> (key % 64) & 1u);
+        keys[key / 64] |= uint64_t(1) << (key % 64);
+    }
+    return !placed;
+}
+
 uint32_t common_width(uint64_t block_bytes, const void* const* a, const void* const* b, uint32_t n) {
     uintptr_t bits = uintptr_t(block_bytes);
     for (uint32_t r = 0; r < n; ++r) bits |= reinterpret_cast<uintptr_t>(a[r]) | reinterpret_cast<uintptr_t>(b[r]);
@@ -646,6 +669,7 @@ Status add_pack(Plan& plan, const void* const* in, void* const* out, uint32_t nr
     L.width = common_width(block_bytes, in, out_c, nranks);
     const uint64_t tiles = pack_tiles(block_bytes);
     L.waves = tiles >= kGroupMinTiles / 4 ? kGroupWaves : 1;  // long blocks take the group form
+    if (L.waves == kGroupWaves && mode == kPackAllGather) L.paced = paced_gather(out_c, nranks, block_bytes) ? 1 : 0;
     // A grid holds 2^31 - 1 workgroups: blocks whose tiles, over all copies, outnumber that are cut into
     // slices of tiles, one launch each (the reference's per-peer copies have no such limit either).
     const uint64_t span = uint64_t(kGroupWaves) * kGroupStride;  // tiles a run of kGroupStride workgroups covers

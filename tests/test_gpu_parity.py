@@ -396,6 +396,19 @@ def test_pack_collectives_group_form(dtype):
         check_pack_collectives(dtype, nranks, length, 0, rng)
 
 
+@pytest.mark.parametrize("pace", ["always", "never"])
+def test_pack_collectives_group_form_with_paced_stores(pace, monkeypatch):
+    """An all_gather of eight ranks that writes a GiB and more into buffers the library did not place issues a
+    wavefront's stores one at a time; MEGRAY_VRANK_PACE forces that on (and off) here at a size the oracle handles.
+    Same permutations either way."""
+    monkeypatch.setenv("MEGRAY_VRANK_PACE", pace)
+    rng = np.random.default_rng(290)
+    for dtype in (orc.UINT8, orc.FLOAT32):
+        length = (1030 * 1024 + 48) // orc.dtype_size(dtype)
+        for nranks in (3, 8):
+            check_pack_collectives(dtype, nranks, length, 0, rng)
+
+
 def check_pack_collectives(dtype, nranks, length, misalign, rng):
     size = orc.dtype_size(dtype)
     gen = orc.UINT8 if dtype == orc.CHAR else dtype
