@@ -30,7 +30,7 @@ extern "C" {
 
 #define MRV_API __attribute__((visibility("default")))
 
-#define MRV_MAX_RANKS 16
+#define MRV_MAX_RANKS 32
 
 /* Which reference loop fixes the order a chunk's contributions are combined in. */
 enum {

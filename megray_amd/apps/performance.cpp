@@ -256,7 +256,7 @@ void show_help(const char* argv0) {
     std::cout << argv0
               << " {OPTIONS}\n\n    Benchmark of the MegRay API on the MEGRAY_VRANK backend.\n\n  OPTIONS:\n"
                  "      -h          this help\n"
-                 "      -d[int]     number of devs = virtual ranks on GPU 0 (default 2, at most 16)\n"
+                 "      -d[int]     number of devs = virtual ranks on GPU 0 (default 2, at most 32)\n"
                  "      -I[string]  master IP (default 127.0.0.1)\n"
                  "      -P[int]     master port (accepted; every run draws a free port)\n"
                  "      -n[int]     number of nodes: only 1 (all ranks share one GPU)\n"
@@ -334,8 +334,8 @@ int main(int argc, char* argv[]) {
         std::cerr << "this build has one backend: VRANK\n";
         return 1;
     }
-    if (args.n_devs < 1 || args.n_devs > 16 || args.iters < 1) {
-        std::cerr << "need 1 <= -d <= 16 and -i >= 1\n";
+    if (args.n_devs < 1 || args.n_devs > 32 || args.iters < 1) {
+        std::cerr << "need 1 <= -d <= 32 and -i >= 1\n";
         return 1;
     }
     int devices = 0;

@@ -197,7 +197,7 @@ int mrv_fold_order(int collective, int order, uint32_t nranks, uint32_t chunk, u
     return guarded([&] {
         if (collective != MRV_ALL_REDUCE && collective != MRV_REDUCE_SCATTER)
             MEGRAY_THROW("fold orders exist for all_reduce and reduce_scatter");
-        if (nranks < 1 || nranks > kMaxRanks) MEGRAY_THROW("nranks must be in [1, 16]");
+        if (nranks < 1 || nranks > kMaxRanks) MEGRAY_THROW("nranks must be in [1, 32]");
         const FoldOrder fo = as_order(order);
         const Collective coll = collective == MRV_ALL_REDUCE ? kAllReduce : kReduceScatter;
         const uint32_t chunks = order_chunks(fo, nranks);

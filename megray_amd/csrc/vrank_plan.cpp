@@ -184,7 +184,7 @@ private:
         std::memset(&step, 0, sizeof(step));
         step.kind = Step::kFlat;
         FlatLaunch& L = step.flat;
-        for (uint32_t r = 0; r < kMaxRanks; ++r) {
+        for (uint32_t r = 0; r < kFlatMaxRanks; ++r) {  // flat_width(): at most eight ranks
             L.in[r] = m_in[r];
             L.out[r] = m_out[r];
         }
@@ -349,7 +349,7 @@ private:
 };
 
 Status check_ranks(uint32_t nranks) {
-    if (nranks < 1 || nranks > kMaxRanks) return invalid("nranks must be in [1, 16]");
+    if (nranks < 1 || nranks > kMaxRanks) return invalid("nranks must be in [1, 32]");
     return MEGRAY_OK;
 }
 

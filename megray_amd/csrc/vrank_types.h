@@ -8,9 +8,12 @@
 namespace MegRay {
 namespace vrank {
 
-constexpr uint32_t kMaxRanks = 16;            // virtual ranks per group
+constexpr uint32_t kMaxRanks = 32;            // virtual ranks per group (the pointer tables of a launch descriptor)
+constexpr uint32_t kFlatMaxRanks = 8;         // ... of a flat launch, whose kernels exist for 2, 3, 4 and 8 ranks
 constexpr uint32_t kMaxChunks = 2 * kMaxRanks;  // the shm order splits a buffer into 2N chunks
-constexpr uint32_t kMaxSegments = 3 * kMaxChunks;  // head / aligned body / tail per chunk
+// Segments one general launch descriptor holds (a chunk gives a head, an aligned body and a tail); a collective with
+// more of them is cut into several launches.  With the pointer tables the descriptor stays below 4 KiB.
+constexpr uint32_t kMaxSegments = 96;
 constexpr uint32_t kThreads = 64;             // one 64-wide wavefront per tile (measured best: 1 KiB per buffer per tile)
 constexpr uint32_t kVecBytes = 16;            // one 128-bit global load / store per lane
 
@@ -93,8 +96,8 @@ constexpr uint32_t flat_meta(uint32_t start, int dir, uint32_t out_first) {
 // input pointers, eight output pointers, the scalars, eight run ends, eight run words: five lines for
 // an all_reduce of eight ranks) and tables a launch does not need (shifts) are never read.
 struct FlatLaunch {
-    const void* in[kMaxRanks];
-    void* out[kMaxRanks];
+    const void* in[kFlatMaxRanks];
+    void* out[kFlatMaxRanks];
     // one line of scalars
     uint64_t count;          // elements per input buffer
     uint64_t hook_target;    // 0: do not wait (see EdgeHooks)

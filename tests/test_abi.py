@@ -60,7 +60,7 @@ def test_chunk_partition_matches_oracle():
 
 def test_fold_order_matches_oracle():
     import megray_amd as mr
-    for nranks in range(1, 17):
+    for nranks in range(1, 33):
         for coll in (orc.COLL_ALL_REDUCE, orc.COLL_REDUCE_SCATTER):
             for order in (orc.ORDER_UCX, orc.ORDER_SHM, orc.ORDER_RANK0):
                 nchunks = orc.fold_order(coll, order, nranks, 0)[2]
@@ -71,7 +71,7 @@ def test_fold_order_matches_oracle():
                 with pytest.raises(mr.MegRayError):
                     mr.fold_order(coll, order, nranks, nchunks)
     with pytest.raises(mr.MegRayError):
-        mr.fold_order(0, 0, 17, 0)
+        mr.fold_order(0, 0, 33, 0)
     with pytest.raises(mr.MegRayError):
         mr.fold_order(0, 5, 4, 0)
 

@@ -134,7 +134,7 @@ def test_group_rendezvous_without_gpu():
     for c in comms:
         c.close()
     with pytest.raises(mr.MegRayError):
-        mr.Communicator(17, 0)  # more ranks than the backend takes
+        mr.Communicator(33, 0)  # more ranks than the backend takes
 
 
 def test_a_rank_that_rejects_its_arguments_releases_the_others_without_gpu():

@@ -53,6 +53,38 @@ def test_all_reduce_fused_all_orders(dtype, nranks):
                                                  f"order={order} rank={r}")
 
 
+@pytest.mark.parametrize("nranks", [17, 24, 32])
+def test_more_than_sixteen_ranks(nranks):
+    """The reference's get_communicator takes any rank count (include/megray.h:33-34); this backend takes up to 32
+    virtual ranks.  Every collective at 17, 24 and 32 ranks against the oracle's literal replays: the folds in all three
+    orders (more chunks than one launch descriptor holds segments for: several launches), reduce towards a root in the
+    tree order, and the block copies; short and long (group form) lengths."""
+    rng = np.random.default_rng(3200 + nranks)
+    for dtype, length in ((orc.FLOAT32, 5 * nranks + 3), (orc.INT8, 40001), (orc.FLOAT32, 300 * 1024 + 7), (orc.FLOAT16, 2 * 1024 * 1024 + 11)):
+        ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+        for op, order in ((orc.SUM, orc.ORDER_UCX), (orc.MAX, orc.ORDER_SHM), (orc.MIN, orc.ORDER_RANK0)):
+            want = orc.fold_all_reduce(ins, dtype, op, order)
+            got = run_all_reduce(ins, dtype, op, order, mr.Schedule.FUSED)
+            for r in range(nranks):
+                assert_same(got[r], want[r], f"all_reduce N={nranks} dtype={dtype} len={length} op={op} order={order} rank={r}")
+        if dtype != orc.FLOAT16:
+            root = nranks - 2
+            out = empty_device(length * orc.dtype_size(dtype))
+            mr.reduce_to_root([to_device(x) for x in ins], out, length, dtype, orc.SUM, root)
+            torch.cuda.synchronize()
+            assert_same(to_host(out, ins[0].dtype), orc.ucx_reduce(ins, dtype, orc.SUM, root)[root], f"reduce N={nranks} dtype={dtype}")
+    recvlen = 1000 + nranks
+    ins = [rand_array(orc.FLOAT32, recvlen * nranks, rng) for _ in range(nranks)]
+    d_out = [empty_device(recvlen * 4) for _ in range(nranks)]
+    mr.reduce_scatter([to_device(x) for x in ins], d_out, recvlen, orc.FLOAT32, orc.SUM)
+    torch.cuda.synchronize()
+    want = orc.ucx_reduce_scatter(ins, orc.FLOAT32, orc.SUM)
+    for r in range(nranks):
+        assert_same(to_host(d_out[r], np.float32), want[r], f"reduce_scatter N={nranks} rank={r}")
+    for length in (77, 140 * 1024 + 5):
+        check_pack_collectives(orc.UINT8, nranks, length, 0, rng)
+
+
 @pytest.mark.parametrize("dtype", REDUCE_TYPES)
 def test_all_reduce_group_form(dtype):
     """Launches of 2048 tiles and more take the group form of the flat kernel (four wavefronts per
@@ -529,7 +561,7 @@ def test_errors_follow_the_reference():
     with pytest.raises(mr.MegRayError, match="overlap"):
         mr.all_reduce([d, d], [o, o], 64, mr.DType.FLOAT32, mr.ReduceOp.SUM)
     with pytest.raises(mr.MegRayError, match="nranks"):
-        mr.all_reduce([d] * 17, [o] * 17, 1, mr.DType.FLOAT32, mr.ReduceOp.SUM)
+        mr.all_reduce([d] * 33, [o] * 33, 1, mr.DType.FLOAT32, mr.ReduceOp.SUM)
     torch.cuda.synchronize()
 
 
