@@ -548,21 +548,36 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
         // a copy: nothing to skew on the load side
         if (have) acc.seed(load_tile_any(static_cast<const char*>(L.in[sv.start]) + in_base + mine * kGroupBytes, tid));
     } else {
+        // Long launches keep two loads per wavefront in flight instead of all SK (L.paced, as in the flat group
+        // kernel): load q + 2 is issued when load q has arrived.
+        const bool paced = L.paced != 0;
+        constexpr uint32_t D = SK < kGroupLoadsInFlight ? SK : kGroupLoadsInFlight;
         for (uint32_t j0 = 0; j0 < nfold; j0 += SK) {
-            u32x4 x[SK];
-#pragma unroll
-            for (uint32_t q = 0; q < SK; ++q) {
+            const auto load_input = [&](uint32_t q, uint32_t lane) -> u32x4 {
                 const uint64_t group = first + ((wave + q) % W) * kGroupStride;
                 if (j0 + q < nfold && group < whole_groups)
-                    x[q] = load_tile_any(static_cast<const char*>(L.in[rotate_rank(sv.start, sv.dir, j0 + q, nr)]) +
+                    return load_tile_any(static_cast<const char*>(L.in[rotate_rank(sv.start, sv.dir, j0 + q, nr)]) +
                                                  in_base + group * kGroupBytes,
-                                         tid);
-                else
-                    x[q] = u32x4{0u, 0u, 0u, 0u};
+                                         lane);
+                return u32x4{0u, 0u, 0u, 0u};
+            };
+            u32x4 x[SK];
+#pragma unroll
+            for (uint32_t q = 0; q < D; ++q) x[q] = load_input(q, tid);
+            if (!paced) {
+#pragma unroll
+                for (uint32_t q = D; q < SK; ++q) x[q] = load_input(q, tid);
             }
             if (K == 0 && j0) __syncthreads();  // the previous four have been folded by everyone
 #pragma unroll
-            for (uint32_t q = 0; q < SK; ++q) stage[(wave + q) % W][q][tid] = x[q];
+            for (uint32_t q = 0; q < SK; ++q) {
+                if (paced && q + D < SK) {
+                    uint32_t lane = tid;
+                    asm volatile("" : "+v"(lane) : "v"(x[q]));  // the next load's address waits for x[q]
+                    x[q + D] = load_input(q + D, lane);
+                }
+                stage[(wave + q) % W][q][tid] = x[q];
+            }
             __syncthreads();
             if (have) {
 #pragma unroll
@@ -594,6 +609,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
             store_tile_any(static_cast<char*>(L.out[rotate_rank(sv.out_first, 1, m, nr)]) + out_base +
                                    (first + uint64_t(k) * kGroupStride) * kGroupBytes,
                            tid, result[k][tid]);
+        if (L.paced && (m + 1) % kGroupStoresInFlight == 0 && m + 1 < nout) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
 }
 

@@ -44,7 +44,10 @@ int pace_override() {
 //   3 ranks, separate allocations                          79.7 -> 80.4 / 83.4 -> 83.3 / 84.0 -> 83.7 / 82.1 -> 83.5 / 81.8 -> 84.2
 // So: buffers that do not lie the way vrank_placement.h lays them out pace from 3 GiB over all of them; buffers
 // that do, only eight-rank launches of 12 GiB and more (where it is worth a few tenths).
-bool paced_launch(const void* const* in, const void* const* out, uint32_t nranks, uint64_t bytes) {
+// The general group kernel (other rank counts, buffers off the 16-byte grid) behaves alike on separate allocations
+// (5 / 7 / 12 / 16 ranks x 512 MiB: 79.4 -> 82.9 / 79.2 -> 81.3 / 76.4 -> 79.3 / 74.8 -> 78.3; x 256 MiB + 1 throughout;
+// x 64 MiB - 1) and loses half a point to a point on placed buffers, where it is left alone (`flat` false).
+bool paced_launch(const void* const* in, const void* const* out, uint32_t nranks, uint64_t bytes, bool flat = true) {
     if (pace_override() >= 0) return pace_override() == 1;
     const void* seen[2 * kMaxRanks];
     uint32_t n = 0;
@@ -68,7 +71,7 @@ bool paced_launch(const void* const* in, const void* const* out, uint32_t nranks
     }
     const uint64_t total = uint64_t(n) * bytes;
     constexpr uint64_t kGiB = uint64_t(1) << 30;
-    return placed ? (nranks >= 8 && total >= 12 * kGiB) : total >= 3 * kGiB;
+    return placed ? (flat && nranks >= 8 && total >= 12 * kGiB) : total >= 3 * kGiB;
 }
 
 bool overlaps(const void* a, uint64_t a_bytes, const void* b, uint64_t b_bytes) {
@@ -238,6 +241,7 @@ private:
         for (const Run& r : m_runs)
             if (natural || same_phase(r)) vector_elems += r.count;
         m_waves = vector_elems / (kThreads * epv) >= kGroupMinTiles ? kGroupWaves : 1;
+        m_paced = m_waves == kGroupWaves && m_nfold >= 3 && paced_launch(m_in, m_out, m_nranks, vector_elems * m_elem, false);
         open_launch();
         for (const Run& r : m_runs) {
             const bool vector = natural || same_phase(r);
@@ -293,6 +297,7 @@ private:
         m_launch.new_wins_ties = m_new_wins ? 1 : 0;
         m_launch.elem_size = m_elem;
         m_launch.waves = m_waves;
+        m_launch.paced = m_paced ? 1 : 0;
     }
 
     void close_launch() {
@@ -344,6 +349,7 @@ private:
     uint64_t m_grid = kVecBytes;
     bool m_tree = false;
     uint32_t m_waves = 1;
+    bool m_paced = false;
     std::vector<Run> m_runs;
     FoldLaunch m_launch;
 };

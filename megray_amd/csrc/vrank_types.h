@@ -68,6 +68,8 @@ struct FoldLaunch {
     uint32_t new_wins_ties;  // float MAX/MIN: an equal / unordered compare keeps the newcomer
     uint32_t elem_size;
     uint32_t waves;          // wavefronts per workgroup: 1, or 4 for the group form (long vector bodies)
+    uint32_t paced;          // group form: a wavefront keeps two loads and two stores in flight (as kFlatPaced)
+    uint32_t reserved;
     EdgeHooks hooks;         // one wavefront per workgroup only
     uint64_t hook_target;
     uint64_t hook_ticket;

@@ -127,6 +127,15 @@ def test_all_reduce_group_form_with_paced_accesses(dtype, monkeypatch):
                 for r in range(nranks):
                     assert_same(got[r], want[r], f"paced group form dtype={dtype} N={nranks} len={length} op={op} "
                                                  f"order={order} inplace={inplace} rank={r}")
+    # the general group kernel paces the same way: five ranks (inputs staged four at a time), and three ranks whose
+    # buffers share an offset from a 16-byte boundary
+    for nranks, offset in ((5, 0), (3, max(size, 4))):
+        length = 4300 * 1024 // size + 7
+        ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+        want = orc.fold_all_reduce(ins, dtype, orc.SUM, orc.ORDER_UCX)
+        got = run_all_reduce(ins, dtype, orc.SUM, orc.ORDER_UCX, mr.Schedule.FUSED, offsets=[offset] * nranks)
+        for r in range(nranks):
+            assert_same(got[r], want[r], f"paced segment group form dtype={dtype} N={nranks} offset={offset} rank={r}")
     monkeypatch.setenv("MEGRAY_VRANK_PACE", "never")
     nranks, length = 8, 5051 * 1024 // size + 5
     ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
