@@ -1,5 +1,9 @@
 #include "vrank_engine.h"
 
+#include <cstdlib>
+#include <cstring>
+#include <memory>
+
 #include "megray/hip_context.h"
 #include "vrank_kernels.h"
 
@@ -123,6 +127,111 @@ Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCal
     return MEGRAY_OK;
 }
 
+namespace {
+
+// The flat entry points plan on every call, and planning a small collective costs as much as launching it (the
+// reference re-derives its chunking per call as well, src/ucx/all_reduce.cpp:33-51).  Callers repeat their
+// collectives on the same buffers, so each thread keeps the last few plans, found by everything a plan depends on:
+// the collective, its arguments and the buffer addresses.  (The communicator keeps such a cache per group, and
+// mrv_plan_* lets a caller hold a plan explicitly.)
+struct FlatKey {
+    int kind, order, sched, pace;
+    uint32_t nranks, root;
+    size_t count;
+    DType dtype;
+    ReduceOp op;
+    int device;
+    const void* send[kMaxRanks];
+    void* recv[kMaxRanks];
+};
+
+struct FlatEntry {
+    FlatKey key;
+    uint64_t signature = 0;  // a mix of the key's words: compared first
+    uint64_t last_used = 0;
+    Plan plan;
+    std::vector<KernelCall> calls;  // point into `plan`
+};
+
+constexpr size_t kFlatCacheSlots = 16;
+
+bool same_key(const FlatKey& a, const FlatKey& b) {
+    return a.kind == b.kind && a.order == b.order && a.sched == b.sched && a.pace == b.pace && a.nranks == b.nranks &&
+           a.root == b.root && a.count == b.count && a.dtype == b.dtype && a.op == b.op && a.device == b.device &&
+           std::memcmp(a.send, b.send, sizeof(a.send)) == 0 && std::memcmp(a.recv, b.recv, sizeof(a.recv)) == 0;
+}
+
+uint64_t key_signature(const FlatKey& key) {
+    static_assert(sizeof(FlatKey) % sizeof(uint64_t) == 0, "the key is hashed word by word");
+    uint64_t words[sizeof(FlatKey) / sizeof(uint64_t)];
+    std::memcpy(words, &key, sizeof(key));
+    uint64_t h = 0x9e3779b97f4a7c15ull;
+    for (uint64_t w : words) {
+        h ^= w + 0x9e3779b97f4a7c15ull + (h << 6) + (h >> 2);
+        h *= 0xff51afd7ed558ccdull;
+    }
+    return h ^ (h >> 32);
+}
+
+int pace_choice() {
+    const char* text = std::getenv("MEGRAY_VRANK_PACE");  // the planner reads it too: part of what a plan depends on
+    return !text ? -1 : std::strcmp(text, "always") == 0 ? 1 : std::strcmp(text, "never") == 0 ? 0 : -1;
+}
+
+}  // namespace
+
+Status run_collective(int kind, const void* const* send, void* const* recv, uint32_t nranks, size_t count, DType dtype,
+                      ReduceOp op, int order, int schedule, uint32_t root, hipStream_t stream) {
+    if (nranks < 1 || nranks > kMaxRanks) {  // the planner says so; nothing to remember
+        Plan plan;
+        const Status st = plan_collective(plan, kind, send, recv, nranks, count, dtype, order, schedule, root);
+        return st == MEGRAY_OK ? execute(plan, dtype, is_reduction(kind) ? op : MEGRAY_SUM, stream) : st;
+    }
+    thread_local std::vector<std::unique_ptr<FlatEntry>> cache;
+    thread_local uint64_t clock = 0;
+    FlatKey key;
+    std::memset(&key, 0, sizeof(key));
+    key.kind = kind, key.order = order, key.sched = schedule, key.pace = pace_choice();
+    key.nranks = nranks, key.root = root, key.count = count, key.dtype = dtype, key.op = is_reduction(kind) ? op : MEGRAY_SUM;
+    if (hipGetDevice(&key.device) != hipSuccess) {
+        (void)hipGetLastError();
+        key.device = -1;
+    }
+    // which pointers a collective looks at: the rooted ones only their root's on one side
+    const bool send_root_only = kind == kCollScatter || kind == kCollBroadcast;
+    const bool recv_root_only = kind == kCollGather || kind == kCollReduce;
+    const uint32_t nsend = kind == kCollReduce2 ? 2 : nranks, nrecv = kind == kCollReduce2 ? 1 : nranks;
+    for (uint32_t r = 0; r < nsend; ++r)
+        if (!send_root_only || r == root) key.send[r] = send[r];
+    for (uint32_t r = 0; r < nrecv; ++r)
+        if (!recv_root_only || r == root) key.recv[r] = recv[r];
+    const uint64_t signature = key_signature(key);
+    FlatEntry* hit = nullptr;
+    for (auto& e : cache)
+        if (e->signature == signature && same_key(e->key, key)) hit = e.get();
+    if (!hit) {
+        auto fresh = std::make_unique<FlatEntry>();
+        fresh->key = key;
+        fresh->signature = signature;
+        Status st = plan_collective(fresh->plan, kind, send, recv, nranks, count, dtype, order, schedule, root);
+        if (st == MEGRAY_OK) st = resolve(fresh->plan, dtype, key.op, fresh->calls);
+        if (st != MEGRAY_OK) return st;
+        if (cache.size() < kFlatCacheSlots) {
+            cache.push_back(std::move(fresh));
+            hit = cache.back().get();
+        } else {
+            size_t oldest = 0;
+            for (size_t i = 1; i < cache.size(); ++i)
+                if (cache[i]->last_used < cache[oldest]->last_used) oldest = i;
+            cache[oldest] = std::move(fresh);
+            hit = cache[oldest].get();
+        }
+    }
+    hit->last_used = ++clock;
+    for (const KernelCall& call : hit->calls) HIP_CHECK(enqueue(call.kernel, call.grid, call.block, call.launch, stream, call.lds));
+    return MEGRAY_OK;
+}
+
 Status execute(const Plan& plan, DType dtype, ReduceOp op, hipStream_t stream) {
     std::vector<KernelCall> calls;
     const Status st = resolve(plan, dtype, op, calls);
@@ -133,76 +242,84 @@ Status execute(const Plan& plan, DType dtype, ReduceOp op, hipStream_t stream) {
 
 Status reduce2(const void* i0, const void* i1, void* o, size_t len, DType dtype, ReduceOp op,
                hipStream_t stream) {
-    const uint32_t size = reduce_elem_size(dtype);
+    (void)reduce_elem_size(dtype);
     check_reduce_op(op);
-    Plan plan;
-    Status st = plan_reduce2(plan, i0, i1, o, len, size);
-    return st == MEGRAY_OK ? execute(plan, dtype, op, stream) : st;
+    const void* send[2] = {i0, i1};
+    void* recv[1] = {o};
+    return run_collective(kCollReduce2, send, recv, 2, len, dtype, op, kOrderUcx, kSchedFused, 0, stream);
 }
 
 Status all_reduce(const void* const* send, void* const* recv, uint32_t nranks, size_t len, DType dtype,
                   ReduceOp op, FoldOrder order, Schedule sched, hipStream_t stream) {
-    const uint32_t size = reduce_elem_size(dtype);
+    (void)reduce_elem_size(dtype);
     check_reduce_op(op);
-    // a ring hop stores its partial result in the element type: FLOAT16 would round N-1 times
-    if (sched == kSchedRing && dtype == MEGRAY_FLOAT16)
-        MEGRAY_THROW("the ring schedule is not offered for FLOAT16 (it would round at every hop)");
-    Plan plan;
-    Status st = plan_all_reduce(plan, send, recv, nranks, len, size, order, sched);
-    return st == MEGRAY_OK ? execute(plan, dtype, op, stream) : st;
+    return run_collective(kCollAllReduce, send, recv, nranks, len, dtype, op, order, sched, 0, stream);
 }
 
 Status reduce_scatter(const void* const* send, void* const* recv, uint32_t nranks, size_t recvlen,
                       DType dtype, ReduceOp op, FoldOrder order, hipStream_t stream) {
-    const uint32_t size = reduce_elem_size(dtype);
+    (void)reduce_elem_size(dtype);
     check_reduce_op(op);
-    Plan plan;
-    Status st = plan_reduce_scatter(plan, send, recv, nranks, recvlen, size, order, kSchedFused);
-    return st == MEGRAY_OK ? execute(plan, dtype, op, stream) : st;
+    return run_collective(kCollReduceScatter, send, recv, nranks, recvlen, dtype, op, order, kSchedFused, 0, stream);
 }
+
+namespace {
+// The rooted collectives' one-sided argument as a per-rank table with the root's entry set.
+struct RootTable {
+    const void* send[kMaxRanks] = {};
+    void* recv[kMaxRanks] = {};
+};
+void check_root(uint32_t nranks, uint32_t root) {
+    if (nranks < 1 || nranks > kMaxRanks) MEGRAY_THROW("nranks must be in [1, 32]");
+    if (root >= nranks) MEGRAY_THROW("root out of range");
+}
+}  // namespace
 
 Status reduce_to_root(const void* const* send, void* recv_root, uint32_t nranks, size_t len, DType dtype,
                       ReduceOp op, FoldOrder order, uint32_t root, hipStream_t stream) {
-    const uint32_t size = reduce_elem_size(dtype);
+    (void)reduce_elem_size(dtype);
     check_reduce_op(op);
-    Plan plan;
-    Status st = plan_reduce(plan, send, recv_root, nranks, len, size, order, root);
-    return st == MEGRAY_OK ? execute(plan, dtype, op, stream) : st;
+    check_root(nranks, root);
+    RootTable t;
+    t.recv[root] = recv_root;
+    return run_collective(kCollReduce, send, t.recv, nranks, len, dtype, op, order, kSchedFused, root, stream);
 }
 
 Status all_gather(const void* const* send, void* const* recv, uint32_t nranks, size_t sendlen, DType dtype,
                   hipStream_t stream) {
-    Plan plan;
-    Status st = plan_all_gather(plan, send, recv, nranks, sendlen, uint32_t(get_dtype_size(dtype)));
-    return st == MEGRAY_OK ? execute(plan, dtype, MEGRAY_SUM, stream) : st;
+    return run_collective(kCollAllGather, send, recv, nranks, sendlen, dtype, MEGRAY_SUM, kOrderUcx, kSchedFused, 0, stream);
 }
 
 Status all_to_all(const void* const* send, void* const* recv, uint32_t nranks, size_t len, DType dtype,
                   hipStream_t stream) {
-    Plan plan;
-    Status st = plan_all_to_all(plan, send, recv, nranks, len, uint32_t(get_dtype_size(dtype)));
-    return st == MEGRAY_OK ? execute(plan, dtype, MEGRAY_SUM, stream) : st;
+    return run_collective(kCollAllToAll, send, recv, nranks, len, dtype, MEGRAY_SUM, kOrderUcx, kSchedFused, 0, stream);
 }
 
 Status scatter(const void* send_root, void* const* recv, uint32_t nranks, size_t recvlen, DType dtype,
                uint32_t root, hipStream_t stream) {
-    Plan plan;
-    Status st = plan_scatter(plan, send_root, recv, nranks, recvlen, uint32_t(get_dtype_size(dtype)), root);
-    return st == MEGRAY_OK ? execute(plan, dtype, MEGRAY_SUM, stream) : st;
+    (void)get_dtype_size(dtype);
+    check_root(nranks, root);
+    RootTable t;
+    t.send[root] = send_root;
+    return run_collective(kCollScatter, t.send, recv, nranks, recvlen, dtype, MEGRAY_SUM, kOrderUcx, kSchedFused, root, stream);
 }
 
 Status gather(const void* const* send, void* recv_root, uint32_t nranks, size_t sendlen, DType dtype,
               uint32_t root, hipStream_t stream) {
-    Plan plan;
-    Status st = plan_gather(plan, send, recv_root, nranks, sendlen, uint32_t(get_dtype_size(dtype)), root);
-    return st == MEGRAY_OK ? execute(plan, dtype, MEGRAY_SUM, stream) : st;
+    (void)get_dtype_size(dtype);
+    check_root(nranks, root);
+    RootTable t;
+    t.recv[root] = recv_root;
+    return run_collective(kCollGather, send, t.recv, nranks, sendlen, dtype, MEGRAY_SUM, kOrderUcx, kSchedFused, root, stream);
 }
 
 Status broadcast(const void* send_root, void* const* recv, uint32_t nranks, size_t len, DType dtype,
                  uint32_t root, hipStream_t stream) {
-    Plan plan;
-    Status st = plan_broadcast(plan, send_root, recv, nranks, len, uint32_t(get_dtype_size(dtype)), root);
-    return st == MEGRAY_OK ? execute(plan, dtype, MEGRAY_SUM, stream) : st;
+    (void)get_dtype_size(dtype);
+    check_root(nranks, root);
+    RootTable t;
+    t.send[root] = send_root;
+    return run_collective(kCollBroadcast, t.send, recv, nranks, len, dtype, MEGRAY_SUM, kOrderUcx, kSchedFused, root, stream);
 }
 
 }  // namespace vrank

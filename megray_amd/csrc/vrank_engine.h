@@ -60,6 +60,11 @@ Status execute(const Plan& plan, DType dtype, ReduceOp op, hipStream_t stream);
 // The same launches, resolved but not enqueued.
 Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCall>& calls);
 
+// Plans collective `kind` (or finds the plan among the calling thread's last few: same arguments, same buffer
+// addresses) and enqueues it.  The flat entry points below all end here.
+Status run_collective(int kind, const void* const* send, void* const* recv, uint32_t nranks, size_t count, DType dtype,
+                      ReduceOp op, int order, int schedule, uint32_t root, hipStream_t stream);
+
 Status reduce2(const void* i0, const void* i1, void* o, size_t len, DType dtype, ReduceOp op,
                hipStream_t stream);
 Status all_reduce(const void* const* send, void* const* recv, uint32_t nranks, size_t len, DType dtype,
