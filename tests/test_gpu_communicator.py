@@ -252,9 +252,9 @@ def test_random_data_orders_and_work_queued_on_rank_streams(nranks):
 
 def test_ranks_that_share_a_stream_and_ranks_that_stop_sharing_it():
     """Ranks on one stream need no cross-stream edges, and a rank skips marking its stream when everyone
-    shared it last time.  Round 1: all four ranks on the default stream.  Round 2: ranks 1 and 3 move to
+    shared it last time.  First pass: all four ranks on the default stream.  Second pass: ranks 1 and 3 move to
     streams of their own, fill their inputs there right before the collective and read the result there
-    right after - the leader has to insert the edges those ranks did not announce.  Round 3: all share
+    right after - the leader has to insert the edges those ranks did not announce.  Third pass: all share
     again."""
     nranks, length = 4, 1 << 16
     rng = np.random.default_rng(99)
