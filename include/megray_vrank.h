@@ -172,7 +172,8 @@ typedef struct mrv_plan_run {
     uint64_t count;         /* fold: elements; pack: bytes */
     uint32_t deal;          /* fold, group form: 1 = the run's tiles share cache lines with their neighbours, so runs of
                                workgroups are dealt to one XCD (one L2) each; pack decides this per copy on the device */
-    uint32_t reserved;
+    uint32_t paced;         /* group form: 1 = the launch spaces its accesses out (a wavefront keeps two loads and two stores in
+                               flight; a pack launch issues a wavefront's stores one at a time): long launches, see vrank_plan.cpp */
 } mrv_plan_run;
 
 /*

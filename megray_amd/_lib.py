@@ -18,7 +18,7 @@ class PlanRun(ctypes.Structure):
         ("start", ctypes.c_uint32), ("dir", ctypes.c_int32), ("out_first", ctypes.c_uint32),
         ("tiles", ctypes.c_uint32), ("reads_recv", ctypes.c_uint32), ("waves", ctypes.c_uint32),
         ("in_begin", ctypes.c_uint64), ("out_begin", ctypes.c_uint64),
-        ("count", ctypes.c_uint64), ("deal", ctypes.c_uint32), ("reserved", ctypes.c_uint32),
+        ("count", ctypes.c_uint64), ("deal", ctypes.c_uint32), ("paced", ctypes.c_uint32),
     ]
 
 

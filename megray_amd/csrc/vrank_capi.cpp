@@ -338,6 +338,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.vector = (sg.flags & kSegVector) ? 1 : 0;
                     run.waves = L.waves;
                     run.deal = (L.waves == kGroupWaves && (sg.flags & kSegDeal)) ? 1 : 0;
+                    run.paced = L.paced;
                     run.start = sg.start;
                     run.dir = sg.dir;
                     run.out_first = sg.out_first;
@@ -368,6 +369,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.vector = 2;
                     run.waves = L.waves;
                     run.deal = (L.exchange & 2u) ? 1 : 0;
+                    run.paced = (L.exchange & kFlatPaced) ? 1 : 0;
                     run.start = start;
                     run.dir = L.tree ? 0 : int(int8_t((L.meta[s] >> 8) & 0xffu));
                     run.out_first = out_first;
@@ -416,6 +418,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.nout = 1;
                     run.vector = L.width;
                     run.waves = L.waves;
+                    run.paced = L.paced;
                     run.dir = 1;
                     run.tiles = L.tiles_per_copy;
                     run.count = slice_bytes;

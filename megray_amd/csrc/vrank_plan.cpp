@@ -46,8 +46,16 @@ int pace_override() {
 // that do, only eight-rank launches of 12 GiB and more (where it is worth a few tenths).
 // The general group kernel (other rank counts, buffers off the 16-byte grid) behaves alike on separate allocations
 // (5 / 7 / 12 / 16 ranks x 512 MiB: 79.4 -> 82.9 / 79.2 -> 81.3 / 76.4 -> 79.3 / 74.8 -> 78.3; x 256 MiB + 1 throughout;
-// x 64 MiB - 1) and loses half a point to a point on placed buffers, where it is left alone (`flat` false).
-bool paced_launch(const void* const* in, const void* const* out, uint32_t nranks, uint64_t bytes, bool flat = true) {
+// x 64 MiB - 1) and loses half a point to a point on placed buffers, where it is left alone (`flat` false) - unless
+// it folds into ONE output (`nout` 1: a reduce_scatter of 3, 5, 6, 7, 9 ... ranks, whose blocks start off the tile
+// grid).  That shape gains wherever the buffers lie, placed / separate, per-rank buffers of 32 / 128 / 512 MiB:
+//   5 ranks   75.6 -> 74.8 / 75.7 -> 74.3     79.1 -> 82.6 / 79.1 -> 82.6     79.9 -> 85.0 / 79.7 -> 84.6
+//   6 ranks   76.7 -> 77.7 / 75.2 -> 76.3     78.1 -> 80.9 / 78.3 -> 80.8     79.8 -> 82.2 / 79.5 -> 81.2
+//   7 ranks   74.4 -> 76.0 / 73.1 -> 76.6     77.8 -> 81.1 / 77.8 -> 81.2     79.4 -> 81.8 / 79.2 -> 81.3
+// (3 / 10 / 12 ranks x 256 MiB placed: 81.0 -> 83.2 / 78.0 -> 81.0 / 77.4 -> 81.1; 16 ranks 83.4 -> 83.5), and paces from
+// 1 GiB over all its buffers.
+bool paced_launch(const void* const* in, const void* const* out, uint32_t nranks, uint64_t bytes, bool flat = true,
+                  uint32_t nout = 0) {
     if (pace_override() >= 0) return pace_override() == 1;
     const void* seen[2 * kMaxRanks];
     uint32_t n = 0;
@@ -71,6 +79,7 @@ bool paced_launch(const void* const* in, const void* const* out, uint32_t nranks
     }
     const uint64_t total = uint64_t(n) * bytes;
     constexpr uint64_t kGiB = uint64_t(1) << 30;
+    if (!flat && nout == 1 && total >= kGiB) return true;
     return placed ? (flat && nranks >= 8 && total >= 12 * kGiB) : total >= 3 * kGiB;
 }
 
@@ -241,7 +250,7 @@ private:
         for (const Run& r : m_runs)
             if (natural || same_phase(r)) vector_elems += r.count;
         m_waves = vector_elems / (kThreads * epv) >= kGroupMinTiles ? kGroupWaves : 1;
-        m_paced = m_waves == kGroupWaves && m_nfold >= 3 && paced_launch(m_in, m_out, m_nranks, vector_elems * m_elem, false);
+        m_paced = m_waves == kGroupWaves && m_nfold >= 3 && paced_launch(m_in, m_out, m_nranks, vector_elems * m_elem, false, m_nout);
         open_launch();
         for (const Run& r : m_runs) {
             const bool vector = natural || same_phase(r);
@@ -623,27 +632,51 @@ Status plan_all_gather(Plan& plan, const void* const* send, void* const* recv, u
 
 namespace {
 
-// Should the group pack kernel of an all_gather issue a wavefront's N stores one at a time (PackLaunch::paced)?
-// Measured on MI355X, uint8 blocks of 16 / 32 / 64 MiB, % of the HBM peak, all stores at once -> one at a time:
-//   8 ranks, separate allocations                      80.5 - 81.2 -> 83.1 / 82.8 - 83.0 -> 84.2 - 84.5 / 81.3 - 82.5 -> 84.8
-//   8 ranks, outputs placed 128 MiB k + 32 MiB apart   83.4 -> 83.8 - 84.0 / 85.4 -> 84.6 / 84.9 -> 84.7
-//   4 ranks, separate allocations                      78.8 - 79.2 -> 79.1 / 80.8 - 82.1 -> 81.6 - 82.0 / 83.8 - 84.4 -> 83.1 - 83.5
-//   4 ranks, placed                                    81.4 - 81.7 -> 79.7 / 84.4 -> 82.3 / 84.0 - 84.7 -> 83.5
-// and a broadcast loses 3 points at 32 MiB either way.  So: eight ranks and more, a GiB and more written, outputs that
-// do not lie 32 MiB-aligned distances apart that differ in address bits 25 - 31 (what vrank_placement.h gives them).
-bool paced_gather(const void* const* out, uint32_t nranks, uint64_t block_bytes) {
+// Should the group pack kernel of an all_gather or a broadcast issue a wavefront's N stores one at a time
+// (PackLaunch::paced)?  A paced wavefront lives N round trips, which costs a short launch and gains a long one: the
+// memory serves N streams of stores better when they do not arrive N at a time.  Measured on MI355X, % of the HBM peak,
+// all stores at once -> one at a time.
+// all_gather, fp32, outputs of 32 / 128 / 512 MiB per rank (blocks of 1 / N of that), on outputs an odd multiple of
+// 128 MiB apart | 128 MiB k + 32 MiB apart (the placement's all_gather rule) | allocated one by one:
+//   4 ranks   81.8 -> 77.5 | 82.0 -> 77.1 | 81.2 -> 77.3     80.1 -> 82.4 | 84.5 -> 82.7 | 79.6 -> 82.3     82.6 -> 84.4 | 85.5 -> 84.5 | 82.6 -> 84.4
+//   5 ranks   78.5 -> 75.6 | 78.9 -> 75.7 | 83.2 -> 76.0     83.1 -> 81.7 | 83.3 -> 82.2 | 81.8 -> 81.6     81.0 -> 83.7 | 81.6 -> 83.7 | 80.4 -> 83.6
+//   6 ranks   78.6 -> 77.0 | 78.9 -> 76.6 | 83.4 -> 79.6     81.6 -> 82.6 | 82.6 -> 83.0 | 80.0 -> 82.3     79.3 -> 83.8 | 77.9 -> 84.0 | 80.9 -> 84.2
+//   7 ranks   78.3 -> 77.8 | 79.3 -> 77.6 | 82.1 -> 80.3     81.4 -> 83.2 | 82.7 -> 83.4 | 80.1 -> 82.6     79.5 -> 83.9 | 77.3 -> 83.6 | 79.4 -> 84.3
+//   8 ranks   84.1 -> 81.5 | 84.9 -> 81.1 | 84.0 -> 80.9     79.7 -> 84.0 | 84.1 -> 83.9 | 81.1 -> 83.2     83.2 -> 84.6 | 85.2 -> 84.8 | 81.1 -> 84.8
+// all_gather, uint8, outputs 128 MiB k + 32 MiB apart, blocks of 1 / 4 / 16 / 64 MiB:
+//   9 ranks     76.8 -> 76.8 / 82.5 -> 82.4 / 84.1 -> 84.2 / 84.6 -> 84.6      (allocated one by one, 16 / 64 MiB: 80.6 -> 83.4 / 80.9 -> 84.6)
+//   12 ranks    79.6 -> 81.6 / 78.0 -> 81.3 / 82.5 -> 84.4 / 81.9 -> 84.6      (allocated one by one: 77.4 -> 83.7 / 75.1 -> 80.2 / 80.6 -> 83.1 / 79.8 -> 84.5)
+//   16 ranks    79.6 -> 80.7 / 76.5 -> 81.8 / 78.0 -> 83.9 / 78.2 -> 82.9      (allocated one by one: 69.1 -> 81.5 / 75.0 -> 80.6 / 77.4 -> 84.5 / 76.2 -> 83.2)
+// So: twelve ranks and more from blocks of a MiB; six ranks and more from 768 MiB written in all; four and five ranks
+// from 2 GiB written; where the outputs lie does not enter.
+bool paced_gather(uint32_t nranks, uint64_t block_bytes) {
     if (pace_override() >= 0) return pace_override() == 1;
-    if (nranks < 8 || block_bytes * nranks * nranks < (uint64_t(1) << 30)) return false;
-    constexpr uintptr_t kUnit = uintptr_t(32) << 20;
-    bool placed = true;
-    uint64_t keys[2] = {0, 0};
-    for (uint32_t r = 0; r < nranks && placed; ++r) {
-        const uintptr_t a = reinterpret_cast<uintptr_t>(out[r]);
-        const uint32_t key = uint32_t((a / kUnit) % 128);
-        placed = (a % kUnit) == (reinterpret_cast<uintptr_t>(out[0]) % kUnit) && !(keys[key / 64] >> (key % 64) & 1u);
-        keys[key / 64] |= uint64_t(1) << (key % 64);
-    }
-    return !placed;
+    constexpr uint64_t kMiB = uint64_t(1) << 20;
+    const uint64_t written = block_bytes * nranks * nranks;
+    if (nranks >= 12) return block_bytes >= kMiB;
+    if (nranks >= 6) return written >= 768 * kMiB;
+    return nranks >= 4 && written >= 2048 * kMiB;
+}
+
+// The same for a broadcast (one load, N stores per wavefront, to the same offset of every output).  fp32, blocks of
+// 32 / 128 / 512 MiB, outputs an odd multiple of 128 MiB apart | allocated one by one:
+//   4 ranks   81.8 -> 77.2 | 81.6 -> 77.0     84.9 -> 82.4 | 84.4 -> 82.3     82.6 -> 84.5 | 80.2 -> 84.3
+//   5 ranks   83.8 -> 78.5 | 83.3 -> 78.5     85.0 -> 83.3 | 78.1 -> 82.8     79.9 -> 85.0 | 79.3 -> 85.0
+//   6 ranks   84.5 -> 80.0 | 84.6 -> 79.8     84.3 -> 82.1 | 77.5 -> 82.2     80.3 -> 82.9 | 83.1 -> 85.3
+//   7 ranks   84.8 -> 80.6 | 84.7 -> 80.3     80.5 -> 82.9 | 79.4 -> 82.8     81.6 -> 84.7 | 81.7 -> 84.4
+//   8 ranks   84.1 -> 81.5 | 83.9 -> 80.9     85.5 -> 84.5 | 84.7 -> 83.4     80.5 -> 84.8 | 79.6 -> 84.3
+// (blocks of 256 MiB, placed, 3 / 5 / 6 / 7 / 8 ranks: 86.3 -> 83.5 / 81.6 -> 84.2 / 79.2 -> 81.7 / 79.2 -> 83.7 / 82.6 -> 84.6);
+// uint8 blocks of 4 / 16 / 64 MiB, placed | allocated one by one:
+//   9 ranks     67.8 -> 67.8 | 67.8 -> 67.7     83.4 -> 85.3 | 82.7 -> 82.6     81.5 -> 81.9 | 78.4 -> 81.1
+//   12 ranks    68.6 -> 67.6 | 67.5 -> 70.2     81.5 -> 83.7 | 80.2 -> 82.5     79.3 -> 82.1 | 76.6 -> 81.6
+//   16 ranks    69.9 -> 72.1 | 71.0 -> 70.5     78.8 -> 82.2 | 78.7 -> 81.4     75.5 -> 81.2 | 74.0 -> 81.1
+// So: nine ranks and more from blocks of 16 MiB, five and more from 256 MiB, four from 512 MiB.
+bool paced_broadcast(uint32_t nranks, uint64_t block_bytes) {
+    if (pace_override() >= 0) return pace_override() == 1;
+    constexpr uint64_t kMiB = uint64_t(1) << 20;
+    if (nranks >= 9) return block_bytes >= 16 * kMiB;
+    if (nranks >= 5) return block_bytes >= 256 * kMiB;
+    return nranks == 4 && block_bytes >= 512 * kMiB;
 }
 
 uint32_t common_width(uint64_t block_bytes, const void* const* a, const void* const* b, uint32_t n) {
@@ -675,7 +708,8 @@ Status add_pack(Plan& plan, const void* const* in, void* const* out, uint32_t nr
     L.width = common_width(block_bytes, in, out_c, nranks);
     const uint64_t tiles = pack_tiles(block_bytes);
     L.waves = tiles >= kGroupMinTiles / 4 ? kGroupWaves : 1;  // long blocks take the group form
-    if (L.waves == kGroupWaves && mode == kPackAllGather) L.paced = paced_gather(out_c, nranks, block_bytes) ? 1 : 0;
+    if (L.waves == kGroupWaves && mode == kPackAllGather) L.paced = paced_gather(nranks, block_bytes) ? 1 : 0;
+    if (L.waves == kGroupWaves && mode == kPackBroadcast) L.paced = paced_broadcast(nranks, block_bytes) ? 1 : 0;
     // A grid holds 2^31 - 1 workgroups: blocks whose tiles, over all copies, outnumber that are cut into
     // slices of tiles, one launch each (the reference's per-peer copies have no such limit either).
     const uint64_t span = uint64_t(kGroupWaves) * kGroupStride;  // tiles a run of kGroupStride workgroups covers

@@ -225,7 +225,7 @@ struct PackLaunch {
     uint32_t width;   // what every block address and the block size are a multiple of: 16, 8, 4, 2 or 1
     uint32_t waves;   // wavefronts per workgroup: 1, or kGroupWaves (long blocks)
     uint32_t groups_per_copy;  // group form: workgroups per block copy
-    uint32_t paced;   // group form, all_gather: a wavefront issues its N stores one at a time (paced_gather in vrank_plan.cpp)
+    uint32_t paced;   // group form, all_gather and broadcast: a wavefront issues its N stores one at a time (paced_gather, paced_broadcast in vrank_plan.cpp)
     uint32_t reserved;
     uint64_t first_tile;  // the launch covers tiles [first_tile, first_tile + tiles_per_copy) of every copy (blocks
                           // too long for one grid are cut into several launches; a multiple of the group span)

@@ -439,15 +439,38 @@ def test_pack_collectives_group_form(dtype):
 
 @pytest.mark.parametrize("pace", ["always", "never"])
 def test_pack_collectives_group_form_with_paced_stores(pace, monkeypatch):
-    """An all_gather of eight ranks that writes a GiB and more into buffers the library did not place issues a
-    wavefront's stores one at a time; MEGRAY_VRANK_PACE forces that on (and off) here at a size the oracle handles.
-    Same permutations either way."""
+    """A long all_gather or broadcast in the group form issues a wavefront's stores one at a time (the planner decides
+    by rank count and size); MEGRAY_VRANK_PACE forces that on (and off) here at a size the oracle handles.  Same
+    permutations either way."""
     monkeypatch.setenv("MEGRAY_VRANK_PACE", pace)
     rng = np.random.default_rng(290)
     for dtype in (orc.UINT8, orc.FLOAT32):
         length = (1030 * 1024 + 48) // orc.dtype_size(dtype)
         for nranks in (3, 8):
             check_pack_collectives(dtype, nranks, length, 0, rng)
+
+
+def test_many_rank_gathers_and_broadcasts_pace_their_stores_by_themselves():
+    """From twelve ranks on an all_gather in the group form issues a wavefront's stores one at a time whatever the
+    buffers' addresses, and so does a broadcast of 16 MiB and more to nine ranks and more: the same permutations."""
+    rng = np.random.default_rng(291)
+    length = 1030 * 1024 + 48
+    for nranks in (12, 16):
+        runs, _, _ = mr.describe(mr.Collective.ALL_GATHER, [(1 << 40) + (r << 30) for r in range(nranks)],
+                                 [(2 << 40) + (r << 34) for r in range(nranks)], length, orc.UINT8)
+        assert runs and all(r["waves"] == 4 and r["paced"] == 1 for r in runs)
+        check_pack_collectives(orc.UINT8, nranks, length, 0, rng)
+    nranks, length, root = 9, (16 << 20) + 48, 4
+    runs, _, _ = mr.describe(mr.Collective.BROADCAST, [1 << 40] * nranks, [(2 << 40) + (r << 34) for r in range(nranks)],
+                             length, orc.UINT8, root=root)
+    assert runs and all(r["waves"] == 4 and r["paced"] == 1 for r in runs)
+    block = rand_array(orc.UINT8, length, rng)
+    d_root = to_device(block)
+    d_out = [empty_device(length) for _ in range(nranks)]
+    mr.broadcast(d_root, d_out, length, orc.UINT8, root)
+    torch.cuda.synchronize()
+    for r in range(nranks):
+        assert_same(to_host(d_out[r], block.dtype), block, f"paced broadcast rank={r}")
 
 
 def check_pack_collectives(dtype, nranks, length, misalign, rng):
