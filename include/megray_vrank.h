@@ -174,6 +174,9 @@ typedef struct mrv_plan_run {
                                workgroups are dealt to one XCD (one L2) each; pack decides this per copy on the device */
     uint32_t paced;         /* group form: 1 = the launch spaces its accesses out (a wavefront keeps two loads and two stores in
                                flight; a pack launch issues a wavefront's stores one at a time): long launches, see vrank_plan.cpp */
+    uint32_t keep;          /* 1 = the launch's stores leave their data in the last-level cache (collectives that write 128 MiB
+                               or less); 0 = they stream past the caches */
+    uint32_t reserved;
 } mrv_plan_run;
 
 /*

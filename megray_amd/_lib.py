@@ -19,6 +19,7 @@ class PlanRun(ctypes.Structure):
         ("tiles", ctypes.c_uint32), ("reads_recv", ctypes.c_uint32), ("waves", ctypes.c_uint32),
         ("in_begin", ctypes.c_uint64), ("out_begin", ctypes.c_uint64),
         ("count", ctypes.c_uint64), ("deal", ctypes.c_uint32), ("paced", ctypes.c_uint32),
+        ("keep", ctypes.c_uint32), ("reserved", ctypes.c_uint32),
     ]
 
 

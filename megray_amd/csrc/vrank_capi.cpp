@@ -339,6 +339,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.waves = L.waves;
                     run.deal = (L.waves == kGroupWaves && (sg.flags & kSegDeal)) ? 1 : 0;
                     run.paced = L.paced;
+                    run.keep = L.keep;
                     run.start = sg.start;
                     run.dir = sg.dir;
                     run.out_first = sg.out_first;
@@ -370,6 +371,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.waves = L.waves;
                     run.deal = (L.exchange & 2u) ? 1 : 0;
                     run.paced = (L.exchange & kFlatPaced) ? 1 : 0;
+                    run.keep = (L.exchange & kFlatKeep) ? 1 : 0;
                     run.start = start;
                     run.dir = L.tree ? 0 : int(int8_t((L.meta[s] >> 8) & 0xffu));
                     run.out_first = out_first;
@@ -392,6 +394,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                 run.nfold = L.nranks;
                 run.nout = 1;
                 run.waves = 1;
+                run.keep = L.keep;
                 run.start = L.root;
                 run.dir = 0;
                 run.out_first = L.root;
@@ -419,6 +422,7 @@ int mrv_describe(int collective, const void* const* sendbuffs, void* const* recv
                     run.vector = L.width;
                     run.waves = L.waves;
                     run.paced = L.paced;
+                    run.keep = L.keep;
                     run.dir = 1;
                     run.tiles = L.tiles_per_copy;
                     run.count = slice_bytes;

@@ -45,8 +45,9 @@ Schedule as_schedule(int schedule) {
 }
 }  // namespace
 
-Status plan_collective(Plan& plan, int kind, const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks,
-                       size_t count, DType dt, int order, int schedule, uint32_t root) {
+namespace {
+Status plan_steps(Plan& plan, int kind, const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks,
+                  size_t count, DType dt, int order, int schedule, uint32_t root) {
     switch (kind) {
         case kCollAllReduce:
             // a ring hop stores its partial result in the element type: FLOAT16 would round N-1 times
@@ -80,6 +81,14 @@ Status plan_collective(Plan& plan, int kind, const void* const* sendbuffs, void*
         default:
             MEGRAY_THROW("unknown collective");
     }
+}
+}  // namespace
+
+Status plan_collective(Plan& plan, int kind, const void* const* sendbuffs, void* const* recvbuffs, uint32_t nranks,
+                       size_t count, DType dt, int order, int schedule, uint32_t root) {
+    const Status st = plan_steps(plan, kind, sendbuffs, recvbuffs, nranks, count, dt, order, schedule, root);
+    if (st == MEGRAY_OK) set_store_policy(plan);
+    return st;
 }
 
 Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCall>& calls) {
@@ -173,11 +182,6 @@ uint64_t key_signature(const FlatKey& key) {
     return h ^ (h >> 32);
 }
 
-int pace_choice() {
-    const char* text = std::getenv("MEGRAY_VRANK_PACE");  // the planner reads it too: part of what a plan depends on
-    return !text ? -1 : std::strcmp(text, "always") == 0 ? 1 : std::strcmp(text, "never") == 0 ? 0 : -1;
-}
-
 }  // namespace
 
 Status run_collective(int kind, const void* const* send, void* const* recv, uint32_t nranks, size_t count, DType dtype,
@@ -191,7 +195,7 @@ Status run_collective(int kind, const void* const* send, void* const* recv, uint
     thread_local uint64_t clock = 0;
     FlatKey key;
     std::memset(&key, 0, sizeof(key));
-    key.kind = kind, key.order = order, key.sched = schedule, key.pace = pace_choice();
+    key.kind = kind, key.order = order, key.sched = schedule, key.pace = plan_overrides();  // the planner reads the environment: part of what a plan depends on
     key.nranks = nranks, key.root = root, key.count = count, key.dtype = dtype, key.op = is_reduction(kind) ? op : MEGRAY_SUM;
     if (hipGetDevice(&key.device) != hipSuccess) {
         (void)hipGetLastError();

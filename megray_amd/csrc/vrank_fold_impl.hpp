@@ -91,10 +91,13 @@ __device__ __forceinline__ void store_vec(char* p, u32x4 x) {
 
 // One tile (1 KiB) of a buffer through buffer instructions with explicit cache policies: measured
 // against plain non-temporal global accesses on MI355X (8 in + 8 out, fp32), non-temporal buffer
-// loads plus "sc1 nt" buffer stores sustain about 5 % more HBM bandwidth.
+// loads plus "sc1 nt" buffer stores sustain about 5 % more HBM bandwidth.  Launches that write little
+// (kKeepMaxBytes in vrank_types.h) store "sc1" without "nt", which leaves the data in the last-level cache;
+// `keep` is uniform over the launch, so the choice is a scalar branch.
 typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
-constexpr int kLoadPolicy = 2;    // nt
-constexpr int kStorePolicy = 18;  // sc1 | nt
+constexpr int kLoadPolicy = 2;        // nt
+constexpr int kStorePolicy = 18;      // sc1 | nt
+constexpr int kStoreKeepPolicy = 16;  // sc1
 constexpr int kRsrcFlags = 0x00020000;  // raw 32-bit data format, no swizzle
 
 __device__ __forceinline__ u32x4 load_tile_vec(const void* tile_base, uint32_t lane) {
@@ -102,10 +105,13 @@ __device__ __forceinline__ u32x4 load_tile_vec(const void* tile_base, uint32_t l
             const_cast<void*>(tile_base), 0, int(kThreads * kVecBytes), kRsrcFlags);
     return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, int(lane * kVecBytes), 0, kLoadPolicy));
 }
-__device__ __forceinline__ void store_tile_vec(void* tile_base, uint32_t lane, u32x4 x) {
+__device__ __forceinline__ void store_tile_vec(void* tile_base, uint32_t lane, u32x4 x, bool keep) {
     __amdgpu_buffer_rsrc_t rsrc =
             __builtin_amdgcn_make_buffer_rsrc(tile_base, 0, int(kThreads * kVecBytes), kRsrcFlags);
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, x), rsrc, int(lane * kVecBytes), 0, kStorePolicy);
+    if (keep)
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, x), rsrc, int(lane * kVecBytes), 0, kStoreKeepPolicy);
+    else
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, x), rsrc, int(lane * kVecBytes), 0, kStorePolicy);
 }
 
 // The same for tiles that may start at any byte address (segments of 1- and 2-byte elements whose inputs are
@@ -115,8 +121,8 @@ __device__ __forceinline__ u32x4 load_tile_any(const char* tile_base, uint32_t l
     if ((reinterpret_cast<uintptr_t>(tile_base) & 3u) == 0) return load_tile_vec(tile_base, lane);
     return load_vec(tile_base + lane * kVecBytes);
 }
-__device__ __forceinline__ void store_tile_any(char* tile_base, uint32_t lane, u32x4 x) {
-    if ((reinterpret_cast<uintptr_t>(tile_base) & 3u) == 0) store_tile_vec(tile_base, lane, x);
+__device__ __forceinline__ void store_tile_any(char* tile_base, uint32_t lane, u32x4 x, bool keep) {
+    if ((reinterpret_cast<uintptr_t>(tile_base) & 3u) == 0) store_tile_vec(tile_base, lane, x, keep);
     else store_vec(tile_base + lane * kVecBytes, x);
 }
 
@@ -477,7 +483,7 @@ __device__ __forceinline__ void fold_tile(const FoldLaunch& L) {
             }
             const u32x4 res = acc.finish();
             for (uint32_t m = 0; m < nout; ++m)
-                store_tile_any(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, nr)]) + out_off, tid, res);
+                store_tile_any(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, nr)]) + out_off, tid, res, L.keep != 0);
         }
     } else {
         fold_element_tile<T, OP>(L, sv, nfold, local_tile, tid);
@@ -597,7 +603,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
 
     if (nout == 1) {
         if (have && live)
-            store_tile_any(static_cast<char*>(L.out[sv.out_first]) + out_base + mine * kGroupBytes, tid, acc.finish());
+            store_tile_any(static_cast<char*>(L.out[sv.out_first]) + out_base + mine * kGroupBytes, tid, acc.finish(), L.keep != 0);
         return;
     }
     if (have) result[wave][tid] = acc.finish();
@@ -608,7 +614,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
         if (folded[k] && live)
             store_tile_any(static_cast<char*>(L.out[rotate_rank(sv.out_first, 1, m, nr)]) + out_base +
                                    (first + uint64_t(k) * kGroupStride) * kGroupBytes,
-                           tid, result[k][tid]);
+                           tid, result[k][tid], L.keep != 0);
         if (L.paced && (m + 1) % kGroupStoresInFlight == 0 && m + 1 < nout) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
 }
@@ -724,7 +730,7 @@ __device__ __forceinline__ void tree_tile(const TreeLaunch& L) {
     if ((uint64_t(blockIdx.x) + 1) * kThreads <= nvec) {
         // a whole tile: buffer instructions with the streaming cache policies
         const u32x4 r = tree_node<T, OP, kMaxRanks, true>(L, tile_off, 0, threadIdx.x).finish();
-        store_tile_any(static_cast<char*>(L.out) + tile_off, threadIdx.x, r);
+        store_tile_any(static_cast<char*>(L.out) + tile_off, threadIdx.x, r, L.keep != 0);
     } else if (lane < nvec) {
         store_vec(static_cast<char*>(L.out) + lane * kVecBytes, tree_vector<T, OP>(L, lane * kVecBytes));
     }
@@ -895,7 +901,7 @@ __device__ __forceinline__ void flat_tile_across_runs(const FlatLaunch& L, uint3
             // all_reduce: every rank's copy of the tile, at the inputs' offset, with the stores of the main path
             const uint64_t tile_off = e_lo * sizeof(T);
 #pragma unroll
-            for (int m = 0; m < K; ++m) store_tile_vec(static_cast<char*>(L.out[m]) + tile_off, tid, res);
+            for (int m = 0; m < K; ++m) store_tile_vec(static_cast<char*>(L.out[m]) + tile_off, tid, res, (L.exchange & kFlatKeep) != 0);
         } else {
 #pragma unroll 1
             for (uint32_t m = 0; m < nout; ++m)
@@ -978,10 +984,10 @@ __device__ __forceinline__ void flat_tile(const FlatLaunch& L, uint32_t tile, ui
         }
         if (nout == uint32_t(K)) {
 #pragma unroll
-            for (int m = 0; m < K; ++m) store_tile_vec(static_cast<char*>(L.out[m]) + out_off, tid, res);
+            for (int m = 0; m < K; ++m) store_tile_vec(static_cast<char*>(L.out[m]) + out_off, tid, res, (L.exchange & kFlatKeep) != 0);
         } else {
             for (uint32_t m = 0; m < nout; ++m)
-                store_tile_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, K)]) + out_off, tid, res);
+                store_tile_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, K)]) + out_off, tid, res, (L.exchange & kFlatKeep) != 0);
         }
         return;
     }
@@ -1101,7 +1107,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
         } else if (live) {
             const uint64_t out_off = uint64_t(mine) * (kThreads * kVecBytes) - out_shift * sizeof(T);
             for (uint32_t m = 0; m < L.nout; ++m)
-                store_tile_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, K)]) + out_off, tid, res);
+                store_tile_vec(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, K)]) + out_off, tid, res, (L.exchange & kFlatKeep) != 0);
         }
     } else if (!live) {
         // nothing is stored
@@ -1121,7 +1127,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
             const uint32_t k = (wave + m) % W;
             if (folded[k] && live) {
                 const uint64_t tile = uint64_t(first) + k * kGroupStride;
-                store_tile_vec(static_cast<char*>(L.out[m]) + tile * (kThreads * kVecBytes), tid, result[k][tid]);
+                store_tile_vec(static_cast<char*>(L.out[m]) + tile * (kThreads * kVecBytes), tid, result[k][tid], (L.exchange & kFlatKeep) != 0);
             }
             // ... and kGroupStoresInFlight stores in flight
             if (paced && (m + 1) % int(kGroupStoresInFlight) == 0 && m + 1 < K) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

@@ -104,7 +104,7 @@ __device__ __forceinline__ void pack_vector_tile(const PackLaunch& L, const Pack
         const uint64_t off = pv.head + (t0 - pv.pad) * kVecBytes;
         const u32x4 x = load_tile_any(src + off, tid);
         for (uint32_t m = 0; m < e.ndst; ++m)
-            store_tile_any(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + off, tid, x);
+            store_tile_any(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + off, tid, x, L.keep != 0);
     } else if (t0 + tid >= pv.pad && t0 + tid - pv.pad < pv.nvec) {
         const uint64_t off = pv.head + (t0 + tid - pv.pad) * kVecBytes;
         const u32x4 x = load_vec(src + off);
@@ -173,7 +173,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
     else if (live)
         pack_vector_tile(L, e, pv, src, dst_off, mine, tid);  // a partial tile at either end: copied to every destination here
     if (e.ndst == 1) {
-        if (whole && live) store_tile_any(static_cast<char*>(L.out[e.dst_rank]) + dst_off + tile_off(mine), tid, x);
+        if (whole && live) store_tile_any(static_cast<char*>(L.out[e.dst_rank]) + dst_off + tile_off(mine), tid, x, L.keep != 0);
         return;
     }
     stage[wave][tid] = x;
@@ -183,7 +183,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) pack_group_kernel(cons
         const uint32_t k = (wave + m) % W;
         if (staged[k] && live)
             store_tile_any(static_cast<char*>(L.out[e.dst_rank + m]) + dst_off + tile_off(first + uint64_t(k) * kGroupStride),
-                            tid, stage[k][tid]);
+                            tid, stage[k][tid], L.keep != 0);
         if (L.paced) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // one store in flight per wavefront
     }
 }

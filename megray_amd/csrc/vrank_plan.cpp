@@ -33,6 +33,14 @@ int pace_override() {
     return -1;
 }
 
+// MEGRAY_VRANK_KEEP in the environment overrides set_store_policy(): "always", "never".
+int keep_override() {
+    const char* text = std::getenv("MEGRAY_VRANK_KEEP");  // read at every planning: tests switch it
+    if (text && std::strcmp(text, "always") == 0) return 1;
+    if (text && std::strcmp(text, "never") == 0) return 0;
+    return -1;
+}
+
 // Should a flat group launch over these buffers (`bytes` each) keep two loads and two stores per wavefront in flight
 // instead of all of them?  Pacing costs a short launch latency and gains a long one bandwidth, the more the worse
 // the buffers lie relative to each other.  Measured on MI355X, fp32 SUM all_reduce, % of the HBM peak, all at once ->
@@ -730,6 +738,20 @@ Status add_pack(Plan& plan, const void* const* in, void* const* out, uint32_t nr
 }
 
 }  // namespace
+
+void set_store_policy(Plan& plan) {
+    const bool keep = keep_override() >= 0 ? keep_override() == 1 : plan.bytes_written <= kKeepMaxBytes;
+    for (Step& step : plan.steps) {
+        switch (step.kind) {
+            case Step::kFold: step.fold.keep = keep ? 1 : 0; break;
+            case Step::kFlat: step.flat.exchange = keep ? step.flat.exchange | kFlatKeep : step.flat.exchange & ~kFlatKeep; break;
+            case Step::kTree: step.tree.keep = keep ? 1 : 0; break;
+            case Step::kPack: step.pack.keep = keep ? 1 : 0; break;
+        }
+    }
+}
+
+int plan_overrides() { return (pace_override() + 1) + 4 * (keep_override() + 1); }
 
 Status plan_all_to_all(Plan& plan, const void* const* send, void* const* recv, uint32_t nranks,
                        uint64_t len, uint32_t elem_size) {

@@ -88,6 +88,13 @@ Status plan_reduce(Plan& plan, const void* const* send, void* recv_root, uint32_
 // o = reduce(i0, i1) with the tie convention of src/ucx/kernel.cu:24-38 (equal / unordered -> i1)
 Status plan_reduce2(Plan& plan, const void* i0, const void* i1, void* o, uint64_t len, uint32_t elem_size);
 
+// Chooses the store policy of a finished plan (kKeepMaxBytes in vrank_types.h): a collective that writes little leaves
+// its results in the last-level cache.  MEGRAY_VRANK_KEEP=always|never in the environment overrides the choice.
+void set_store_policy(Plan& plan);
+// What the environment says about the planner's choices (pacing, store policy), as one number: part of what a cached
+// plan depends on.
+int plan_overrides();
+
 const char* plan_error();  // text for the last MEGRAY_INVALID_ARGUMENT of this thread
 void set_plan_error(const char* text);  // lets a thread pass the text on to the threads it planned for
 

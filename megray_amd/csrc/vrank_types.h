@@ -69,7 +69,7 @@ struct FoldLaunch {
     uint32_t elem_size;
     uint32_t waves;          // wavefronts per workgroup: 1, or 4 for the group form (long vector bodies)
     uint32_t paced;          // group form: a wavefront keeps two loads and two stores in flight (as kFlatPaced)
-    uint32_t reserved;
+    uint32_t keep;           // 1: the stores leave their data in the last-level cache (as kFlatKeep)
     EdgeHooks hooks;         // one wavefront per workgroup only
     uint64_t hook_target;
     uint64_t hook_ticket;
@@ -77,6 +77,17 @@ struct FoldLaunch {
 
 constexpr uint32_t kFlatGuarded = 4;  // FlatLaunch::exchange
 constexpr uint32_t kFlatPaced = 8;    // FlatLaunch::exchange, group form: a wavefront keeps two loads and two stores in flight
+constexpr uint32_t kFlatKeep = 16;    // FlatLaunch::exchange: the stores leave their data in the last-level cache
+
+// Store policy.  Results normally stream past the caches ("sc1 nt" stores: written through, not kept), which sustains the
+// most HBM bandwidth on long launches.  A collective that writes no more than kKeepMaxBytes in all leaves its results in
+// the last-level cache instead ("sc1" stores: written through, kept; 256 MiB on MI355X, shared with what the launch reads): whoever
+// reads them next finds them there.  Measured on MI355X, all_reduce fp32 over 8 ranks inside a chain "elementwise kernel
+// over every rank's result -> all_reduce", time per link, streamed -> kept, per-rank buffers of 4 / 8 / 16 / 32 / 64 / 128 MiB:
+// 40.0 -> 38.4 / 55.2 -> 53.4 / 91.8 -> 80.7 / 178 -> 184 / 343 -> 351 / 664 -> 681 us (the all_reduce alone, back to back, % of
+// the HBM peak: 96 -> 101 / 80 -> 83 / 77 -> 83 / 81 -> 87 / 83 -> 82.5 / 84.5 -> 83.8).  So: up to 128 MiB written.
+// (Loads stay "nt": keeping what a collective reads once gains the chain 4 % up to 8 MiB and costs it 5 % from 32 MiB.)
+constexpr uint64_t kKeepMaxBytes = uint64_t(128) << 20;
 
 constexpr uint32_t kMaxFlatRuns = 48;  // 2N chunks cut again at N-1 rank borders
 
@@ -115,6 +126,7 @@ struct FlatLaunch {
     uint32_t exchange;  // group form: bit 0 = every rank is an output at the inputs' offsets, results are exchanged too;
                         // bit 1 = tiles share cache lines with their neighbours, deal runs of workgroups to XCDs;
                         // bit 3 (kFlatPaced) = a wavefront keeps kGroupLoadsInFlight loads / stores in flight instead of all;
+                        // either form: bit 4 (kFlatKeep) = the stores leave their data in the last-level cache;
                         // either form: bit 2 (kFlatGuarded) = the launch belongs to a communicator group, hooks.words
                         // is set and the group's poison is tested before anything is stored (the flag sits here, in
                         // the line of scalars every wavefront reads anyway; `hooks` lies several cache lines further)
@@ -198,6 +210,8 @@ struct TreeLaunch {
     uint32_t total_tiles;  // kThreads lanes per tile
     uint32_t vector;       // 1: a lane takes a 16-byte vector (the last workgroup also the odd elements at the end);
                            // 0: a lane takes one element
+    uint32_t keep;         // 1: the stores leave their data in the last-level cache
+    uint32_t reserved;
     EdgeHooks hooks;
     uint64_t hook_target;
     uint64_t hook_ticket;
@@ -226,7 +240,7 @@ struct PackLaunch {
     uint32_t waves;   // wavefronts per workgroup: 1, or kGroupWaves (long blocks)
     uint32_t groups_per_copy;  // group form: workgroups per block copy
     uint32_t paced;   // group form, all_gather and broadcast: a wavefront issues its N stores one at a time (paced_gather, paced_broadcast in vrank_plan.cpp)
-    uint32_t reserved;
+    uint32_t keep;    // 1: the stores leave their data in the last-level cache
     uint64_t first_tile;  // the launch covers tiles [first_tile, first_tile + tiles_per_copy) of every copy (blocks
                           // too long for one grid are cut into several launches; a multiple of the group span)
     EdgeHooks hooks;      // one wavefront per workgroup only

@@ -145,6 +145,36 @@ def test_all_reduce_group_form_with_paced_accesses(dtype, monkeypatch):
         assert_same(got[r], want[r], f"unpaced group form dtype={dtype} rank={r}")
 
 
+@pytest.mark.parametrize("keep", ["never", "always"])
+def test_either_store_policy_gives_the_same_results(keep, monkeypatch):
+    """A collective that writes 128 MiB or less leaves its results in the last-level cache, longer ones stream past it:
+    two store instructions, chosen per launch.  Every test at a size the oracle handles runs the first; here
+    MEGRAY_VRANK_KEEP forces the streaming stores (and, for completeness, the keeping ones) through every kernel form:
+    flat (one wavefront per tile, and the group form), general (one wavefront, group form), tree, pack (both forms)."""
+    monkeypatch.setenv("MEGRAY_VRANK_KEEP", keep)
+    rng = np.random.default_rng(4100)
+    for dtype in (orc.FLOAT32, orc.UINT8, orc.FLOAT16):
+        size = orc.dtype_size(dtype)
+        for nranks, length, offsets in ((8, 40000 // size, None), (8, 5051 * 1024 // size + 5, None), (5, 9000 // size + 3, None),
+                                        (5, 4300 * 1024 // size + 7, None), (3, 4300 * 1024 // size + 7, [max(size, 4)] * 3)):
+            ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+            want = orc.fold_all_reduce(ins, dtype, orc.SUM, orc.ORDER_UCX)
+            got = run_all_reduce(ins, dtype, orc.SUM, orc.ORDER_UCX, mr.Schedule.FUSED, offsets=offsets)
+            for r in range(nranks):
+                assert_same(got[r], want[r], f"keep={keep} all_reduce dtype={dtype} N={nranks} len={length} rank={r}")
+        for length in (3000 // size, 4300 * 1024 // size + 7) if dtype != orc.FLOAT16 else ():   # the binomial tree towards a root
+            nranks, root = 5, 3
+            ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+            want = orc.ucx_reduce(ins, dtype, orc.MAX, root)[root]
+            d_in = [to_device(x) for x in ins]
+            d_out = empty_device(length * size)
+            mr.reduce_to_root(d_in, d_out, length, dtype, orc.MAX, root)
+            torch.cuda.synchronize()
+            assert_same(to_host(d_out, ins[0].dtype), want, f"keep={keep} tree reduce dtype={dtype} len={length}")
+    for length in (1000, 1030 * 1024 + 48):
+        check_pack_collectives(orc.UINT8, 8, length, 0, rng)
+
+
 @pytest.mark.parametrize("dtype", REDUCE_TYPES)
 def test_segment_group_form(dtype):
     """The general fold kernel with long vector bodies (512 groups of 64 vectors and more) runs in its

@@ -118,3 +118,36 @@ def test_the_other_pack_collectives_never_pace():
     assert not is_paced(mr.Collective.ALL_TO_ALL, ins, outs, block, mr.DType.UINT8)
     assert not is_paced(mr.Collective.SCATTER, [ins[0]] + [0] * (n - 1), outs, block, mr.DType.UINT8, root=0, nranks=n)
     assert not is_paced(mr.Collective.GATHER, ins, [outs[0]] + [0] * (n - 1), block, mr.DType.UINT8, root=0, nranks=n)
+
+
+def keeps(coll, send, recv, count, dtype=mr.DType.FLOAT32, **kw):
+    runs, _, written = mr.describe(coll, send, recv, count, dtype, **kw)
+    flags = {r["keep"] for r in runs}
+    assert len(flags) == 1, "one store policy per plan"
+    return flags.pop() == 1, written
+
+
+def test_results_of_128_mib_and_less_stay_in_the_last_level_cache(monkeypatch):
+    """The stores of a collective that writes up to 128 MiB in all leave their data in the cache; longer ones stream."""
+    monkeypatch.delenv("MEGRAY_VRANK_KEEP", raising=False)
+    for elems, want in ((1 << 10, True), (1 << 22, True), ((1 << 22) + 256, False), (1 << 28, False)):   # 8 x 16 MiB is the border
+        bufs = placed(16, 4 * elems)
+        got, written = keeps(mr.Collective.ALL_REDUCE, bufs[:8], bufs[8:], elems)
+        assert got == want and written == 8 * 4 * elems
+    # every launch of a multi-launch plan follows the plan's total
+    bufs = placed(16, 1 << 26)
+    for sched in (mr.Schedule.TWO_PHASE, mr.Schedule.RING):
+        assert keeps(mr.Collective.ALL_REDUCE, bufs[:8], bufs[8:], 1 << 20, schedule=sched)[0]
+        assert not keeps(mr.Collective.ALL_REDUCE, bufs[:8], bufs[8:], 1 << 24, schedule=sched)[0]
+    # a reduce_scatter writes one block per rank, an all_gather N blocks per rank
+    assert keeps(mr.Collective.REDUCE_SCATTER, bufs[:8], bufs[8:], 1 << 21)[0]          # 8 x 8 MiB written of 8 x 64 MiB read
+    ins, outs = placed(8, 16 * MIB), placed(8, 128 * MIB, BASE + (1 << 40))
+    assert keeps(mr.Collective.ALL_GATHER, ins, outs, 2 * MIB, mr.DType.UINT8)[0]        # 128 MiB written
+    assert not keeps(mr.Collective.ALL_GATHER, ins, outs, 2 * MIB + 16, mr.DType.UINT8)[0]
+    assert keeps(mr.Collective.BROADCAST, [BASE] + [0] * 7, outs, 16 * MIB, mr.DType.UINT8, root=0, nranks=8)[0]
+    assert not keeps(mr.Collective.BROADCAST, [BASE] + [0] * 7, outs, 17 * MIB, mr.DType.UINT8, root=0, nranks=8)[0]
+    assert keeps(mr.Collective.REDUCE, bufs[:5], [0, 0, bufs[8], 0, 0], 1 << 24, root=2, nranks=5)[0]   # the tree kernel: 64 MiB
+    monkeypatch.setenv("MEGRAY_VRANK_KEEP", "never")
+    assert not keeps(mr.Collective.ALL_REDUCE, bufs[:8], bufs[8:], 1 << 10)[0]
+    monkeypatch.setenv("MEGRAY_VRANK_KEEP", "always")
+    assert keeps(mr.Collective.ALL_REDUCE, bufs[:8], bufs[8:], 1 << 24)[0]
