@@ -51,7 +51,7 @@ int keep_override() {
 //   4 ranks, placed                                        81.4 -> 81.2 / 83.5 -> 83.0 / 84.1 -> 84.0 / 84.1 -> 84.0 / 84.0 -> 83.1
 //   3 ranks, separate allocations                          79.7 -> 80.4 / 83.4 -> 83.3 / 84.0 -> 83.7 / 82.1 -> 83.5 / 81.8 -> 84.2
 // So: buffers that do not lie the way vrank_placement.h lays them out pace from 3 GiB over all of them; buffers
-// that do, only eight-rank launches of 12 GiB and more (where it is worth a few tenths).
+// that do, never (8 ranks x 1 GiB placed, interleaved in one process on three boxes: 84.2 -> 84.0, 83.7 -> 83.2, 83.4 -> 82.6).
 // The general group kernel (other rank counts, buffers off the 16-byte grid) behaves alike on separate allocations
 // (5 / 7 / 12 / 16 ranks x 512 MiB: 79.4 -> 82.9 / 79.2 -> 81.3 / 76.4 -> 79.3 / 74.8 -> 78.3; x 256 MiB + 1 throughout;
 // x 64 MiB - 1) and loses half a point to a point on placed buffers, where it is left alone (`flat` false) - unless
@@ -88,7 +88,7 @@ bool paced_launch(const void* const* in, const void* const* out, uint32_t nranks
     const uint64_t total = uint64_t(n) * bytes;
     constexpr uint64_t kGiB = uint64_t(1) << 30;
     if (!flat && nout == 1 && total >= kGiB) return true;
-    return placed ? (flat && nranks >= 8 && total >= 12 * kGiB) : total >= 3 * kGiB;
+    return !placed && total >= 3 * kGiB;
 }
 
 bool overlaps(const void* a, uint64_t a_bytes, const void* b, uint64_t b_bytes) {

@@ -49,10 +49,11 @@ def test_all_reduce_on_buffers_the_library_did_not_place_paces_from_three_gib():
     assert not all_reduce_paced(2, 1 << 20, separate)
 
 
-def test_all_reduce_on_placed_buffers_paces_from_twelve_gib_on_eight_ranks():
-    assert all_reduce_paced(8, 1 << 28, placed)         # the headline: 16 GiB
-    assert not all_reduce_paced(8, 1 << 27, placed)     # 8 GiB
-    assert not all_reduce_paced(4, 1 << 29, placed)     # 16 GiB, but four ranks
+def test_all_reduce_on_placed_buffers_never_paces():
+    assert not all_reduce_paced(8, 1 << 28, placed)     # the headline: 16 GiB
+    assert not all_reduce_paced(8, 1 << 27, placed)
+    assert not all_reduce_paced(4, 1 << 29, placed)
+    assert not all_reduce_paced(5, 1 << 28, placed)     # the general kernel, every rank an output
 
 
 def test_the_environment_overrides_the_rule(monkeypatch):
