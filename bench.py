@@ -265,6 +265,18 @@ def comm_api_large():
     return out
 
 
+def side_leg(leg, *leg_args):
+    """Runs one of the legs that report beside the headline in child processes.  A leg that fails (a child that
+    exits with an error, or does not come back in time) is reported as {"error": ...} in its place and on stderr:
+    the headline measurement does not depend on it."""
+    try:
+        return leg(*leg_args)
+    except (SystemExit, subprocess.SubprocessError, OSError, ValueError, KeyError, IndexError) as failure:
+        text = " ".join(str(failure).split())[:600]
+        print(f"bench.py: {leg.__name__} failed: {text}", file=sys.stderr)
+        return {"error": text}
+
+
 def other_layout_fresh(args):
     """The headline launches on buffers laid out the OTHER way, in a process of its own (started before this one
     touches the GPU): what a caller gets who allocates its rank buffers first thing.  Where the driver puts
@@ -476,10 +488,10 @@ def main():
               "(use --gpus 1, rank count is --ranks)", file=sys.stderr)
         return 2
     headline = args.workload == "all_reduce"
-    # the thread-per-rank leg runs in a child process, before this process touches the GPU
-    comm_api = comm_api_sweep() if headline and not args.no_comm else None
-    comm_large = comm_api_large() if headline and not args.no_comm and args.log2n == 28 else None
-    other_fresh = other_layout_fresh(args) if headline and not args.no_others else None
+    # the thread-per-rank legs and the other layout's processes run as children, before this process touches the GPU
+    comm_api = side_leg(comm_api_sweep) if headline and not args.no_comm else None
+    comm_large = side_leg(comm_api_large) if headline and not args.no_comm and args.log2n == 28 else None
+    other_fresh = side_leg(other_layout_fresh, args) if headline and not args.no_others else None
 
     import numpy as np
     import torch
@@ -576,8 +588,12 @@ def main():
         same = {"ms_per_step": round(other_ms / args.steps, 4),
                 "pct_of_peak": round(100.0 * bmin / (other_ms / args.steps * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
                 "process": "this one, after the headline's buffers were allocated and freed"}
-        result["other_layout"] = dict(other_fresh, same_process=same) if other_fresh else dict(
-            same, layout=LAYOUT_TEXT[other], steps=args.steps, warmup=args.warmup)
+        if other_fresh and "error" not in other_fresh:
+            result["other_layout"] = dict(other_fresh, same_process=same)
+        else:  # no processes of their own (switched off, or they failed): this process's figure stands in
+            result["other_layout"] = dict(same, layout=LAYOUT_TEXT[other], steps=args.steps, warmup=args.warmup)
+            if other_fresh:
+                result["other_layout"]["processes_of_their_own"] = other_fresh
         del ins, outs
         torch.cuda.empty_cache()
     props = torch.cuda.get_device_properties(0)
