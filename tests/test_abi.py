@@ -145,3 +145,24 @@ def test_python_wrappers_reject_lists_of_different_lengths():
     runs, _, _ = mr.describe(mr.Collective.GATHER, [0x100000, 0x200000, 0x300000], [None, 0x900000], 16,
                              mr.DType.UINT8, root=1)
     assert len(runs) == 3 and all(r["out_first"] == 1 for r in runs)
+
+
+def test_the_header_is_plain_c_and_the_python_binding_lays_the_run_record_out_the_same_way(tmp_path):
+    """megray_vrank.h is what a foreign binding reads: it must compile as C99 on its own, and the ctypes mirror of
+    mrv_plan_run must agree with the compiler field by field."""
+    import subprocess
+
+    from megray_amd import _lib
+
+    fields = [name for name, _ in _lib.PlanRun._fields_]
+    prints = "\n".join(f'    printf("{f} %zu\\n", offsetof(mrv_plan_run, {f}));' for f in fields)
+    src = tmp_path / "layout.c"
+    src.write_text(f'#include <stddef.h>\n#include <stdio.h>\n#include "megray_vrank.h"\nint main(void) {{\n'
+                   f'    printf("sizeof %zu\\n", sizeof(mrv_plan_run));\n{prints}\n    return 0;\n}}\n')
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", f"-I{os.path.join(ROOT, 'include')}",
+                    str(src), "-o", str(exe)], check=True, capture_output=True, text=True)
+    lines = dict(line.split() for line in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines())
+    assert int(lines["sizeof"]) == ctypes.sizeof(_lib.PlanRun)
+    for f in fields:
+        assert int(lines[f]) == getattr(_lib.PlanRun, f).offset, f
