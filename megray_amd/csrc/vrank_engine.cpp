@@ -102,10 +102,15 @@ Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCal
                         &step.fold};
                 break;
             case Step::kFlat:
-                if (step.flat.waves == kGroupWaves)
+                if (step.flat.waves == kGroupWaves) {
                     call = {flat_kernel_for(step.flat, dtype, op), group_grid(step.flat.total_tiles),
                             kThreads * kGroupWaves, &step.flat};
-                else {
+                    // long all_reduce shapes that issue a wavefront's accesses at once run at fewer workgroups per CU
+                    const uint64_t bytes = step.flat.count * step.flat.elem_size;
+                    if ((step.flat.exchange & 1u) && !(step.flat.exchange & kFlatPaced) &&
+                        bytes >= (step.flat.nranks >= 8 ? kGroupCapMinBytes8 : kGroupCapMinBytes))
+                        call.lds = lds_for_waves_per_cu(call.kernel, group_cap_per_cu(step.flat.nranks));
+                } else {
                     call = {flat_kernel_for(step.flat, dtype, op), step.flat.total_tiles, kThreads, &step.flat};
                     // the planner leaves a launch this large at one wavefront per tile only to have it run at a
                     // reduced occupancy (flat_one_out)

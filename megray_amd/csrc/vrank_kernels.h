@@ -23,7 +23,8 @@ hipError_t enqueue(const void* kernel, uint32_t grid, uint32_t block, const void
                    uint32_t lds = 0);
 
 // LDS bytes to reserve per workgroup of `kernel`, on top of what it declares, so that at most `waves_per_cu`
-// of its one-wavefront workgroups share a CU (160 KiB of LDS each); 0 if the kernel's own LDS already sees to that.
+// of its workgroups share a CU (160 KiB of LDS each; for the one-wavefront kernels that is wavefronts per CU, for the
+// group forms workgroups of four); 0 if the kernel's own LDS already sees to that.
 uint32_t lds_for_waves_per_cu(const void* kernel, uint32_t waves_per_cu);
 
 }  // namespace vrank
