@@ -91,15 +91,42 @@ Status plan_collective(Plan& plan, int kind, const void* const* sendbuffs, void*
     return st;
 }
 
+namespace {
+// Workgroups per CU for the group form of the general fold kernel with a run-time fold width (5, 6, 7 and 9 - 32
+// inputs, staged through LDS four at a time; its LDS allows 7), 0 = as many as fit.  Measured on MI355X, fp32, placed
+// buffers, % of the HBM peak, interleaved in one process, as the LDS allows -> capped:
+//   all_reduce shapes (every rank an output), accesses at once, 256 MiB per rank -> 4 per CU:
+//     6 / 7 / 10 / 12 / 16 ranks 81.3 -> 82.3 / 81.5 -> 82.0 / 80.5 -> 82.5 / 80.3 -> 81.8 / 80.9 -> 81.6
+//     (3 per CU: 78 / 80 / 81.3 / 82.2 / 82.1; 5 per CU: 82.4 / 82.3 / 81.6 / 81.0 / 81.9); 64 MiB per rank, 6 / 7 / 12 ranks:
+//     78.9 -> 79.7 / 78.7 -> 80.8 / 78.6 -> 80.8; 5 ranks gain nothing at any occupancy
+//   folds into one output that pace their accesses (reduce_scatter from 1 GiB over all buffers) -> 6 per CU:
+//     6 / 7 / 10 / 12 / 16 ranks x 256 MiB 80.1 -> 84.0 / 80.9 -> 83.6 / 81.7 -> 83.7 / 82.0 -> 84.2 / 84.3 -> 85.4 (5 ranks 82.8 -> 82.3;
+//     at 7 per CU, reserved the same way, nothing changes; 5 per CU loses 1 - 7 points)
+uint32_t general_group_per_cu(const FoldLaunch& L) {
+    if (L.nfold < 6 || L.nfold == 8) return 0;  // 1, 2, 3, 4 and 8 inputs run kernels of their own
+    if (L.nout == 1) return L.paced ? 6u : 0u;
+    const bool long_launch = L.total_tiles >= 16384;  // 64 MiB per buffer: a workgroup takes 4 KiB of each
+    return L.nout == L.nranks && !L.paced && long_launch ? 4u : 0u;
+}
+}  // namespace
+
 Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCall>& calls) {
     calls.clear();
     calls.reserve(plan.steps.size());
+    // MEGRAY_VRANK_GROUP_PER_CU=n in the environment runs every group-form fold at n workgroups per CU instead of
+    // what the tables say (for measurements; 0 or unset: the tables)
+    const char* forced_text = std::getenv("MEGRAY_VRANK_GROUP_PER_CU");
+    const uint32_t forced = forced_text ? uint32_t(std::strtoul(forced_text, nullptr, 10)) : 0;
     for (const Step& step : plan.steps) {
         KernelCall call{nullptr, 0, kThreads, nullptr};
         switch (step.kind) {
             case Step::kFold:
                 call = {fold_kernel_for(step.fold, dtype, op), step.fold.total_tiles, kThreads * step.fold.waves,
                         &step.fold};
+                if (step.fold.waves == kGroupWaves) {
+                    const uint32_t per_cu = forced ? forced : general_group_per_cu(step.fold);
+                    if (per_cu) call.lds = lds_for_waves_per_cu(call.kernel, per_cu);
+                }
                 break;
             case Step::kFlat:
                 if (step.flat.waves == kGroupWaves) {
@@ -110,6 +137,7 @@ Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCal
                     if ((step.flat.exchange & 1u) && !(step.flat.exchange & kFlatPaced) &&
                         bytes >= (step.flat.nranks >= 8 ? kGroupCapMinBytes8 : kGroupCapMinBytes))
                         call.lds = lds_for_waves_per_cu(call.kernel, group_cap_per_cu(step.flat.nranks));
+                    if (forced) call.lds = lds_for_waves_per_cu(call.kernel, forced);
                 } else {
                     call = {flat_kernel_for(step.flat, dtype, op), step.flat.total_tiles, kThreads, &step.flat};
                     // the planner leaves a launch this large at one wavefront per tile only to have it run at a
