@@ -102,6 +102,19 @@ namespace {
 //   folds into one output that pace their accesses (reduce_scatter from 1 GiB over all buffers) -> 6 per CU:
 //     6 / 7 / 10 / 12 / 16 ranks x 256 MiB 80.1 -> 84.0 / 80.9 -> 83.6 / 81.7 -> 83.7 / 82.0 -> 84.2 / 84.3 -> 85.4 (5 ranks 82.8 -> 82.3;
 //     at 7 per CU, reserved the same way, nothing changes; 5 per CU loses 1 - 7 points)
+// The same for the group form of the flat fold: long launches that issue a wavefront's accesses at once run at fewer
+// workgroups per CU than their LDS allows - the all_reduce shapes (tables at group_cap_per_cu in vrank_types.h), and
+// the fold of two inputs into one output, which is the reference's own kernel shape (mrv_reduce) and the reduce_scatter
+// of two ranks: 1 GiB per buffer 86.3 -> 87.4 % of the HBM peak at 5 per CU (6: 86.8, 4: 83.4, 3: 71.2), reduce_scatter of
+// 2 x 512 MiB 84.8 -> 86.0; at 128 MiB per buffer the cap costs a point (87.9 -> 86.9) and is not applied.
+uint32_t flat_group_per_cu(const FlatLaunch& L) {
+    if (L.exchange & kFlatPaced) return 0;
+    const uint64_t bytes = L.count * L.elem_size;
+    if (L.exchange & 1u) return bytes >= (L.nranks >= 8 ? kGroupCapMinBytes8 : kGroupCapMinBytes) ? group_cap_per_cu(L.nranks) : 0;
+    if (L.nranks == 2 && L.nout == 1) return bytes >= (uint64_t(512) << 20) ? 5u : 0u;
+    return 0;
+}
+
 uint32_t general_group_per_cu(const FoldLaunch& L) {
     if (L.nfold < 6 || L.nfold == 8) return 0;  // 1, 2, 3, 4 and 8 inputs run kernels of their own
     if (L.nout == 1) return L.paced ? 6u : 0u;
@@ -132,12 +145,8 @@ Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCal
                 if (step.flat.waves == kGroupWaves) {
                     call = {flat_kernel_for(step.flat, dtype, op), group_grid(step.flat.total_tiles),
                             kThreads * kGroupWaves, &step.flat};
-                    // long all_reduce shapes that issue a wavefront's accesses at once run at fewer workgroups per CU
-                    const uint64_t bytes = step.flat.count * step.flat.elem_size;
-                    if ((step.flat.exchange & 1u) && !(step.flat.exchange & kFlatPaced) &&
-                        bytes >= (step.flat.nranks >= 8 ? kGroupCapMinBytes8 : kGroupCapMinBytes))
-                        call.lds = lds_for_waves_per_cu(call.kernel, group_cap_per_cu(step.flat.nranks));
-                    if (forced) call.lds = lds_for_waves_per_cu(call.kernel, forced);
+                    const uint32_t per_cu = forced ? forced : flat_group_per_cu(step.flat);
+                    if (per_cu) call.lds = lds_for_waves_per_cu(call.kernel, per_cu);
                 } else {
                     call = {flat_kernel_for(step.flat, dtype, op), step.flat.total_tiles, kThreads, &step.flat};
                     // the planner leaves a launch this large at one wavefront per tile only to have it run at a
