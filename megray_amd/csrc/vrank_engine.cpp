@@ -161,10 +161,11 @@ Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCal
                     call.lds = lds_for_waves_per_cu(call.kernel, kTreeCapWavesPerCu);
                 break;
             case Step::kPack:
-                if (step.pack.waves == kGroupWaves)
+                if (step.pack.waves == kGroupWaves) {
                     call = {pack_kernel_for(step.pack), step.pack.ncopies * step.pack.groups_per_copy,
                             kThreads * kGroupWaves, &step.pack};
-                else
+                    if (forced) call.lds = lds_for_waves_per_cu(call.kernel, forced);
+                } else
                     call = {pack_kernel_for(step.pack), step.pack.ncopies * step.pack.tiles_per_copy, kThreads,
                             &step.pack};
                 break;
