@@ -126,6 +126,36 @@ __device__ __forceinline__ void store_tile_any(char* tile_base, uint32_t lane, u
     else store_vec(tile_base + lane * kVecBytes, x);
 }
 
+// One element at byte `offset` (a multiple of the element size, below 1 KiB) of a tile, with the tile stores' cache
+// policy: written through, so that the kernel's end finds nothing to write back (a plain store leaves its line dirty
+// in the L2, and a short launch then waits for the write-back).
+template <typename T>
+__device__ __forceinline__ void store_tile_element(char* tile_base, uint32_t offset, T value, bool keep) {
+    if ((reinterpret_cast<uintptr_t>(tile_base) & 3u) != 0) {
+        *reinterpret_cast<T*>(tile_base + offset) = value;
+        return;
+    }
+    __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(tile_base, 0, int(kThreads * kVecBytes), kRsrcFlags);
+    if constexpr (sizeof(T) == 1) {
+        const auto bits = __builtin_bit_cast(uint8_t, value);
+        if (keep) __builtin_amdgcn_raw_buffer_store_b8(bits, rsrc, int(offset), 0, kStoreKeepPolicy);
+        else __builtin_amdgcn_raw_buffer_store_b8(bits, rsrc, int(offset), 0, kStorePolicy);
+    } else if constexpr (sizeof(T) == 2) {
+        const auto bits = __builtin_bit_cast(uint16_t, value);
+        if (keep) __builtin_amdgcn_raw_buffer_store_b16(bits, rsrc, int(offset), 0, kStoreKeepPolicy);
+        else __builtin_amdgcn_raw_buffer_store_b16(bits, rsrc, int(offset), 0, kStorePolicy);
+    } else if constexpr (sizeof(T) == 4) {
+        const auto bits = __builtin_bit_cast(uint32_t, value);
+        if (keep) __builtin_amdgcn_raw_buffer_store_b32(bits, rsrc, int(offset), 0, kStoreKeepPolicy);
+        else __builtin_amdgcn_raw_buffer_store_b32(bits, rsrc, int(offset), 0, kStorePolicy);
+    } else {
+        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+        const auto bits = __builtin_bit_cast(u32x2, value);
+        if (keep) __builtin_amdgcn_raw_buffer_store_b64(bits, rsrc, int(offset), 0, kStoreKeepPolicy);
+        else __builtin_amdgcn_raw_buffer_store_b64(bits, rsrc, int(offset), 0, kStorePolicy);
+    }
+}
+
 __device__ __forceinline__ uint32_t rotate_rank(uint32_t start, int dir, uint32_t j, uint32_t n) {
     // (start + dir*j) mod n for j < n, without a division
     if (dir > 0) {
@@ -793,46 +823,6 @@ __device__ __forceinline__ void uniform_scan(const RunBatch& b, uint64_t e_lo, u
     }
 }
 
-// One tile of a flat launch element by element: a tile that straddles a run border or the end of
-// the buffers.  One run at a time, so that ranks and destinations stay uniform.
-template <typename T, int OP, int K, bool TREE>
-__device__ __forceinline__ void flat_tile_by_element(const FlatLaunch& L, uint32_t tile, uint32_t tid) {
-    using A = typename Wide<T>::type;
-    constexpr uint32_t EPV = kVecBytes / sizeof(T);
-    constexpr uint32_t TILE = kThreads * EPV;
-    const bool new_wins = L.new_wins_ties != 0;
-    const uint32_t nout = L.nout;
-    const uint64_t e_lo = uint64_t(tile) * TILE;
-    const uint64_t e_hi = e_lo + TILE < L.count ? e_lo + TILE : L.count;
-    for (uint32_t i = 0; i < L.nruns; ++i) {
-        const uint64_t run_begin = i ? L.end[i - 1] : 0, run_end = L.end[i];
-        const uint64_t b = run_begin > e_lo ? run_begin : e_lo;
-        const uint64_t e = run_end < e_hi ? run_end : e_hi;
-        if (b >= e) continue;
-        const uint32_t start = meta_start(L.meta[i]);
-        const int dir = meta_dir(L.meta[i]);
-        const uint32_t out_first = meta_out_first(L.meta[i]);
-        const uint64_t shift = L.shift[i];
-        for (uint32_t k = 0; k < EPV; ++k) {
-            const uint64_t el = e_lo + uint64_t(tid) * EPV + k;
-            if (el < b || el >= e) continue;
-            T r;
-            if constexpr (TREE) {
-                r = tree_element<T, OP, K>(L, K, start, el);
-            } else {
-                A a = static_cast<A>(static_cast<const T*>(L.in[start])[el]);
-                for (uint32_t j = 1; j < uint32_t(K); ++j)
-                    a = combine<OP, A>(
-                            a, static_cast<A>(static_cast<const T*>(L.in[rotate_rank(start, dir, j, K)])[el]),
-                            new_wins);
-                r = static_cast<T>(a);
-            }
-            for (uint32_t m = 0; m < nout; ++m)
-                static_cast<T*>(L.out[rotate_rank(out_first, 1, m, K)])[el - shift] = r;
-        }
-    }
-}
-
 // What a lane knows about the run its own 16-byte vector lies in.
 struct LaneRun {
     bool inside = false;  // the vector lies wholly inside one run (whose order and destinations follow)
@@ -863,32 +853,125 @@ __device__ __forceinline__ void lane_scan(const RunBatch& w, uint32_t tile, uint
     }
 }
 
-// A tile that lies inside the buffers but straddles run borders, its K input vectors staged in LDS
-// as staged[r][lane].  Every lane has looked up the run its own vector lies in (LaneRun) and folds
-// its vector in that run's order, fetching the inputs from LDS by rank: one straight pass whatever
-// the number of runs in the tile, which is what the smallest messages consist of (8 ranks x 4 KiB:
-// every tile holds two chunks).  The few lanes whose vector is cut by a run border (chunk lengths
-// need not be multiples of a vector) then go element by element from global memory, run by run.
+// A tile that lies inside the buffers but straddles run borders, its K input vectors staged in LDS as
+// staged[r][lane].  Every lane has looked up the run its own vector lies in (LaneRun); the lanes whose vector lies
+// wholly inside one run fold it in that run's order, fetching the inputs from LDS by rank: one straight pass
+// whatever the number of runs in the tile, which is what the smallest messages consist of (8 ranks x 4 KiB: every
+// tile holds two chunks).  Returns the folded vector (of those lanes); `store`: also stores it to the run's outputs.
+// Lanes whose vector a run border cuts are left to flat_tile_ragged.
 template <typename T, int OP, int K, bool TREE>
-__device__ __forceinline__ void flat_tile_across_runs(const FlatLaunch& L, uint32_t tile, uint32_t tid,
-                                                      const u32x4 (*staged)[kThreads], const LaneRun& lr) {
-    using A = typename Wide<T>::type;
+__device__ __forceinline__ u32x4 flat_tile_whole_vectors(const FlatLaunch& L, uint32_t tile, uint32_t tid,
+                                                         const u32x4 (*staged)[kThreads], const LaneRun& lr, bool store) {
     constexpr uint32_t EPV = kVecBytes / sizeof(T);
     constexpr uint32_t TILE = kThreads * EPV;
-    const uint64_t e_lo = uint64_t(tile) * TILE, e_hi = e_lo + TILE;
-    const uint64_t lane_lo = e_lo + uint64_t(tid) * EPV;
+    u32x4 res = {0u, 0u, 0u, 0u};
+    if (!lr.inside) return res;
     const bool new_wins = L.new_wins_ties != 0;
-    const uint32_t nout = L.nout;
     const uint32_t start = meta_start(lr.meta), out_first = meta_out_first(lr.meta);
     const int dir = meta_dir(lr.meta);
-    const uint64_t shift = uint64_t(lr.shift_lo) | (uint64_t(lr.shift_hi) << 32);
-    if (lr.inside) {
+    if constexpr (TREE) {
+        u32x4 x[K];
+#pragma unroll
+        for (int r = 0; r < K; ++r) x[r] = staged[r][tid];
+        res = tree_from<T, OP, K>(x, start);
+    } else {
+        AccFor<T, OP> acc;
+        acc.seed(staged[start][tid]);
+#pragma unroll
+        for (uint32_t j = 1; j < uint32_t(K); ++j) acc.fold(staged[rotate_rank(start, dir, j, K)][tid], new_wins);
+        res = acc.finish();
+    }
+    if (store) {
+        const uint64_t shift = uint64_t(lr.shift_lo) | (uint64_t(lr.shift_hi) << 32);
+        const uint64_t out_el = uint64_t(tile) * TILE + uint64_t(tid) * EPV - shift;
+#pragma unroll 1
+        for (uint32_t m = 0; m < L.nout; ++m)
+            store_vec(reinterpret_cast<char*>(static_cast<T*>(L.out[rotate_rank(out_first, 1, m, K)]) + out_el), res);
+    }
+    return res;
+}
+
+// The buffers' last tile, which their end cuts: x[r] = this lane's vector of input r, lane by lane (nothing may be
+// read beyond the end), zero where the buffers have ended.  The vector that the end cuts is put together in LDS:
+// the elements that exist are loaded one per lane (all of them in flight together) and written where they belong in
+// a vector of zeros, which the lane that owns it then reads back.  `cut` is LDS of the workgroup that only the one
+// wavefront holding this tile touches (a wavefront's LDS instructions execute in order).
+template <typename T, int K>
+__device__ __forceinline__ void load_tile_at_the_end(const FlatLaunch& L, uint32_t tile, uint32_t tid, u32x4 (&x)[K],
+                                                     u32x4* cut) {
+    constexpr uint32_t EPV = kVecBytes / sizeof(T);
+    constexpr uint32_t TILE = kThreads * EPV;
+    const uint64_t e_lo = uint64_t(tile) * TILE;
+    const uint32_t nvalid = uint32_t(L.count - e_lo);  // below TILE
+    const uint32_t nfull = nvalid / EPV, ntail = nvalid % EPV;
+    T last[K];
+#pragma unroll
+    for (int r = 0; r < K; ++r) {
+        const T* p = static_cast<const T*>(L.in[r]) + e_lo;
+        x[r] = u32x4{0u, 0u, 0u, 0u};
+        if (tid < nfull) x[r] = load_vec(reinterpret_cast<const char*>(p + tid * EPV));
+        last[r] = T(0);
+        if (tid < ntail) last[r] = __builtin_nontemporal_load(p + nfull * EPV + tid);
+    }
+    if (!ntail) return;
+    if (tid < uint32_t(K)) cut[tid] = u32x4{0u, 0u, 0u, 0u};
+    __builtin_amdgcn_wave_barrier();
+    if (tid < ntail) {
+#pragma unroll
+        for (int r = 0; r < K; ++r) reinterpret_cast<T*>(&cut[r])[tid] = last[r];
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (tid == nfull) {
+#pragma unroll
+        for (int r = 0; r < K; ++r) x[r] = cut[r];
+    }
+}
+
+// One tile of a flat launch that no single run covers, or that the buffers' end cuts.  staged[r][lane] (LDS) is the lane's
+// vector of input r (zero where the buffers have ended); `pending` lanes have not stored their vector yet.  Run by run (uniform;
+// the runs that reach into the tile are found with eight runs per round of scalar loads, they are in order and none
+// is empty): the whole wavefront folds its vectors in that run's order, and every pending lane stores what of its
+// vector lies in the run - the whole vector if all of it does, else element by element (chunk lengths need not be
+// multiples of a vector, so a border may cut one, and so may the buffers' end).  No second pass over memory.
+template <typename T, int OP, int K, bool TREE, bool MERGE>
+__device__ __forceinline__ void flat_tile_ragged(const FlatLaunch& L, uint32_t tile, uint32_t tid,
+                                                 const u32x4 (*staged)[kThreads], bool pending, u32x4& merged) {
+    constexpr uint32_t EPV = kVecBytes / sizeof(T);
+    constexpr uint32_t TILE = kThreads * EPV;
+    const uint64_t e_lo = uint64_t(tile) * TILE;
+    const uint64_t e_hi = e_lo + TILE < L.count ? e_lo + TILE : L.count;
+    const uint32_t lane_off = tid * EPV;  // the lane's vector, in elements from the tile's start
+    const bool new_wins = L.new_wins_ties != 0;
+    const bool keep = (L.exchange & kFlatKeep) != 0;
+    const uint32_t nout = L.nout;
+    uint32_t first_run = L.nruns, last_run = 0;
+    for (uint32_t base = 0; base < L.nruns; base += 8) {
+        const RunBatch w = load_batch(L, base);
+        if (w.begin0 >= e_hi) break;
+#pragma unroll
+        for (uint32_t i = 0; i < 8; ++i) {
+            const bool reaches = (w.begin(i) < e_hi) & (w.end[i] > e_lo);  // unused entries end at 0
+            first_run = reaches && base + i < first_run ? base + i : first_run;
+            last_run = reaches ? base + i : last_run;
+        }
+    }
+    // one run at a time (not unrolled: one copy of the fold, whose seed rank and direction are uniform)
+#pragma unroll 1
+    for (uint32_t i = first_run; i <= last_run && i < L.nruns; ++i) {
+        const uint64_t run_begin = i ? L.end[i - 1] : 0, run_end = L.end[i];
+        const uint32_t b = uint32_t((run_begin > e_lo ? run_begin : e_lo) - e_lo);
+        const uint32_t e = uint32_t((run_end < e_hi ? run_end : e_hi) - e_lo);
+        const uint32_t meta = L.meta[i];
+        const uint32_t start = meta_start(meta), out_first = meta_out_first(meta);
+        const int dir = meta_dir(meta);
+        const uint64_t shift = L.unshifted ? 0 : L.shift[i];
+        // the inputs come from LDS by rank, in the run's order: no copy of the fold per seed rank, no registers held
         u32x4 res;
         if constexpr (TREE) {
-            u32x4 x[K];
+            u32x4 y[K];
 #pragma unroll
-            for (int r = 0; r < K; ++r) x[r] = staged[r][tid];
-            res = tree_from<T, OP, K>(x, start);
+            for (int v = 0; v < K; ++v) y[v] = staged[rotate_rank(start, 1, uint32_t(v), K)][tid];
+            res = tree_static<T, OP, K, 0>(y);
         } else {
             AccFor<T, OP> acc;
             acc.seed(staged[start][tid]);
@@ -896,49 +979,95 @@ __device__ __forceinline__ void flat_tile_across_runs(const FlatLaunch& L, uint3
             for (uint32_t j = 1; j < uint32_t(K); ++j) acc.fold(staged[rotate_rank(start, dir, j, K)][tid], new_wins);
             res = acc.finish();
         }
-        const uint64_t out_el = lane_lo - shift;
-        if (nout == uint32_t(K) && L.unshifted) {
-            // all_reduce: every rank's copy of the tile, at the inputs' offset, with the stores of the main path
-            const uint64_t tile_off = e_lo * sizeof(T);
+        const uint32_t lo = lane_off > b ? lane_off : b;
+        const uint32_t hi = lane_off + EPV < e ? lane_off + EPV : e;
+        if (!pending || lo >= hi) continue;
+        VecOf<T> v;
+        v.raw = res;
+        if constexpr (MERGE) {
+            // every rank receives the whole tile at the inputs' offsets: the lane collects its vector, the caller stores it
+            VecOf<T> sum;
+            sum.raw = merged;
 #pragma unroll
-            for (int m = 0; m < K; ++m) store_tile_vec(static_cast<char*>(L.out[m]) + tile_off, tid, res, (L.exchange & kFlatKeep) != 0);
+            for (uint32_t k = 0; k < EPV; ++k)
+                if (lane_off + k >= lo && lane_off + k < hi) sum.v[k] = v.v[k];
+            merged = sum.raw;
         } else {
-#pragma unroll 1
-            for (uint32_t m = 0; m < nout; ++m)
-                store_vec(reinterpret_cast<char*>(static_cast<T*>(L.out[rotate_rank(out_first, 1, m, K)]) + out_el), res);
+            const uint64_t tile_out = (e_lo - shift) * sizeof(T);  // where the tile begins in the outputs, in bytes
+            const bool whole_vector = hi - lo == EPV;
+            for (uint32_t m = 0; m < nout; ++m) {
+                char* out_tile = static_cast<char*>(L.out[rotate_rank(out_first, 1, m, K)]) + tile_out;
+                if (whole_vector) {
+                    store_tile_any(out_tile, tid, res, keep);
+                } else {
+                    T* out = reinterpret_cast<T*>(out_tile) + lane_off;
+#pragma unroll
+                    for (uint32_t k = 0; k < EPV; ++k)
+                        if (lane_off + k >= lo && lane_off + k < hi) out[k] = v.v[k];
+                }
+            }
         }
     }
-    if (!__builtin_amdgcn_ballot_w64(lr.cut)) return;
-    for (uint32_t i = 0; i < L.nruns; ++i) {
-        const uint64_t run_begin = i ? L.end[i - 1] : 0, run_end = L.end[i];
-        const uint64_t b = run_begin > e_lo ? run_begin : e_lo;
-        const uint64_t e = run_end < e_hi ? run_end : e_hi;
-        if (b >= e) continue;
-        const bool whole = lane_lo >= b && lane_lo + EPV <= e;
-        if (whole || lane_lo >= e || lane_lo + EPV <= b) continue;
-        const uint32_t rstart = meta_start(L.meta[i]);
-        const int rdir = meta_dir(L.meta[i]);
-        const uint32_t rout = meta_out_first(L.meta[i]);
-        const uint64_t rshift = L.shift[i];
-#pragma unroll 1
-        for (uint32_t k = 0; k < EPV; ++k) {
-            const uint64_t el = lane_lo + k;
-            if (el < b || el >= e) continue;
-            T r;
-            if constexpr (TREE) {
-                r = tree_element<T, OP, K>(L, K, rstart, el);
-            } else {
-                A a = static_cast<A>(static_cast<const T*>(L.in[rstart])[el]);
-#pragma unroll 1
-                for (uint32_t j = 1; j < uint32_t(K); ++j)
-                    a = combine<OP, A>(
-                            a, static_cast<A>(static_cast<const T*>(L.in[rotate_rank(rstart, rdir, j, K)])[el]),
-                            new_wins);
-                r = static_cast<T>(a);
-            }
-#pragma unroll 1
-            for (uint32_t m = 0; m < nout; ++m)
-                static_cast<T*>(L.out[rotate_rank(rout, 1, m, K)])[el - rshift] = r;
+}
+
+// A tile of a flat launch that no single run covers (or that the buffers' end cuts, `whole` false), from the lane's
+// vectors x[r]; `staged` is LDS of K x 64 vectors that this wavefront may use, and holds them already if `parked`.
+// Where every rank receives the whole tile at the inputs' offsets (all_reduce) each lane collects its vector of
+// results, whatever runs it spans, and the tile is stored like any other: whole cache lines, once.  Otherwise the
+// pieces go to their runs' outputs as they are folded.
+template <typename T, int OP, int K, bool TREE>
+__device__ __forceinline__ void flat_tile_uncovered(const FlatLaunch& L, uint32_t tile, uint32_t tid, u32x4 (&x)[K],
+                                                    u32x4 (*staged)[kThreads], bool parked, bool whole, const RunBatch& first) {
+    constexpr uint32_t EPV = kVecBytes / sizeof(T);
+    constexpr uint32_t TILE = kThreads * EPV;
+    const bool merge = L.nout == uint32_t(K) && L.unshifted;
+    const bool keep = (L.exchange & kFlatKeep) != 0;
+    const uint64_t tile_off = uint64_t(tile) * (kThreads * kVecBytes);
+    u32x4 merged = {0u, 0u, 0u, 0u};
+    if (whole) {
+        if (!parked) {
+            // each lane parks its vectors in LDS, where its own run's fold order can index them
+#pragma unroll
+            for (int r = 0; r < K; ++r) staged[r][tid] = x[r];
+        }
+        LaneRun lr;
+        lane_scan<T>(first, tile, tid, lr);
+        for (uint32_t base = 8; base < L.nruns; base += 8) lane_scan<T>(load_batch(L, base), tile, tid, lr);
+        merged = flat_tile_whole_vectors<T, OP, K, TREE>(L, tile, tid, staged, lr, !merge);
+        if (__builtin_amdgcn_ballot_w64(lr.cut)) {
+            if (merge) flat_tile_ragged<T, OP, K, TREE, true>(L, tile, tid, staged, lr.cut, merged);
+            else flat_tile_ragged<T, OP, K, TREE, false>(L, tile, tid, staged, lr.cut, merged);
+        }
+        if (merge) {
+#pragma unroll
+            for (int m = 0; m < K; ++m) store_tile_vec(static_cast<char*>(L.out[m]) + tile_off, tid, merged, keep);
+        }
+        return;
+    }
+    // the buffers' last tile
+    load_tile_at_the_end<T, K>(L, tile, tid, x, &staged[0][0]);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int r = 0; r < K; ++r) staged[r][tid] = x[r];
+    if (!merge) {
+        flat_tile_ragged<T, OP, K, TREE, false>(L, tile, tid, staged, true, merged);
+        return;
+    }
+    flat_tile_ragged<T, OP, K, TREE, true>(L, tile, tid, staged, true, merged);
+    const uint32_t nvalid = uint32_t(L.count - uint64_t(tile) * TILE);
+    const uint32_t nfull = nvalid / EPV, ntail = nvalid % EPV;
+    VecOf<T> v;
+    v.raw = merged;
+#pragma unroll
+    for (int m = 0; m < K; ++m) {
+        char* out_tile = static_cast<char*>(L.out[m]) + tile_off;
+        if (tid < nfull) {
+            store_tile_any(out_tile, tid, merged, keep);
+        } else if (tid == nfull) {  // the elements behind the last whole vector
+            T* out = reinterpret_cast<T*>(out_tile) + tid * EPV;
+#pragma unroll
+            for (uint32_t k = 0; k < EPV; ++k)
+                if (k < ntail) out[k] = v.v[k];
         }
     }
 }
@@ -992,18 +1121,8 @@ __device__ __forceinline__ void flat_tile(const FlatLaunch& L, uint32_t tile, ui
         return;
     }
 
-    if (whole) {
-        // each lane parks its vectors in LDS, where its own run's fold order can index them
-        __shared__ u32x4 parked[K][kThreads];
-#pragma unroll
-        for (int r = 0; r < K; ++r) parked[r][tid] = x[r];
-        LaneRun lr;
-        lane_scan<T>(first, tile, tid, lr);
-        for (uint32_t base = 8; base < L.nruns; base += 8) lane_scan<T>(load_batch(L, base), tile, tid, lr);
-        flat_tile_across_runs<T, OP, K, TREE>(L, tile, tid, parked, lr);
-    } else {
-        flat_tile_by_element<T, OP, K, TREE>(L, tile, tid);
-    }
+    __shared__ u32x4 parked[K][kThreads];
+    flat_tile_uncovered<T, OP, K, TREE>(L, tile, tid, x, parked, false, whole, first);
 }
 
 // TREE selects the binomial-tree combination; it is a template parameter, not a run-time branch,
@@ -1111,13 +1230,11 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_group_kernel(cons
         }
     } else if (!live) {
         // nothing is stored
-    } else if ((uint64_t(mine) + 1) * TILE <= L.count) {
-        // inside the buffers but across run borders: from the staged vectors, stored by this wavefront
-        LaneRun lr;
-        for (uint32_t base = 0; base < L.nruns; base += 8) lane_scan<T>(load_batch(L, base), mine, tid, lr);
-        flat_tile_across_runs<T, OP, K, TREE>(L, mine, tid, stage[wave], lr);
     } else if (mine < L.total_tiles) {
-        flat_tile_by_element<T, OP, K, TREE>(L, mine, tid);  // the buffers' last, partial tile
+        // across run borders (from the staged vectors), or the buffers' last, partial tile (which nobody has loaded);
+        // stored by this wavefront
+        const bool whole = (uint64_t(mine) + 1) * TILE <= L.count;
+        flat_tile_uncovered<T, OP, K, TREE>(L, mine, tid, x, stage[wave], whole, whole, load_batch(L, 0));
     }
     if (exchange) {
         if (tid == 0) folded[wave] = run >= 0 ? 1u : 0u;
