@@ -335,55 +335,55 @@ __device__ __forceinline__ SegmentView find_segment(const FoldLaunch& L, uint32_
 }
 
 // Element tiles: run heads / tails and buffers that are not 16-byte aligned.  A lane takes
-// kElemsPerLane elements, a wavefront's lanes consecutive ones, four at a time in flight.
+// elems_per_lane(L) elements, a wavefront's lanes consecutive ones, four at a time; the loads of up to eight ranks
+// are in flight together (one memory round trip for up to nine inputs, not one per input).
 template <typename T, int OP>
 __device__ __forceinline__ void fold_element_tile(const FoldLaunch& L, const SegmentView& sv, uint32_t nfold,
                                                   uint32_t local_tile, uint32_t tid) {
     using A = typename Wide<T>::type;
-    constexpr uint32_t G = 4;
+    constexpr uint32_t G = 4, B = 8;
     const uint64_t in_begin = sv.in_begin, out_begin = sv.out_begin, count = sv.count;
     const uint32_t start = sv.start, out_first = sv.out_first, nr = L.nranks, nout = L.nout;
     const int dir = sv.dir;
     const bool new_wins = L.new_wins_ties != 0;
-    const uint64_t ebase = uint64_t(local_tile) * (kThreads * kElemsPerLane);
-    for (uint32_t g = 0; g < kElemsPerLane; g += G) {
+    const uint32_t per_lane = elems_per_lane(L);
+    const uint64_t ebase = uint64_t(local_tile) * (kThreads * per_lane);
+    for (uint32_t g = 0; g < per_lane; g += G) {
         const uint64_t gbase = ebase + uint64_t(g) * kThreads;
         if (gbase >= count) break;
         const uint64_t left = count - gbase;
         const uint64_t ie = in_begin + gbase + tid;
         const uint64_t oe = out_begin + gbase + tid;
-        if (left >= uint64_t(G) * kThreads) {
-            A a[G];
-            const T* seed = static_cast<const T*>(L.in[start]) + ie;
+        bool have[G];
 #pragma unroll
-            for (uint32_t q = 0; q < G; ++q) a[q] = static_cast<A>(seed[q * kThreads]);
-            for (uint32_t j = 1; j < nfold; ++j) {
-                const T* src = static_cast<const T*>(L.in[rotate_rank(start, dir, j, nr)]) + ie;
-                T x[G];
+        for (uint32_t q = 0; q < G; ++q) have[q] = uint64_t(q) * kThreads + tid < left;
+        A a[G];
+        const T* seed = static_cast<const T*>(L.in[start]) + ie;
 #pragma unroll
-                for (uint32_t q = 0; q < G; ++q) x[q] = src[q * kThreads];
+        for (uint32_t q = 0; q < G; ++q) a[q] = have[q] ? static_cast<A>(seed[q * kThreads]) : A(0);
+        for (uint32_t j0 = 1; j0 < nfold; j0 += B) {
+            T x[B][G];
 #pragma unroll
-                for (uint32_t q = 0; q < G; ++q) a[q] = combine<OP, A>(a[q], static_cast<A>(x[q]), new_wins);
+            for (uint32_t b = 0; b < B; ++b) {
+                if (j0 + b < nfold) {
+                    const T* src = static_cast<const T*>(L.in[rotate_rank(start, dir, j0 + b, nr)]) + ie;
+#pragma unroll
+                    for (uint32_t q = 0; q < G; ++q) x[b][q] = have[q] ? src[q * kThreads] : T(0);
+                }
             }
-            for (uint32_t m = 0; m < nout; ++m) {
-                T* dst = static_cast<T*>(L.out[rotate_rank(out_first, 1, m, nr)]) + oe;
 #pragma unroll
-                for (uint32_t q = 0; q < G; ++q) dst[q * kThreads] = static_cast<T>(a[q]);
+            for (uint32_t b = 0; b < B; ++b) {
+                if (j0 + b < nfold) {
+#pragma unroll
+                    for (uint32_t q = 0; q < G; ++q) a[q] = combine<OP, A>(a[q], static_cast<A>(x[b][q]), new_wins);
+                }
             }
-        } else {
-            for (uint32_t q = 0; q < G; ++q) {
-                const uint32_t e = q * kThreads + tid;
-                if (e >= left) break;
-                A a = static_cast<A>(static_cast<const T*>(L.in[start])[ie + q * kThreads]);
-                for (uint32_t j = 1; j < nfold; ++j)
-                    a = combine<OP, A>(
-                            a,
-                            static_cast<A>(static_cast<const T*>(L.in[rotate_rank(start, dir, j, nr)])[ie + q * kThreads]),
-                            new_wins);
-                const T r = static_cast<T>(a);
-                for (uint32_t m = 0; m < nout; ++m)
-                    static_cast<T*>(L.out[rotate_rank(out_first, 1, m, nr)])[oe + q * kThreads] = r;
-            }
+        }
+        for (uint32_t m = 0; m < nout; ++m) {
+            T* dst = static_cast<T*>(L.out[rotate_rank(out_first, 1, m, nr)]) + oe;
+#pragma unroll
+            for (uint32_t q = 0; q < G; ++q)
+                if (have[q]) dst[q * kThreads] = static_cast<T>(a[q]);
         }
     }
 }
@@ -400,8 +400,15 @@ __device__ __forceinline__ void fold_vector_remainder(const FoldLaunch& L, const
     const uint64_t out_off = sv.out_begin * sizeof(T) + (vbase + tid) * kVecBytes;
     AccFor<T, OP> a;
     a.seed(load_vec(static_cast<const char*>(L.in[sv.start]) + in_off));
-    for (uint32_t j = 1; j < nfold; ++j)
-        a.fold(load_vec(static_cast<const char*>(L.in[rotate_rank(sv.start, sv.dir, j, nr)]) + in_off), new_wins);
+    for (uint32_t j0 = 1; j0 < nfold; j0 += 8) {  // the loads of up to eight ranks in flight together
+        u32x4 x[8];
+#pragma unroll
+        for (uint32_t b = 0; b < 8; ++b)
+            if (j0 + b < nfold) x[b] = load_vec(static_cast<const char*>(L.in[rotate_rank(sv.start, sv.dir, j0 + b, nr)]) + in_off);
+#pragma unroll
+        for (uint32_t b = 0; b < 8; ++b)
+            if (j0 + b < nfold) a.fold(x[b], new_wins);
+    }
     const u32x4 r = a.finish();
     for (uint32_t m = 0; m < L.nout; ++m)
         store_vec(static_cast<char*>(L.out[rotate_rank(sv.out_first, 1, m, nr)]) + out_off, r);
@@ -476,8 +483,9 @@ __device__ __forceinline__ void fold_tile(const FoldLaunch& L) {
         // A tile is kVecIters groups of kThreads vectors, taken one after the other: the segment
         // lookup above is paid once per tile while the registers of one group suffice.
         const uint64_t nvec = sv.count / EPV;
-        for (uint32_t it = 0; it < kVecIters; ++it) {
-            const uint64_t vbase = (uint64_t(local_tile) * kVecIters + it) * kThreads;
+        const uint32_t iters = vec_iters(L);
+        for (uint32_t it = 0; it < iters; ++it) {
+            const uint64_t vbase = (uint64_t(local_tile) * iters + it) * kThreads;
             if (vbase >= nvec) break;
             const uint64_t left = nvec - vbase;  // vectors from this group's start to the segment's end
             if (left < kThreads) {
@@ -496,20 +504,22 @@ __device__ __forceinline__ void fold_tile(const FoldLaunch& L) {
 #pragma unroll
                 for (int j = 1; j < K; ++j) acc.fold(x[j], new_wins);
             } else {
-                acc.seed(load_tile_any(static_cast<const char*>(L.in[start]) + in_off, tid));
-                uint32_t j = 1;
-                for (; j + 4 <= nfold; j += 4) {
-                    u32x4 x[4];
+                // seven inputs at a time in flight, the seed among the first (eight cost twice the registers)
+                for (uint32_t j0 = 0; j0 < nfold; j0 += 7) {
+                    u32x4 x[7];
 #pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        x[q] = load_tile_any(
-                                static_cast<const char*>(L.in[rotate_rank(start, dir, j + q, nr)]) + in_off, tid);
+                    for (uint32_t q = 0; q < 7; ++q)
+                        if (j0 + q < nfold)
+                            x[q] = load_tile_any(
+                                    static_cast<const char*>(L.in[rotate_rank(start, dir, j0 + q, nr)]) + in_off, tid);
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) acc.fold(x[q], new_wins);
+                    for (uint32_t q = 0; q < 7; ++q) {
+                        if (j0 + q < nfold) {
+                            if (j0 + q == 0) acc.seed(x[q]);
+                            else acc.fold(x[q], new_wins);
+                        }
+                    }
                 }
-                for (; j < nfold; ++j)
-                    acc.fold(load_tile_any(static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off, tid),
-                             new_wins);
             }
             const u32x4 res = acc.finish();
             for (uint32_t m = 0; m < nout; ++m)

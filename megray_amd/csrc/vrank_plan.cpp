@@ -259,6 +259,9 @@ private:
             if (natural || same_phase(r)) vector_elems += r.count;
         m_waves = vector_elems / (kThreads * epv) >= kGroupMinTiles ? kGroupWaves : 1;
         m_paced = m_waves == kGroupWaves && m_nfold >= 3 && paced_launch(m_in, m_out, m_nranks, vector_elems * m_elem, false, m_nout);
+        uint64_t all_elems = 0;
+        for (const Run& r : m_runs) all_elems += r.count;
+        m_short = m_waves == 1 && all_elems * m_elem <= kShortTilesMaxBytes;  // short launches: small tiles, more wavefronts
         open_launch();
         for (const Run& r : m_runs) {
             const bool vector = natural || same_phase(r);
@@ -315,6 +318,7 @@ private:
         m_launch.elem_size = m_elem;
         m_launch.waves = m_waves;
         m_launch.paced = m_paced ? 1 : 0;
+        m_launch.short_tiles = m_short ? 1 : 0;
     }
 
     void close_launch() {
@@ -366,6 +370,7 @@ private:
     uint64_t m_grid = kVecBytes;
     bool m_tree = false;
     uint32_t m_waves = 1;
+    bool m_short = false;
     bool m_paced = false;
     std::vector<Run> m_runs;
     FoldLaunch m_launch;
