@@ -294,11 +294,12 @@ def other_layout_fresh(args):
             raise SystemExit(f"bench: {' '.join(cmd)} failed:\n{proc.stdout}\n{proc.stderr}")
         child = json.loads([line for line in proc.stdout.splitlines() if line.startswith("{")][-1])
         runs.append((child["roofline"]["frac"], child["roofline"]["kernel_ms"]))
+    in_order = [round(100.0 * f, 2) for f, _ in runs]
     runs.sort()
     frac, ms = runs[1]
     return {"layout": LAYOUT_TEXT[other], "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
             "pct_of_peak": round(100.0 * frac, 2), "process": "median of three processes of their own, buffers allocated first thing",
-            "all_three_pct": [round(100.0 * f, 2) for f, _ in runs]}
+            "all_three_pct": in_order}  # in the order they ran
 
 
 def copy_yardstick(torch, mr):
