@@ -720,7 +720,15 @@ Status add_pack(Plan& plan, const void* const* in, void* const* out, uint32_t nr
     L.ncopies = ncopies;
     L.width = common_width(block_bytes, in, out_c, nranks);
     const uint64_t tiles = pack_tiles(block_bytes);
-    L.waves = tiles >= kGroupMinTiles / 4 ? kGroupWaves : 1;  // long blocks take the group form
+    // Long blocks take the group form.  An all_to_all of five ranks and more is a launch of 25 and more copies
+    // whichever form it takes, and up to 4 MiB per block one wavefront per tile serves it better: the group form's
+    // grid comes in runs of 32 workgroups per copy, half of them idle on a block of 129 tiles.  Measured on MI355X,
+    // uint8, microseconds per all_to_all, group form -> one wavefront per tile, blocks of 128 KiB / 512 KiB / 2 MiB / 4 MiB:
+    //   16 ranks 18.3 -> 12.3 / 45.5 -> 40.4 / 160 -> 159 / 314 -> 318;  8 ranks 6.2 -> 4.6 / 13.2 -> 12.1 / 41.1 -> 39.7 / 80.5 -> 81.0;
+    //   5 ranks 4.4 -> 3.8 / 6.3 -> 6.1 / 17.8 -> 17.1 / 31.9 -> 31.4;  4 ranks 3.3 -> 3.4 / 4.9 -> 4.6 / 12.0 -> 12.1 / 21.4 -> 21.5 (left alone).
+    // all_gather and broadcast need the group form from 128 tiles on (8 ranks x 128 KiB: 4.7 against 5.4 us; 16 MiB: 181 against 234).
+    const uint64_t group_min = mode == kPackAllToAll && nranks >= 5 ? 4096 : kGroupMinTiles / 4;
+    L.waves = tiles >= group_min ? kGroupWaves : 1;
     if (L.waves == kGroupWaves && mode == kPackAllGather) L.paced = paced_gather(nranks, block_bytes) ? 1 : 0;
     if (L.waves == kGroupWaves && mode == kPackBroadcast) L.paced = paced_broadcast(nranks, block_bytes) ? 1 : 0;
     // A grid holds 2^31 - 1 workgroups: blocks whose tiles, over all copies, outnumber that are cut into
