@@ -660,14 +660,18 @@ namespace {
 //   9 ranks     76.8 -> 76.8 / 82.5 -> 82.4 / 84.1 -> 84.2 / 84.6 -> 84.6      (allocated one by one, 16 / 64 MiB: 80.6 -> 83.4 / 80.9 -> 84.6)
 //   12 ranks    79.6 -> 81.6 / 78.0 -> 81.3 / 82.5 -> 84.4 / 81.9 -> 84.6      (allocated one by one: 77.4 -> 83.7 / 75.1 -> 80.2 / 80.6 -> 83.1 / 79.8 -> 84.5)
 //   16 ranks    79.6 -> 80.7 / 76.5 -> 81.8 / 78.0 -> 83.9 / 78.2 -> 82.9      (allocated one by one: 69.1 -> 81.5 / 75.0 -> 80.6 / 77.4 -> 84.5 / 76.2 -> 83.2)
-// So: twelve ranks and more from blocks of a MiB; six ranks and more from 768 MiB written in all; four and five ranks
+// all_gather, fp32, 6 / 7 / 8 / 10 ranks, outputs of 48 / 64 / 96 MiB per rank, placed | placed for the all_gather | one by one:
+//   6 ranks   77.0 -> 80.0 | 80.5 -> 79.7 | 79.7 -> 79.9     79.4 -> 81.8 | 82.6 -> 82.2 | 82.7 -> 82.2     80.1 -> 82.8 | 82.5 -> 82.4 | 80.8 -> 82.1
+//   8 ranks   79.3 -> 80.5 | 80.5 -> 80.3 | 78.3 -> 80.0     80.1 -> 82.1 | 81.7 -> 81.8 | 77.6 -> 81.8     80.4 -> 82.9 | 83.0 -> 83.0 | 81.7 -> 82.5
+//   10 ranks  76.2 -> 80.6 | 76.9 -> 80.7 | 76.7 -> 79.8     76.2 -> 80.9 | 76.9 -> 81.3 | 77.4 -> 81.9     76.8 -> 82.4 | 76.6 -> 82.8 | 77.3 -> 82.2
+// So: twelve ranks and more from blocks of a MiB; six ranks and more from 384 MiB written in all; four and five ranks
 // from 2 GiB written; where the outputs lie does not enter.
 bool paced_gather(uint32_t nranks, uint64_t block_bytes) {
     if (pace_override() >= 0) return pace_override() == 1;
     constexpr uint64_t kMiB = uint64_t(1) << 20;
     const uint64_t written = block_bytes * nranks * nranks;
     if (nranks >= 12) return block_bytes >= kMiB;
-    if (nranks >= 6) return written >= 768 * kMiB;
+    if (nranks >= 6) return written >= 384 * kMiB;
     return nranks >= 4 && written >= 2048 * kMiB;
 }
 

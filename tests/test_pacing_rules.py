@@ -76,9 +76,10 @@ def gather_layout(count, size, start):
 def test_all_gather_paces_its_stores_by_rank_count_and_bytes_written_wherever_the_outputs_lie():
     for layout in (separate, placed, gather_layout):
         assert all_gather_paced(8, 16 * MIB, layout)            # 1 GiB written
-        assert all_gather_paced(6, 22 * MIB, layout)            # 792 MiB
-        assert not all_gather_paced(8, 8 * MIB, layout)         # 512 MiB
-        assert not all_gather_paced(6, 21 * MIB, layout)        # 756 MiB
+        assert all_gather_paced(8, 6 * MIB, layout)             # 384 MiB
+        assert all_gather_paced(6, 11 * MIB, layout)            # 396 MiB
+        assert not all_gather_paced(8, 5 * MIB, layout)         # 320 MiB
+        assert not all_gather_paced(6, 10 * MIB, layout)        # 360 MiB
         assert all_gather_paced(4, 128 * MIB, layout)           # 2 GiB
         assert not all_gather_paced(5, 64 * MIB, layout)        # 1.6 GiB on fewer than six ranks
         assert not all_gather_paced(3, 512 * MIB, layout)       # fewer than four ranks: never
