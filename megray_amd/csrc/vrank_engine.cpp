@@ -98,7 +98,9 @@ namespace {
 //   all_reduce shapes (every rank an output), accesses at once, 256 MiB per rank -> 4 per CU:
 //     6 / 7 / 10 / 12 / 16 ranks 81.3 -> 82.3 / 81.5 -> 82.0 / 80.5 -> 82.5 / 80.3 -> 81.8 / 80.9 -> 81.6
 //     (3 per CU: 78 / 80 / 81.3 / 82.2 / 82.1; 5 per CU: 82.4 / 82.3 / 81.6 / 81.0 / 81.9); 64 MiB per rank, 6 / 7 / 12 ranks:
-//     78.9 -> 79.7 / 78.7 -> 80.8 / 78.6 -> 80.8; 5 ranks gain nothing at any occupancy
+//     78.9 -> 79.7 / 78.7 -> 80.8 / 78.6 -> 80.8; 16 / 32 MiB per rank, 6 / 7 / 10 / 12 / 16 ranks: 77.8 -> 78.8 / 75.7 -> 78.3 / 71.7 -> 72.9 /
+//     71.7 -> 73.9 / 72.7 -> 75.7 and 74.9 -> 75.2 / 76.1 -> 78.1 / 75.5 -> 77.2 / 76.3 -> 78.4 / 77.3 -> 79.5; at 8 MiB + 1 to - 1;
+//     5 ranks gain nothing at any occupancy
 //   folds into one output that pace their accesses (reduce_scatter from 1 GiB over all buffers) -> 6 per CU:
 //     6 / 7 / 10 / 12 / 16 ranks x 256 MiB 80.1 -> 84.0 / 80.9 -> 83.6 / 81.7 -> 83.7 / 82.0 -> 84.2 / 84.3 -> 85.4 (5 ranks 82.8 -> 82.3;
 //     at 7 per CU, reserved the same way, nothing changes; 5 per CU loses 1 - 7 points)
@@ -118,7 +120,7 @@ uint32_t flat_group_per_cu(const FlatLaunch& L) {
 uint32_t general_group_per_cu(const FoldLaunch& L) {
     if (L.nfold < 6 || L.nfold == 8) return 0;  // 1, 2, 3, 4 and 8 inputs run kernels of their own
     if (L.nout == 1) return L.paced ? 6u : 0u;
-    const bool long_launch = L.total_tiles >= 16384;  // 64 MiB per buffer: a workgroup takes 4 KiB of each
+    const bool long_launch = L.total_tiles >= 4096;  // 16 MiB per buffer: a workgroup takes 4 KiB of each
     return L.nout == L.nranks && !L.paced && long_launch ? 4u : 0u;
 }
 }  // namespace
