@@ -154,7 +154,7 @@ Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCal
                     // the planner leaves a launch this large at one wavefront per tile only to have it run at a
                     // reduced occupancy (flat_one_out)
                     if (step.flat.total_tiles >= kFlatOneOutMinTiles)
-                        call.lds = lds_for_waves_per_cu(call.kernel, flat_one_out_waves_per_cu(step.flat.nranks));
+                        call.lds = lds_for_waves_per_cu(call.kernel, flat_one_out_waves_per_cu(step.flat.nranks, step.flat.total_tiles));
                 }
                 break;
             case Step::kTree:

@@ -177,10 +177,20 @@ constexpr uint32_t kFlatGroupMinTiles = 2048;
 //            the group form
 // Below 8192 tiles per buffer the group form is level or ahead.  (The figures in parentheses are what was asked
 // for at the time; LDS is handed out in 128 units per CU, so 13 / 12 / 11 / 10 / 9 / 5 asked for were 12 / 11 / 10 / 9 / 9 / 4
-// had: the four-rank launches have always run at 12.)
+// had: the four-rank launches have always run at 12.)  With the occupancy set exactly, eight ranks of fp32 by size
+// of one rank's buffer, 7 / 8 / 9 / 10 wavefronts per CU, buffers placed (and on separate allocations):
+//   reduce_scatter  32 MiB 79.6 / 83.5 / 84.1 / 84.8 (83.4 / 83.4 / 81.8 / 80.2)   64 MiB 84.7 / 87.2 / 88.1 / 87.3 (84.7 / 87.7 / 87.9 / 87.3)
+//                   128 MiB - / 89.0 / 89.9 / 89.3                                  256 MiB 85.2 / 86.8 / 84.6 / 83.0 (78.7 / 78.1 / 77.8 / 77.6)
+//                   512 MiB 85.0 / 86.2 / 83.8 / 82.3 (79.3 / 78.5 / 78.0 / 77.8)
+//   reduce          32 MiB 79.2 / 81.3 / 83.9 / 83.9 (77.6 / 80.5 / 81.4 / 80.5)   64 MiB 83.0 / 84.7 / 86.9 / 87.4 (81.7 / 84.3 / 85.3 / 85.1)
+//                   256 MiB 83.5 / 84.7 / 83.7 / 83.1 (79.4 / 80.6 / 80.7 / 80.4)   512 MiB 83.4 / 84.4 / 83.5 / 82.8 (77.8 / 78.5 / 78.0 / 77.8)
+// so eight ranks run at 9 below 256 MiB per buffer and at 8 from there on (fp16 at 128 MiB: 87.6 / 90.0 / 89.6 at 8 / 9 / 10).
+// Four ranks at 128 MiB per buffer, 10 / 11 / 12 / 14 / 16 per CU: fp32 87.6 / 90.4 / 92.0 / 89.7 / 87.6, fp16 85.4 / 89.4 / 92.0 /
+// 92.3 / 88.2; three ranks are level from 10 to 18.
 constexpr uint32_t kFlatOneOutMinTiles = 8192;
-constexpr uint32_t flat_one_out_waves_per_cu(uint32_t nranks) {
-    return nranks >= 8 ? 8u : nranks == 4 ? 12u : 14u;
+constexpr uint32_t kFlatOneOutEightRanksLargeTiles = 1u << 18;  // 256 MiB per buffer
+constexpr uint32_t flat_one_out_waves_per_cu(uint32_t nranks, uint32_t tiles_per_buffer) {
+    return nranks >= 8 ? (tiles_per_buffer < kFlatOneOutEightRanksLargeTiles ? 9u : 8u) : nranks == 4 ? 12u : 14u;
 }
 // The tree kernel (reduce towards a root for rank counts the flat kernels do not have) walks its tree depth first with
 // a few loads in flight per wavefront, and likes 16 wavefronts per CU for elements of 4 and 8 bytes from 64 MiB per buffer
