@@ -151,10 +151,13 @@ Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCal
                     if (per_cu) call.lds = lds_for_waves_per_cu(call.kernel, per_cu);
                 } else {
                     call = {flat_kernel_for(step.flat, dtype, op), step.flat.total_tiles, kThreads, &step.flat};
-                    // the planner leaves a launch this large at one wavefront per tile only to have it run at a
-                    // reduced occupancy (flat_one_out)
-                    if (step.flat.total_tiles >= kFlatOneOutMinTiles)
-                        call.lds = lds_for_waves_per_cu(call.kernel, flat_one_out_waves_per_cu(step.flat.nranks, step.flat.total_tiles));
+                    // the planner leaves a launch this large at one wavefront per tile only to have it run at an
+                    // occupancy of its own (flat_one_out_waves_per_cu)
+                    if (step.flat.total_tiles >= kFlatOneOutMinTiles) {
+                        const bool keep = (step.flat.exchange & kFlatKeep) != 0;
+                        const uint32_t per_cu = flat_one_out_waves_per_cu(step.flat.nranks, step.flat.total_tiles, keep, step.flat.elem_size);
+                        if (per_cu) call.lds = lds_for_waves_per_cu(call.kernel, per_cu);
+                    }
                 }
                 break;
             case Step::kTree:

@@ -163,34 +163,64 @@ constexpr uint32_t kGroupStoresInFlight = 2;
 constexpr uint32_t kGroupMinTiles = 512;
 constexpr uint32_t kFlatGroupMinTiles = 2048;
 // Large flat folds with ONE output (reduce_scatter, reduce, the first launch of the two-phase all_reduce), three
-// or more inputs and input tiles on cache-line boundaries stay at one wavefront per tile and run at a reduced occupancy
-// instead: a wavefront has its K loads of 1 KiB in flight at once, and what HBM needs to stay busy (bandwidth x
+// or more inputs and input tiles on cache-line boundaries stay at one wavefront per tile and run at an occupancy of
+// their own: a wavefront has its K loads of 1 KiB in flight at once, and what HBM needs to stay busy (bandwidth x
 // latency, 32 - 64 KiB per CU) is in flight with far fewer wavefronts than a CU can hold - the rest only queue up
 // in the memory system and get in each other's way.  The occupancy is set by LDS reserved per workgroup at launch,
-// on top of what the kernel declares, which nothing ever touches (lds_for_waves_per_cu).  Measured on MI355X, % of
-// the HBM peak, fp32, 2^26 elements per rank (fp16, int8 and int64 behave alike), group form against one wavefront
-// per tile at the given wavefronts per CU:
-//   8 ranks  reduce_scatter 81 against 83 (12), 85 (10), 85 (9), 86 - 87 (8), 84 (7), 78 (6), 69 (5); reduce 82 against 87 (8)
-//   4 ranks  reduce_scatter 80 against 85.5 (13), 85.5 (11), 82 (10); reduce 80 against 87 (13), 84 (11), 80 (10)
-//   3 ranks  reduce_scatter 80 against 80 (14), 80 (12), 80 (10); reduce 82 against 86 (14), 81 (12), 77 (10)
-//   2 ranks  84 against 84 (16), 76 (13), 69 (11): two loads per wavefront need every wavefront there is; left in
-//            the group form
-// Below 8192 tiles per buffer the group form is level or ahead.  (The figures in parentheses are what was asked
-// for at the time; LDS is handed out in 128 units per CU, so 13 / 12 / 11 / 10 / 9 / 5 asked for were 12 / 11 / 10 / 9 / 9 / 4
-// had: the four-rank launches have always run at 12.)  With the occupancy set exactly, eight ranks of fp32 by size
-// of one rank's buffer, 7 / 8 / 9 / 10 wavefronts per CU, buffers placed (and on separate allocations):
-//   reduce_scatter  32 MiB 79.6 / 83.5 / 84.1 / 84.8 (83.4 / 83.4 / 81.8 / 80.2)   64 MiB 84.7 / 87.2 / 88.1 / 87.3 (84.7 / 87.7 / 87.9 / 87.3)
-//                   128 MiB - / 89.0 / 89.9 / 89.3                                  256 MiB 85.2 / 86.8 / 84.6 / 83.0 (78.7 / 78.1 / 77.8 / 77.6)
-//                   512 MiB 85.0 / 86.2 / 83.8 / 82.3 (79.3 / 78.5 / 78.0 / 77.8)
-//   reduce          32 MiB 79.2 / 81.3 / 83.9 / 83.9 (77.6 / 80.5 / 81.4 / 80.5)   64 MiB 83.0 / 84.7 / 86.9 / 87.4 (81.7 / 84.3 / 85.3 / 85.1)
-//                   256 MiB 83.5 / 84.7 / 83.7 / 83.1 (79.4 / 80.6 / 80.7 / 80.4)   512 MiB 83.4 / 84.4 / 83.5 / 82.8 (77.8 / 78.5 / 78.0 / 77.8)
-// so eight ranks run at 9 below 256 MiB per buffer and at 8 from there on (fp16 at 128 MiB: 87.6 / 90.0 / 89.6 at 8 / 9 / 10).
-// Four ranks at 128 MiB per buffer, 10 / 11 / 12 / 14 / 16 per CU: fp32 87.6 / 90.4 / 92.0 / 89.7 / 87.6, fp16 85.4 / 89.4 / 92.0 /
-// 92.3 / 88.2; three ranks are level from 10 to 18.
-constexpr uint32_t kFlatOneOutMinTiles = 8192;
-constexpr uint32_t kFlatOneOutEightRanksLargeTiles = 1u << 18;  // 256 MiB per buffer
-constexpr uint32_t flat_one_out_waves_per_cu(uint32_t nranks, uint32_t tiles_per_buffer) {
-    return nranks >= 8 ? (tiles_per_buffer < kFlatOneOutEightRanksLargeTiles ? 9u : 8u) : nranks == 4 ? 12u : 14u;
+// on top of what the kernel declares, which nothing ever touches (lds_for_waves_per_cu; LDS is handed out in 128
+// units per CU, so only occupancies of 128 / n are to be had).  How many wavefronts serve best depends on the size
+// of the buffers, with a step between 128 and 256 MiB per buffer whatever the number of buffers (see below).  Measured on MI355X,
+// % of the HBM peak, fp32, buffers placed, reduce_scatter (reduce), by MiB per buffer; "group" is the group form,
+// the numbers name wavefronts per CU, "all" no reservation (18 / 25 / 28 per CU for 8 / 4 / 3 ranks):
+//   8 ranks    group        7            8            9            10           12           14           all
+//      8     82.9 (85.7)  79.1 (80.3)  83.7 (83.2)  83.6 (84.0)  84.7 (87.5)  89.5 (93.4)  90.5 (92.8)  89.5 (90.9)
+//     16     85.3 (85.9)  82.1 (79.1)  84.9 (82.2)  85.8 (84.5)  86.9 (87.2)  88.0 (88.6)  88.1 (88.9)  86.7 (87.3)
+//     32     80.2 (80.8)  81.7 (79.0)  84.5 (81.2)  84.7 (84.1)  84.9 (85.0)  84.5 (84.9)  84.4 (84.7)  82.3 (82.8)
+//     64     82.5 (83.1)  85.0 (83.2)  87.5 (85.1)  88.5 (87.7)  87.7 (87.9)  87.3 (87.8)  87.1 (87.3)  84.8 (85.1)
+//    128     83.3 (83.4)  85.5 (84.7)  89.0 (86.8)  89.9 (89.3)  89.1 (89.3)  88.4 (88.9)  88.1 (87.9)  85.8 (85.7)
+//    256     81.1 (81.3)  85.4 (83.5)  87.0 (85.0)  85.1 (84.1)  83.4 (83.4)  82.7 (82.5)  81.6 (81.8)  79.5 (79.3)
+//   1024     82.3 (82.0)  85.9 (84.4)  85.4 (84.7)  84.3 (83.6)  83.1 (82.7)  82.0 (81.7)  80.2 (80.2)  77.7 (77.4)
+//   4 ranks    group        11           12           14           16           18           21           all
+//      8     84.5 (86.1)  74.6 (77.1)  76.2 (79.2)  78.4 (78.3)  80.2 (81.5)  81.1 (81.4)  80.6 (82.2)  81.2 (83.8)
+//     16     89.4 (89.6)  81.4 (83.4)  83.1 (84.0)  85.3 (86.2)  87.2 (89.0)  88.6 (91.0)  91.0 (93.0)  91.5 (91.9)
+//     32     88.7 (88.8)  79.3 (78.5)  81.1 (80.9)  83.0 (82.9)  84.5 (85.2)  85.7 (85.0)  84.3 (82.7)  84.9 (83.3)
+//     64     84.9 (85.0)  86.2 (81.8)  87.4 (82.7)  86.3 (85.1)  86.1 (86.7)  86.2 (86.4)  86.1 (85.2)  85.5 (85.6)
+//    128     86.7 (87.0)  90.3 (85.2)  91.6 (86.3)  90.6 (89.4)  87.6 (88.4)  87.6 (87.6)  88.5 (87.6)  88.4 (87.9)
+//    256     80.2 (80.9)  86.9 (83.8)  87.0 (84.8)  82.6 (82.9)  81.4 (80.5)  81.0 (80.5)  80.7 (80.6)  80.4 (80.2)
+//   1024     81.2 (81.4)  87.9 (85.4)  87.4 (85.9)  83.4 (83.0)  81.8 (82.1)  81.7 (81.7)  81.6 (81.9)  81.4 (81.6)
+//   3 ranks    group        12           14           16           18           21           25           all
+//      8     72.0 (74.5)  70.2 (72.4)  73.0 (74.4)  77.0 (78.4)  77.6 (81.1)  80.9 (83.7)  84.2 (83.2)  83.6 (86.1)
+//     16     87.0 (89.3)  77.6 (79.8)  82.1 (83.6)  84.2 (85.9)  85.6 (87.2)  87.2 (88.2)  87.7 (88.4)  87.9 (88.1)
+//     32     89.1 (90.4)  78.8 (80.1)  81.1 (82.5)  84.1 (84.7)  87.3 (87.5)  90.0 (90.8)  90.5 (90.2)  90.2 (90.4)
+//     64     85.7 (84.8)  77.3 (77.0)  80.0 (80.2)  81.7 (82.1)  84.5 (85.8)  87.5 (88.2)  88.2 (88.6)  88.2 (88.5)
+//    128     88.7 (88.1)  82.2 (81.7)  84.1 (83.5)  86.7 (87.0)  90.0 (90.0)  91.1 (92.1)  91.6 (91.7)  91.1 (92.3)
+//    256     81.2 (81.2)  84.2 (82.2)  86.2 (83.8)  83.9 (83.3)  82.3 (82.3)  81.4 (81.6)  81.1 (81.8)  80.6 (81.7)
+//   1024     82.0 (82.8)  86.3 (83.7)  87.6 (85.2)  84.5 (84.6)  83.5 (83.7)  82.8 (82.5)  82.5 (82.4)  82.7 (82.7)
+//   2 ranks  84 in the group form against 84 / 76 / 69 at 16 / 12 / 11: two loads per wavefront need every wavefront there
+//            is; left in the group form
+// The step between 128 and 256 MiB per buffer is the store policy (kKeepMaxBytes: up to 128 MiB written the stores
+// leave their data in the last-level cache, beyond that they stream past it), not the size: with the policy forced,
+// 8 / 9 / 12 per CU for eight ranks, 12 / 14 / 18 for four, 14 / 18 / all for three, reduce_scatter (reduce):
+//   kept      64 MiB  87.3 / 88.4 / 87.7 (85.5 / 87.9 / 87.1)   87.2 / 86.5 / 84.9 (82.2 / 85.2 / 85.7)   79.4 / 84.5 / 87.5 (80.8 / 85.8 / 88.6)
+//            256 MiB  88.3 / 89.7 / 88.0 (86.8 / 89.4 / 88.2)   93.5 / 92.4 / 88.8 (88.4 / 91.3 / 89.0)   87.4 / 91.9 / 92.0 (85.2 / 91.9 / 92.7)
+//   streamed  64 MiB  85.4 / 84.2 / 82.1 (83.3 / 83.4 / 81.9)   82.3 / 79.5 / 79.3 (79.6 / 79.7 / 78.6)   78.4 / 79.9 / 79.4 (77.8 / 79.6 / 79.4)
+//            256 MiB  87.5 / 85.2 / 82.8 (85.1 / 84.7 / 82.5)   86.8 / 82.5 / 81.0 (84.7 / 82.3 / 79.9)   86.1 / 82.4 / 81.5 (82.9 / 81.9 / 81.1)
+// (buffers of 132 MiB already behave like those of 256: 87.1 / 84.6 at 8 / 9 for eight ranks, 83.8 / 81.3 at 14 / all
+// for three).  Hence, for launches whose stores are kept: eight ranks 14 per CU below 32 MiB per buffer and 9 from there
+// on; four ranks stay in the group form below 64 MiB per buffer, then 14 (elements of 4 and 8 bytes) or 12 (of 1 and
+// 2 bytes: at 64 / 128 MiB fp16 reduce 86.9 / 90.0 at 14 against 87.8 / 91.9 at 12, int8 86.8 / 89.7 against 88.0 /
+// 91.8; fp32 85.3 / 89.3 against 82.1 / 86.3, int64 84.9 / 88.8 against 82.4 / 86.4); three ranks all that fit.  For
+// launches whose stores stream: 8 / 12 / 14 for eight / four / three ranks.  Below 8 MiB per buffer (4 MiB: group
+// 85 - 91 against 80 at best for eight ranks) the group form is level or ahead for every rank count.
+constexpr uint32_t kFlatOneOutMinTiles = 8192;                  // 8 MiB per buffer
+constexpr uint32_t kFlatOneOutMinTilesFourRanks = 65536;        // 64 MiB per buffer
+constexpr uint32_t kFlatOneOutSmallTiles = 32768;               // 32 MiB per buffer
+// wavefronts per CU of such a launch; 0 = all that fit
+constexpr uint32_t flat_one_out_waves_per_cu(uint32_t nranks, uint64_t tiles_per_buffer, bool keep, uint32_t elem_size) {
+    if (!keep) return nranks >= 8 ? 8u : nranks == 4 ? 12u : 14u;
+    return nranks >= 8   ? (tiles_per_buffer < kFlatOneOutSmallTiles ? 14u : 9u)
+           : nranks == 4 ? (elem_size >= 4 ? 14u : 12u)
+                         : 0u;
 }
 // The tree kernel (reduce towards a root for rank counts the flat kernels do not have) walks its tree depth first with
 // a few loads in flight per wavefront, and likes 16 wavefronts per CU for elements of 4 and 8 bytes from 64 MiB per buffer
@@ -213,7 +243,7 @@ constexpr uint64_t kGroupCapMinBytes8 = uint64_t(256) << 20;  // per-rank buffer
 constexpr uint64_t kGroupCapMinBytes = uint64_t(128) << 20;   // ... and launches of two to four ranks
 constexpr uint32_t group_cap_per_cu(uint32_t nranks) { return nranks >= 8 ? 3u : nranks == 2 ? 5u : 4u; }  // workgroups per CU
 constexpr bool flat_one_out(uint32_t nranks, uint32_t nout, uint64_t total_tiles) {
-    return nout == 1 && nranks >= 3 && total_tiles >= kFlatOneOutMinTiles;
+    return nout == 1 && nranks >= 3 && total_tiles >= (nranks == 4 ? kFlatOneOutMinTilesFourRanks : kFlatOneOutMinTiles);
 }
 // One-wavefront launches below this many workgroups carry the thread-per-rank API's stream ordering
 // themselves (EdgeHooks).  Beyond it the release fence every workgroup then executes (it writes the L2 back)
