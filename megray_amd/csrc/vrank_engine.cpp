@@ -162,7 +162,7 @@ Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCal
                 break;
             case Step::kTree:
                 call = {tree_kernel_for(step.tree, dtype, op), step.tree.total_tiles, kThreads, &step.tree};
-                if (step.tree.vector && step.tree.elem_size >= 4 && step.tree.total_tiles >= kTreeCapMinTiles)
+                if (step.tree.vector && step.tree.elem_size >= 4 && step.tree.total_tiles >= tree_cap_min_tiles(step.tree.nranks))
                     call.lds = lds_for_waves_per_cu(call.kernel, kTreeCapWavesPerCu);
                 break;
             case Step::kPack:

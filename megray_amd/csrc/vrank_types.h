@@ -223,10 +223,17 @@ constexpr uint32_t flat_one_out_waves_per_cu(uint32_t nranks, uint64_t tiles_per
                          : 0u;
 }
 // The tree kernel (reduce towards a root for rank counts the flat kernels do not have) walks its tree depth first with
-// a few loads in flight per wavefront, and likes 16 wavefronts per CU for elements of 4 and 8 bytes from 64 MiB per buffer
-// on (fp32: 5 / 7 / 12 / 16 ranks 80 / 80 / 77 / 77 -> 86 / 87 / 81 / 81 % of the HBM peak, int64 and fp64 79 -> 84 - 85; at 32 MiB
-// level, below that behind); elements of 1 and 2 bytes spend longer on their conversions and lose 10 points to any cap.
-constexpr uint32_t kTreeCapMinTiles = 65536;
+// a few loads in flight per wavefront, and likes 16 wavefronts per CU for elements of 4 and 8 bytes once its launches are
+// long (fp32 at 256 MiB per buffer: 5 / 7 / 12 / 16 ranks 80 / 81 / 79 / 78 -> 85 / 87 / 84 / 82 % of the HBM peak, int64 and
+// fp64 79 -> 84 - 85).  How long depends on the number of ranks; all that fit against 16 per CU, fp32, by MiB per buffer:
+//   5 - 7 ranks   16 MiB 83 - 84 against 77 - 80   32 MiB 82 - 84 against 79 - 82   64 MiB 84 - 84.5 against 82 - 86   128 MiB 84 - 86 against 87 - 89
+//   9 - 11 ranks  16 MiB 81.9 - 82.7 against 81.1 - 83.5   32 MiB 80.8 - 81.3 against 82.9 - 83.5   64 MiB 81.7 - 83.4 against 85.7 - 86.5
+//   12 - 32 ranks  8 MiB 77.5 - 83.8 against 80.6 - 85.0   16 MiB 82.2 - 83.1 against 83.3 - 86.8   32 MiB 80.6 - 81.4 against 84.0 - 85.6
+// (14 and 18 per CU are behind 16 throughout).  Elements of 1 and 2 bytes spend longer on their conversions and lose 10
+// points to any cap.
+constexpr uint32_t tree_cap_min_tiles(uint32_t nranks) {  // tiles of 1 KiB per buffer
+    return nranks >= 12 ? 16384u : nranks >= 9 ? 32768u : 65536u;
+}
 constexpr uint32_t kTreeCapWavesPerCu = 16;
 // The group form of the flat fold behaves the same way once its launches are long: with all of a wavefront's accesses
 // issued at once (launches that do not pace them, kFlatPaced) fewer workgroups per CU than its LDS allows serve the
