@@ -238,13 +238,14 @@ def tree_expectation(ins, dtype, op, root):
 
 @pytest.mark.parametrize("dtype", [orc.FLOAT32, orc.FLOAT16, orc.INT8, orc.INT64])
 def test_large_folds_into_one_output_at_reduced_occupancy(dtype):
-    """reduce_scatter, reduce towards a root and the two-phase all_reduce from 8192 tiles per buffer on, tiles on
-    cache-line boundaries, three or more ranks: one wavefront per tile, launched with LDS reserved per workgroup so
-    that fewer wavefronts share a CU - eagerly, as a planned HIP graph (the reservation is part of the kernel
-    node) and with two ranks (which stay in the group form)."""
+    """reduce_scatter, reduce towards a root and the two-phase all_reduce from 8192 tiles per buffer on (four ranks:
+    from 65536 on), tiles on cache-line boundaries, three or more ranks: one wavefront per tile, launched with LDS
+    reserved per workgroup so that the number of wavefronts sharing a CU is the one that serves the shape best -
+    eagerly, as a planned HIP graph (the reservation is part of the kernel node), with four ranks on either side of
+    their threshold and with two ranks (which stay in the group form)."""
     size = orc.dtype_size(dtype)
     rng = np.random.default_rng(991 + dtype)
-    for nranks, tiles, waves in ((8, 8200, 1), (3, 8200, 1), (2, 8200, 4)):
+    for nranks, tiles, waves in ((8, 8200, 1), (3, 8200, 1), (2, 8200, 4), (4, 8200, 4), (4, 65600, 1)):
         recvlen = (tiles * 1024 // size + nranks - 1) // nranks // 128 * 128 + 128  # chunks on 128-byte boundaries
         length = recvlen * nranks
         ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
