@@ -282,6 +282,10 @@ def test_full_size_plan_shapes():
     assert moved and all(r["waves"] == 4 and r["deal"] == 1 for r in moved)
     pair, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, sp[:2], rp[:2], 1 << 24, orc.FLOAT32, nranks=2)
     assert pair and all(r["waves"] == 4 for r in pair)
+    # four ranks stay in the group form up to 65535 tiles per buffer
+    for recvlen, waves in ((1 << 21, 4), ((1 << 22) - 256, 4), (1 << 22, 1), (1 << 24, 1)):
+        four, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, sp[:4], rp[:4], recvlen, orc.FLOAT32, nranks=4)
+        assert four and all(r["waves"] == waves for r in four), recvlen
     for coll, count in ((mr.Collective.ALL_REDUCE, 1 << 15), (mr.Collective.REDUCE_SCATTER, 1 << 12),
                         (mr.Collective.REDUCE, 1 << 15)):
         small, _, _ = mr.describe(coll, sp, rp, count, orc.FLOAT32)
