@@ -234,7 +234,7 @@ private:
         // flat_one_out; the one output in nine streams may be shifted by a part of a line - a receive length that is no
         // multiple of 128 bytes: 82 - 84 % of the HBM peak against 79 - 80 in the group form - but with every buffer
         // off the lines the group form, which deals its workgroups to the XCDs, is 8 points ahead)
-        const bool one_wave = total < kFlatGroupMinTiles || (base_on_lines && flat_one_out(m_nranks, m_nout, total));
+        const bool one_wave = total < flat_group_min_tiles(m_nranks) || (base_on_lines && flat_one_out(m_nranks, m_nout, total));
         L.waves = one_wave ? 1 : kGroupWaves;
         L.exchange = (L.waves == kGroupWaves && !m_tree && m_nout == m_nranks && unshifted) ? 1 : 0;
         if (L.waves == kGroupWaves && !on_lines) L.exchange |= 2u;

@@ -142,10 +142,16 @@ struct FlatLaunch {
 };
 
 // Group form: a workgroup of kGroupWaves wavefronts owns kGroupWaves tiles that lie kGroupStride tiles
-// apart.  Short launches keep one wavefront per tile.  Measured crossovers on MI355X: the flat fold
-// from 2048 tiles per buffer (8 ranks, all_reduce fp32: 1 MiB per rank 3.95 us against 4.54 in the
-// group form, 2 MiB 5.3 against 5.75, 3.5 MiB 7.3 against 7.5, 4 MiB 11.1 against 8.5; reduce_scatter
-// and 2 or 4 ranks cross between 2 and 4 MiB as well), the segment and pack kernels from 512.
+// apart.  Short launches keep one wavefront per tile: as long as (nearly) every wavefront of the launch finds room on
+// the device at once, one tile per wavefront is the shorter way, and a fold of fewer inputs takes fewer registers and
+// less LDS, so more of its wavefronts fit.  Measured crossovers on MI355X, all_reduce, microseconds per launch, group
+// form / one wavefront per tile, by tiles per buffer (fp32; fp16 and int64 cross at the same points; reduce_scatter and
+// reduce cross at these points or later):
+//   8 ranks   2048 5.64 / 4.87   2560 6.62 / 6.86   3072 6.91 / 7.81   4096 8.33 / 11.71
+//   4 ranks   4096 5.14 / 4.68   6144 6.55 / 6.18   7168 8.44 / 9.79   8192 9.86 / 10.84
+//   3 ranks   8192 6.70 / 5.99   9216 7.47 / 6.87   10240 8.26 / 8.01   12288 10.73 / 12.35
+//   2 ranks   12288 6.75 / 6.26   14336 7.64 / 6.97   16384 9.70 / 10.54
+// The segment and pack kernels take the group form from 512 tiles on.
 constexpr uint32_t kGroupWaves = 4;
 constexpr uint32_t kGroupStride = 32;
 // A wavefront of the flat group kernel has this many loads in flight, and (where every rank is an output) this many
@@ -161,7 +167,9 @@ constexpr uint32_t kGroupStride = 32;
 constexpr uint32_t kGroupLoadsInFlight = 2;
 constexpr uint32_t kGroupStoresInFlight = 2;
 constexpr uint32_t kGroupMinTiles = 512;
-constexpr uint32_t kFlatGroupMinTiles = 2048;
+constexpr uint32_t flat_group_min_tiles(uint32_t nranks) {  // the flat fold's group form starts here
+    return nranks >= 8 ? 2560u : nranks == 4 ? 6400u : nranks == 3 ? 10752u : 15360u;
+}
 // Large flat folds with ONE output (reduce_scatter, reduce, the first launch of the two-phase all_reduce), three
 // or more inputs and input tiles on cache-line boundaries stay at one wavefront per tile and run at an occupancy of
 // their own: a wavefront has its K loads of 1 KiB in flight at once, and what HBM needs to stay busy (bandwidth x

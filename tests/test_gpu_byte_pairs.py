@@ -24,7 +24,7 @@ import megray_amd as mr  # noqa: E402
 from gpu_util import bits_equal, empty_device, first_mismatch, rand_array, to_device, to_host  # noqa: E402
 
 OPS = [orc.SUM, orc.MAX, orc.MIN]
-REPEATS = {"short": 1, "long": 40}  # 64 tiles / 2560 tiles of 1 KiB: below and above the group forms' thresholds
+REPEATS = {"short": 1, "long": 240}  # 64 tiles / 15360 tiles of 1 KiB: below and above the group forms' thresholds (two ranks': 15360)
 
 
 def all_pairs(dtype, repeats):

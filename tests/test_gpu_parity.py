@@ -87,12 +87,13 @@ def test_more_than_sixteen_ranks(nranks):
 
 @pytest.mark.parametrize("dtype", REDUCE_TYPES)
 def test_all_reduce_group_form(dtype):
-    """Launches of 2048 tiles and more take the group form of the flat kernel (four wavefronts per
-    workgroup, four tiles 32 tiles apart): ragged lengths, so that chunk borders fall inside tiles and the
-    last group of tiles is incomplete; out of place and in place."""
+    """Long launches take the group form of the flat kernel (four wavefronts per workgroup, four tiles 32 tiles
+    apart; the fewer the ranks, the later: from 15360 / 10752 / 6400 / 2560 tiles per buffer for 2 / 3 / 4 / 8 ranks):
+    ragged lengths, so that chunk borders fall inside tiles and the last group of tiles is incomplete; out of place
+    and in place."""
     size = orc.dtype_size(dtype)
     rng = np.random.default_rng(77 + dtype)
-    for nranks, tiles in ((2, 4096), (3, 4500), (4, 4301), (8, 5051)):
+    for nranks, tiles in ((2, 15400), (3, 10800), (4, 6401), (8, 5051)):
         length = (tiles * 1024 + 1024 - 16 * (nranks - 1)) // size - 3
         ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
         d_in = [to_device(x) for x in ins]
@@ -117,7 +118,7 @@ def test_all_reduce_group_form_with_paced_accesses(dtype, monkeypatch):
     monkeypatch.setenv("MEGRAY_VRANK_PACE", "always")
     size = orc.dtype_size(dtype)
     rng = np.random.default_rng(1077 + dtype)
-    for nranks, tiles in ((3, 4500), (4, 4301), (8, 5051)):
+    for nranks, tiles in ((3, 10800), (4, 6401), (8, 5051)):
         length = (tiles * 1024 + 1024 - 16 * (nranks - 1)) // size - 3
         ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
         for op, order in ((orc.SUM, orc.ORDER_UCX), (orc.MAX, orc.ORDER_SHM), (orc.MIN, orc.ORDER_RANK0)):
@@ -245,7 +246,7 @@ def test_large_folds_into_one_output_at_reduced_occupancy(dtype):
     their threshold and with two ranks (which stay in the group form)."""
     size = orc.dtype_size(dtype)
     rng = np.random.default_rng(991 + dtype)
-    for nranks, tiles, waves in ((8, 8200, 1), (3, 8200, 1), (2, 8200, 4), (4, 8200, 4), (4, 65600, 1)):
+    for nranks, tiles, waves in ((8, 8200, 1), (3, 8200, 1), (2, 15400, 4), (4, 8200, 4), (4, 65600, 1)):
         recvlen = (tiles * 1024 // size + nranks - 1) // nranks // 128 * 128 + 128  # chunks on 128-byte boundaries
         length = recvlen * nranks
         ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
@@ -290,7 +291,7 @@ def test_group_form_with_one_output(dtype):
     group form in which every wavefront stores the tile it folded (shifted outputs, one destination)."""
     size = orc.dtype_size(dtype)
     rng = np.random.default_rng(177 + dtype)
-    for nranks, tiles in ((3, 4200), (8, 4999)):
+    for nranks, tiles in ((4, 6500), (8, 4999)):
         recvlen = (tiles * 1024 // size) // nranks // 16 * 16 + 16  # keeps chunk r of rank r on a 16-byte boundary
         length = recvlen * nranks
         ins = [rand_array(dtype, length, rng) for _ in range(nranks)]

@@ -61,14 +61,15 @@ def test_lengths_around_vector_and_tile_borders(dtype, nranks):
 
 @pytest.mark.parametrize("dtype", [orc.UINT8, orc.FLOAT32])
 def test_the_group_form_at_the_buffers_end(dtype):
-    """2048 tiles and more: four wavefronts per workgroup; the wavefront that holds the buffers' last tile loads it
-    lane by lane, and tiles across chunk borders come out of the group's LDS."""
+    """Long launches (10752 tiles and more for three ranks, 2560 for eight): four wavefronts per workgroup; the
+    wavefront that holds the buffers' last tile loads it lane by lane, and tiles across chunk borders come out of the
+    group's LDS."""
     size = orc.dtype_size(dtype)
     rng = np.random.default_rng(8900 + dtype)
     per_vector, per_tile = 16 // size, 1024 // size
     for nranks in (3, 8):
         for extra in (1, per_vector - 1, per_vector + 1, per_tile - 1, 5 * per_vector + 3):
-            length = 2100 * per_tile + extra
+            length = {3: 10800, 8: 2600}[nranks] * per_tile + extra
             ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
             d_in = [to_device(x) for x in ins]
             runs, _, _ = mr.describe(mr.Collective.ALL_REDUCE, d_in, d_in, length, dtype)

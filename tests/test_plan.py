@@ -262,7 +262,7 @@ def test_full_size_plan_shapes():
     assert sum(r["count"] for r in runs) == n
     assert br == bw == 8 * n * 4
     assert all(r["waves"] == 4 for r in runs)  # the group form: four wavefronts, four tiles per workgroup
-    # so do reduce_scatter and tree launches of 2048 to 8191 tiles per buffer; short launches keep one wavefront per tile
+    # so do reduce_scatter and tree launches of 2560 to 8191 tiles per buffer; short launches keep one wavefront per tile
     rs, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, sp, rp, 1 << 17, orc.FLOAT32)
     assert rs and all(r["waves"] == 4 and r["vector"] == 2 for r in rs)
     tree, _, _ = mr.describe(mr.Collective.REDUCE, sp, rp, 1 << 20, orc.FLOAT32, root=3)
@@ -282,6 +282,11 @@ def test_full_size_plan_shapes():
     assert moved and all(r["waves"] == 4 and r["deal"] == 1 for r in moved)
     pair, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, sp[:2], rp[:2], 1 << 24, orc.FLOAT32, nranks=2)
     assert pair and all(r["waves"] == 4 for r in pair)
+    # the group form starts the later the fewer the ranks (a tile is 256 fp32 elements)
+    for ranks, first in ((8, 2560), (4, 6400), (3, 10752), (2, 15360)):
+        for tiles, waves in ((first - 1, 1), (first, 4)):
+            ar, _, _ = mr.describe(mr.Collective.ALL_REDUCE, sp[:ranks], rp[:ranks], tiles * 256, orc.FLOAT32, nranks=ranks)
+            assert ar and all(r["waves"] == waves for r in ar), (ranks, tiles)
     # four ranks stay in the group form up to 65535 tiles per buffer
     for recvlen, waves in ((1 << 21, 4), ((1 << 22) - 256, 4), (1 << 22, 1), (1 << 24, 1)):
         four, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, sp[:4], rp[:4], recvlen, orc.FLOAT32, nranks=4)
