@@ -257,11 +257,20 @@ private:
         uint64_t vector_elems = 0;
         for (const Run& r : m_runs)
             if (natural || same_phase(r)) vector_elems += r.count;
-        m_waves = vector_elems / (kThreads * epv) >= kGroupMinTiles ? kGroupWaves : 1;
-        m_paced = m_waves == kGroupWaves && m_nfold >= 3 && paced_launch(m_in, m_out, m_nranks, vector_elems * m_elem, false, m_nout);
         uint64_t all_elems = 0;
         for (const Run& r : m_runs) all_elems += r.count;
-        m_short = m_waves == 1 && all_elems * m_elem <= kShortTilesMaxBytes;  // short launches: small tiles, more wavefronts
+        // short launches keep one wavefront per tile, and small tiles; folds that are vectors throughout keep them
+        // longer (kShortVectorMaxBytes)
+        const uint64_t vector_tiles = vector_elems / (kThreads * epv);
+        if (vector_elems == all_elems && m_nfold >= 2) {
+            const uint64_t one_out_max = m_elem == 1 ? kShortVectorMaxBytesOneOut / 2 : kShortVectorMaxBytesOneOut;
+            m_short = all_elems * m_elem <= (m_nout == 1 ? one_out_max : kShortVectorMaxBytes);
+            m_waves = !m_short && vector_tiles >= kGroupMinTiles ? kGroupWaves : 1;
+        } else {
+            m_waves = vector_tiles >= kGroupMinTiles ? kGroupWaves : 1;
+            m_short = m_waves == 1 && all_elems * m_elem <= kShortTilesMaxBytes;
+        }
+        m_paced = m_waves == kGroupWaves && m_nfold >= 3 && paced_launch(m_in, m_out, m_nranks, vector_elems * m_elem, false, m_nout);
         open_launch();
         for (const Run& r : m_runs) {
             const bool vector = natural || same_phase(r);
@@ -730,8 +739,25 @@ Status add_pack(Plan& plan, const void* const* in, void* const* out, uint32_t nr
     // uint8, microseconds per all_to_all, group form -> one wavefront per tile, blocks of 128 KiB / 512 KiB / 2 MiB / 4 MiB:
     //   16 ranks 18.3 -> 12.3 / 45.5 -> 40.4 / 160 -> 159 / 314 -> 318;  8 ranks 6.2 -> 4.6 / 13.2 -> 12.1 / 41.1 -> 39.7 / 80.5 -> 81.0;
     //   5 ranks 4.4 -> 3.8 / 6.3 -> 6.1 / 17.8 -> 17.1 / 31.9 -> 31.4;  4 ranks 3.3 -> 3.4 / 4.9 -> 4.6 / 12.0 -> 12.1 / 21.4 -> 21.5 (left alone).
-    // all_gather and broadcast need the group form from 128 tiles on (8 ranks x 128 KiB: 4.7 against 5.4 us; 16 MiB: 181 against 234).
-    const uint64_t group_min = mode == kPackAllToAll && nranks >= 5 ? 4096 : kGroupMinTiles / 4;
+    // A broadcast is one copy with N destinations, and an all_gather N of them: as long as the launch is short, one
+    // wavefront per tile is the shorter way for them as well.  Group form / one wavefront per tile, microseconds, device
+    // in its steady state, by KiB per block:
+    //   broadcast   4 ranks  128 3.10 / 2.78   512 3.10 / 2.81   1024 3.16 / 2.98   2048 3.45 / 3.42   4096 4.49 / 4.64
+    //               8 ranks  128 3.74 / 3.05   512 3.74 / 3.07   1024 3.79 / 3.41   2048 4.35 / 4.40   4096 6.60 / 6.82
+    //              16 ranks  128 5.56 / 4.71   512 5.69 / 4.71   1024 5.77 / 5.05   2048 6.39 / 6.69   4096 10.8 / 10.5
+    //   all_gather  2 ranks  512 2.92 / 2.79   4096 5.22 / 4.84   8192 7.58 / 6.73   16384 15.5 / 16.4
+    //               4 ranks  128 3.10 / 2.88   1024 4.76 / 4.56   4096 10.7 / 10.4   8192 24.5 / 29.5
+    //               6 ranks  128 3.63 / 3.06   1024 7.26 / 6.71   3072 16.3 / 15.4   4096 24.6 / 26.3
+    //               8 ranks  128 4.01 / 4.19   192 4.02 / 3.93   1024 11.6 / 10.1   2048 18.8 / 17.7   3072 34.3 / 35.2   4096 45.0 / 51.5
+    //              12 ranks  128 5.69 / 6.59   256 8.07 / 6.81   512 12.0 / 10.9   1024 25.0 / 27.0   (16 ranks alike: left alone)
+    // (blocks on 4-byte boundaries only cross earlier: fp32, 4 ranks x 5 MiB + 4 B 12.7 / 15.5, 3 ranks x 10 MiB + 4 B 17.9 / 21.9;
+    // 9 and 11 ranks x 2 MiB 28.2 / 30.1 and 40.9 / 44.1, x 1 MiB 13.9 / 12.3 and 18.4 / 16.9.)
+    // scatter, gather and send / recv keep the group form from 128 tiles on.
+    uint64_t group_min = kGroupMinTiles / 4;
+    if (mode == kPackAllToAll && nranks >= 5) group_min = 4096;
+    if (mode == kPackBroadcast) group_min = 2048;
+    if (mode == kPackAllGather && nranks < 12)
+        group_min = nranks <= 3 ? 8192 : nranks == 4 ? 4096 : nranks <= 7 ? 3072 : nranks == 8 ? 2048 : 1280;
     L.waves = tiles >= group_min ? kGroupWaves : 1;
     if (L.waves == kGroupWaves && mode == kPackAllGather) L.paced = paced_gather(nranks, block_bytes) ? 1 : 0;
     if (L.waves == kGroupWaves && mode == kPackBroadcast) L.paced = paced_broadcast(nranks, block_bytes) ? 1 : 0;

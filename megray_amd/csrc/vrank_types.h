@@ -344,8 +344,26 @@ constexpr uint32_t kVecIters = 4;
 // of that per workgroup: a wavefront goes through its groups one after the other, one memory round trip each, and
 // when every wavefront of the launch fits the device at once anyway, four times the wavefronts finish in a quarter of
 // the time (5 ranks x 256 KiB fp32 all_reduce: 10.9 -> 5 us).
+// Launches whose buffers are all vectors keep that form well beyond the point where the device is full, because the
+// group form (which begins where it ends) only pays on long launches.  Measured on MI355X, microseconds per launch,
+// group form / one wavefront per group of vectors, fp32 (fp16 alike), by KiB per buffer:
+//   all_reduce      5 ranks  1024 6.29 / 5.68   2048 6.97 / 6.37   3072 8.43 / 7.38   4096 8.90 / 9.31    8192 15.6 / 16.4
+//                   7 ranks  1024 7.01 / 6.42   2048 8.61 / 7.90   3072 10.2 / 8.91   4096 11.4 / 12.3    8192 21.0 / 21.4
+//                  12 ranks  1024 9.40 / 8.21   2048 12.9 / 10.1   3072 13.8 / 14.5   4096 19.3 / 22.1    8192 35.5 / 34.8
+//                  16 ranks  1024 8.20 / 7.79   2048 11.9 / 11.5   3072 21.1 / 18.8   4096 22.5 / 25.4    8192 43.1 / 44.8
+//   reduce_scatter  5 ranks  1024 5.62 / 5.01   2048 5.80 / 5.20   4096 6.63 / 6.13   8192 10.1 / 9.48   16384 16.9 / 17.3
+//                   7 ranks  1024 5.83 / 5.32   2048 6.03 / 5.67   4096 7.10 / 7.37   8192 13.2 / 12.5   16384 21.0 / 22.2
+//                  12 ranks  1024 7.43 / 6.41   2048 7.71 / 8.35   4096 10.8 / 10.6   8192 22.4 / 20.1   16384 35.2 / 37.3
+//                  16 ranks  1024 7.40 / 7.16   2048 8.06 / 7.56   4096 12.5 / 12.6   8192 23.5 / 22.4   16384 43.8 / 44.8
+// (with the usual four groups per wavefront the one-wavefront form takes 9 - 25 us at 2048 KiB); from 16 MiB to 256 MiB
+// the group form is 2 - 20 % ahead.  Hence: up to 3 MiB per buffer, and up to 8 MiB where every element has one
+// destination (4 MiB for elements of one byte: int8 reduce_scatter of 5 ranks, odd receive length, 6 MiB 9.2 / 10.5).
+// Buffers off the vector grid gain most: fp16 all_reduce of 8 ranks x 1.5 MiB at 48 bytes off 12.2 / 8.8, int8 10.1 / 6.1.  Launches with element tiles (buffers at differing offsets from a 4-byte boundary) keep the 1 MiB limit
+// and take the group form for their vector bodies from kGroupMinTiles on.
 constexpr uint32_t kShortElemsPerLane = 4;
 constexpr uint64_t kShortTilesMaxBytes = uint64_t(1) << 20;
+constexpr uint64_t kShortVectorMaxBytes = uint64_t(3) << 20;
+constexpr uint64_t kShortVectorMaxBytesOneOut = uint64_t(8) << 20;
 constexpr uint32_t vec_iters(const FoldLaunch& L) { return L.short_tiles ? 1u : kVecIters; }
 constexpr uint32_t elems_per_lane(const FoldLaunch& L) { return L.short_tiles ? kShortElemsPerLane : kElemsPerLane; }
 

@@ -117,16 +117,18 @@ def test_the_vector_forms_are_what_runs():
     nranks, length = 8, 33001 * 4 + 1
     send = [(1 << 40) + (r << 32) for r in range(nranks)]
     recv = [(2 << 40) + (r << 34) for r in range(nranks)]
-    runs, _, _ = mr.describe(mr.Collective.ALL_GATHER, send, recv, length, orc.FLOAT32)
-    assert runs and all(r["vector"] == 4 and r["waves"] == 4 for r in runs)
+    for elems, waves in ((length, 1), (4 * length + 1, 4)):  # an all_gather of eight ranks takes the group form from 2 MiB per block
+        runs, _, _ = mr.describe(mr.Collective.ALL_GATHER, send, recv, elems, orc.FLOAT32)
+        assert runs and all(r["vector"] == 4 and r["waves"] == waves for r in runs), elems
     # an all_to_all of five ranks and more keeps one wavefront per tile up to 4 MiB per block (its launch is long either way)
     for ranks, elems, waves in ((8, length, 1), (4, length, 4), (8, (1 << 20) + 1, 4)):
         runs, _, _ = mr.describe(mr.Collective.ALL_TO_ALL, send[:ranks], recv[:ranks], elems, orc.FLOAT32)
         assert runs and all(r["vector"] == 4 and r["waves"] == waves for r in runs), (ranks, elems)
-    runs, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, send, recv, length, orc.FLOAT32)
-    body = sum(r["count"] for r in runs if r["vector"] == 1)
-    assert body >= nranks * length - nranks * 3 * 300  # all but heads and tails of at most a tile's worth per run
-    assert all(r["waves"] == 4 for r in runs)
+    for length, waves in ((33001 * 4 + 1, 1), (300001, 4)):  # folds into one output take the group form beyond 8 MiB per buffer
+        runs, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, send, recv, length, orc.FLOAT32)
+        body = sum(r["count"] for r in runs if r["vector"] == 1)
+        assert body >= nranks * length - nranks * 3 * 300  # all but heads and tails of at most a tile's worth per run
+        assert all(r["waves"] == waves for r in runs), length
 
 
 @pytest.mark.parametrize("dtype", [orc.FLOAT32, orc.INT32, orc.FLOAT64, orc.INT64, orc.FLOAT16, orc.INT8, orc.UINT8])

@@ -176,6 +176,39 @@ def test_either_store_policy_gives_the_same_results(keep, monkeypatch):
         check_pack_collectives(orc.UINT8, 8, length, 0, rng)
 
 
+@pytest.mark.parametrize("dtype", [orc.INT8, orc.FLOAT16, orc.FLOAT32, orc.INT64])
+def test_general_folds_of_a_few_mib_keep_one_wavefront_per_group_of_vectors(dtype):
+    """Folds through the general kernel whose buffers are vectors throughout keep one wavefront per group of 64
+    vectors up to 3 MiB per buffer (8 MiB where every element has one destination; 4 MiB for one-byte elements):
+    rank counts without a flat kernel, and eight ranks at a common offset from a 16-byte boundary."""
+    size = orc.dtype_size(dtype)
+    rng = np.random.default_rng(377 + dtype)
+    for nranks, offset, kib in ((5, 0, 2900), (7, 0, 1500), (8, max(size, 4), 2100)):
+        length = kib * 1024 // size + 5
+        ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+        d_in = [to_device(x, offset) for x in ins]
+        d_out = [empty_device(length * size, offset) for _ in range(nranks)]
+        runs, _, _ = mr.describe(mr.Collective.ALL_REDUCE, d_in, d_out, length, dtype)
+        assert runs and all(r["waves"] == 1 for r in runs), "not the form this test is about"
+        for op, order in ((orc.SUM, orc.ORDER_UCX), (orc.MIN, orc.ORDER_SHM)):
+            want = orc.fold_all_reduce(ins, dtype, op, order)
+            got = run_all_reduce(ins, dtype, op, order, mr.Schedule.FUSED, offsets=[offset] * nranks)
+            for r in range(nranks):
+                assert_same(got[r], want[r], f"all_reduce dtype={dtype} N={nranks} offset={offset} op={op} rank={r}")
+    for nranks, kib in ((6, 3900 if size == 1 else 7900), (12, 3000)):
+        recvlen = kib * 1024 // size // nranks // 16 * 16 + 16
+        ins = [rand_array(dtype, recvlen * nranks, rng) for _ in range(nranks)]
+        d_in = [to_device(x) for x in ins]
+        parts = [empty_device(recvlen * size) for _ in range(nranks)]
+        runs, _, _ = mr.describe(mr.Collective.REDUCE_SCATTER, d_in, parts, recvlen, dtype)
+        assert runs and all(r["waves"] == 1 for r in runs), "not the form this test is about"
+        want = orc.fold_reduce_scatter(ins, dtype, orc.SUM, orc.ORDER_UCX)
+        mr.reduce_scatter(d_in, parts, recvlen, dtype, orc.SUM, orc.ORDER_UCX)
+        torch.cuda.synchronize()
+        for r in range(nranks):
+            assert_same(to_host(parts[r], ins[0].dtype), want[r], f"reduce_scatter dtype={dtype} N={nranks} rank={r}")
+
+
 @pytest.mark.parametrize("dtype", REDUCE_TYPES)
 def test_segment_group_form(dtype):
     """The general fold kernel with long vector bodies (512 groups of 64 vectors and more) runs in its
@@ -457,15 +490,23 @@ def test_pack_collectives(dtype):
 
 @pytest.mark.parametrize("dtype", [orc.UINT8, orc.FLOAT16, orc.INT64])
 def test_pack_collectives_group_form(dtype):
-    """Blocks of 128 tiles and more go through the group form of the pack kernel (four wavefronts, four
-    tiles per workgroup); the block ends in a partial tile."""
+    """Long blocks go through the group form of the pack kernel (four wavefronts, four tiles per workgroup; an
+    all_gather of three ranks from 8192 tiles per block on, of eight from 2048, a broadcast from 2048, the others from
+    128); the block ends in a partial tile."""
     rng = np.random.default_rng(190 + dtype)
     size = orc.dtype_size(dtype)
-    length = (1030 * 1024 + 48) // size
-    for nranks in (3, 8):
+    for nranks, tiles in ((3, 8200), (8, 2060)):
+        length = (tiles * 1024 + 48) // size
         runs, _, _ = mr.describe(mr.Collective.ALL_GATHER, [(1 << 40) + (r << 30) for r in range(nranks)],
                                  [(2 << 40) + (r << 34) for r in range(nranks)], length, dtype)
         assert runs and all(r["waves"] == 4 and r["vector"] == 16 for r in runs), "the group form is not what runs here"
+        check_pack_collectives(dtype, nranks, length, 0, rng)
+    # just below those sizes an all_gather and a broadcast keep one wavefront per tile, the others are in the group form
+    for nranks, tiles in ((3, 8100), (8, 2000)):
+        length = (tiles * 1024 + 48) // size
+        runs, _, _ = mr.describe(mr.Collective.ALL_GATHER, [(1 << 40) + (r << 30) for r in range(nranks)],
+                                 [(2 << 40) + (r << 34) for r in range(nranks)], length, dtype)
+        assert runs and all(r["waves"] == 1 and r["vector"] == 16 for r in runs), "one wavefront per tile is not what runs here"
         check_pack_collectives(dtype, nranks, length, 0, rng)
 
 
@@ -477,9 +518,8 @@ def test_pack_collectives_group_form_with_paced_stores(pace, monkeypatch):
     monkeypatch.setenv("MEGRAY_VRANK_PACE", pace)
     rng = np.random.default_rng(290)
     for dtype in (orc.UINT8, orc.FLOAT32):
-        length = (1030 * 1024 + 48) // orc.dtype_size(dtype)
-        for nranks in (3, 8):
-            check_pack_collectives(dtype, nranks, length, 0, rng)
+        for nranks, tiles in ((3, 8200), (8, 2060)):  # long enough for the group form of every pack collective
+            check_pack_collectives(dtype, nranks, (tiles * 1024 + 48) // orc.dtype_size(dtype), 0, rng)
 
 
 def test_many_rank_gathers_and_broadcasts_pace_their_stores_by_themselves():

@@ -99,7 +99,8 @@ def test_ten_mib_row_agrees_with_an_event_timing(tmp_path):
     assert record["bufsize"] == nbytes and record["streams"] == "shared"
     assert record["avg_us"] == pytest.approx(avg_us, rel=1e-3)
     print(f"performance tool, one stream: {hbm:.0f} GB/s, event timing {event_gbps:.0f} GB/s")
-    assert hbm == pytest.approx(event_gbps, rel=0.10)
+    # 160 MiB in all: the buffers fit the last-level cache, and how well depends on where each process's allocations lie
+    assert hbm == pytest.approx(event_gbps, rel=0.15)
     # every rank on a stream of its own (the reference's harness): each collective waits for all streams and
     # all streams wait for it, a chain of dependent launches that adds a few microseconds per call
     out = run_cli("-d", str(nranks), "-f", "all_reduce", "-s", str(nbytes), "-w", "100", "-i", "500")
