@@ -37,7 +37,7 @@ def check_guards(what):
 
 
 def draw_length(rng, nranks):
-    bytes_ = int(np.exp(rng.uniform(np.log(1), np.log(6e6))))
+    bytes_ = int(np.exp(rng.uniform(np.log(1), np.log(2e7))))
     return max(0, bytes_ + int(rng.integers(-3, 4)))
 
 
