@@ -334,11 +334,78 @@ __device__ __forceinline__ SegmentView find_segment(const FoldLaunch& L, uint32_
     return sv;
 }
 
+// Where a kernel finds its rank pointers.  ArgPtrs reads them from the launch descriptor as they are needed: a
+// scalar load per pointer whose index is known only after the segment lookup, one more memory round trip before
+// the first data load.  LanePtrs holds the tables in a register instead - lane l the descriptor's in[l], lane
+// kMaxRanks + l its out[l], read by the whole wavefront at once when the kernel starts - and picks by readlane.
+struct ArgPtrs {
+    const FoldLaunch& L;
+    __device__ __forceinline__ const char* in(uint32_t r) const { return static_cast<const char*>(L.in[r]); }
+    __device__ __forceinline__ char* out(uint32_t r) const { return static_cast<char*>(L.out[r]); }
+};
+struct LanePtrs {
+    uint32_t lo, hi;
+    __device__ __forceinline__ char* pick(uint32_t lane) const {
+        const uint64_t a = uint64_t(uint32_t(__builtin_amdgcn_readlane(int(lo), int(lane)))) |
+                           uint64_t(uint32_t(__builtin_amdgcn_readlane(int(hi), int(lane)))) << 32;
+        return reinterpret_cast<char*>(a);
+    }
+    __device__ __forceinline__ const char* in(uint32_t r) const { return pick(r); }
+    __device__ __forceinline__ char* out(uint32_t r) const { return pick(kMaxRanks + r); }
+};
+static_assert(2 * kMaxRanks == kThreads, "one lane per entry of in[] and out[]");
+static_assert(offsetof(FoldLaunch, out) == offsetof(FoldLaunch, in) + kMaxRanks * sizeof(void*), "out[] follows in[]");
+static_assert(sizeof(FoldSegment) == 32 && kMaxSegments >= kThreads, "a lane reads one segment, two vectors");
+
+// What a one-wavefront kernel reads of its launch descriptor before anything else, every lane its share, all four
+// loads in flight together: lane l holds first_tile[l], seg[l] and one rank pointer.  The segment lookup is then a
+// ballot and a handful of readlanes, and the rank pointers are at hand: one memory round trip between the kernel's
+// start and its first data load, where the scalar lookup (find_segment, then seg[s], then in[r]) takes three.
+struct LaneArgs {
+    uint32_t first_tile;
+    u32x4 seg_a, seg_b;
+    LanePtrs ptrs;
+};
+__device__ __forceinline__ LaneArgs load_lane_args(uint32_t lane) {
+    using Constant = const __attribute__((address_space(4))) char;
+    Constant* base = (Constant*)__builtin_amdgcn_kernarg_segment_ptr();  // the descriptor is the only argument
+    LaneArgs a;
+    a.first_tile = *reinterpret_cast<const __attribute__((address_space(4))) uint32_t*>(
+            base + offsetof(FoldLaunch, first_tile) + lane * sizeof(uint32_t));
+    const auto* seg = reinterpret_cast<const __attribute__((address_space(4))) u32x4*>(
+            base + offsetof(FoldLaunch, seg) + lane * sizeof(FoldSegment));
+    a.seg_a = seg[0];
+    a.seg_b = seg[1];
+    const auto* ptr = reinterpret_cast<const __attribute__((address_space(4))) uint32_t*>(
+            base + offsetof(FoldLaunch, in) + lane * sizeof(void*));
+    a.ptrs.lo = ptr[0];
+    a.ptrs.hi = ptr[1];
+    return a;
+}
+// (launches of more than kThreads segments - 22 and more ranks off the vector grid - look the segment up the scalar way)
+__device__ __forceinline__ SegmentView find_segment(const FoldLaunch& L, const LaneArgs& a, uint32_t tile) {
+    if (L.nseg > kThreads) return find_segment(L, tile);
+    const uint32_t s = uint32_t(__popcll(__ballot(a.first_tile <= tile))) - 1u;
+    const auto pick = [&](uint32_t v) { return uint32_t(__builtin_amdgcn_readlane(int(v), int(s))); };
+    SegmentView sv;
+    sv.in_begin = uint64_t(pick(a.seg_a.x)) | uint64_t(pick(a.seg_a.y)) << 32;
+    sv.out_begin = uint64_t(pick(a.seg_a.z)) | uint64_t(pick(a.seg_a.w)) << 32;
+    sv.count = uint64_t(pick(a.seg_b.x)) | uint64_t(pick(a.seg_b.y)) << 32;
+    sv.local_tile = tile - pick(a.first_tile);
+    const uint32_t bytes = pick(a.seg_b.w);  // start, dir, out_first, flags
+    sv.start = bytes & 0xffu;
+    sv.dir = int(int8_t((bytes >> 8) & 0xffu));
+    sv.out_first = (bytes >> 16) & 0xffu;
+    sv.vector = ((bytes >> 24) & kSegVector) != 0;
+    sv.deal = ((bytes >> 24) & kSegDeal) != 0;
+    return sv;
+}
+
 // Element tiles: run heads / tails and buffers that are not 16-byte aligned.  A lane takes
 // elems_per_lane(L) elements, a wavefront's lanes consecutive ones, four at a time; the loads of up to eight ranks
 // are in flight together (one memory round trip for up to nine inputs, not one per input).
-template <typename T, int OP>
-__device__ __forceinline__ void fold_element_tile(const FoldLaunch& L, const SegmentView& sv, uint32_t nfold,
+template <typename T, int OP, typename P>
+__device__ __forceinline__ void fold_element_tile(const FoldLaunch& L, const P& ptrs, const SegmentView& sv, uint32_t nfold,
                                                   uint32_t local_tile, uint32_t tid) {
     using A = typename Wide<T>::type;
     constexpr uint32_t G = 4, B = 8;
@@ -358,7 +425,7 @@ __device__ __forceinline__ void fold_element_tile(const FoldLaunch& L, const Seg
 #pragma unroll
         for (uint32_t q = 0; q < G; ++q) have[q] = uint64_t(q) * kThreads + tid < left;
         A a[G];
-        const T* seed = static_cast<const T*>(L.in[start]) + ie;
+        const T* seed = reinterpret_cast<const T*>(ptrs.in(start)) + ie;
 #pragma unroll
         for (uint32_t q = 0; q < G; ++q) a[q] = have[q] ? static_cast<A>(seed[q * kThreads]) : A(0);
         for (uint32_t j0 = 1; j0 < nfold; j0 += B) {
@@ -366,7 +433,7 @@ __device__ __forceinline__ void fold_element_tile(const FoldLaunch& L, const Seg
 #pragma unroll
             for (uint32_t b = 0; b < B; ++b) {
                 if (j0 + b < nfold) {
-                    const T* src = static_cast<const T*>(L.in[rotate_rank(start, dir, j0 + b, nr)]) + ie;
+                    const T* src = reinterpret_cast<const T*>(ptrs.in(rotate_rank(start, dir, j0 + b, nr))) + ie;
 #pragma unroll
                     for (uint32_t q = 0; q < G; ++q) x[b][q] = have[q] ? src[q * kThreads] : T(0);
                 }
@@ -380,7 +447,7 @@ __device__ __forceinline__ void fold_element_tile(const FoldLaunch& L, const Seg
             }
         }
         for (uint32_t m = 0; m < nout; ++m) {
-            T* dst = static_cast<T*>(L.out[rotate_rank(out_first, 1, m, nr)]) + oe;
+            T* dst = reinterpret_cast<T*>(ptrs.out(rotate_rank(out_first, 1, m, nr))) + oe;
 #pragma unroll
             for (uint32_t q = 0; q < G; ++q)
                 if (have[q]) dst[q * kThreads] = static_cast<T>(a[q]);
@@ -390,8 +457,8 @@ __device__ __forceinline__ void fold_element_tile(const FoldLaunch& L, const Seg
 
 // Up to kThreads vectors at vector index `vbase` of a segment, each lane folding one vector by itself
 // with plain global accesses: the incomplete last group of a segment's vector body.
-template <typename T, int OP>
-__device__ __forceinline__ void fold_vector_remainder(const FoldLaunch& L, const SegmentView& sv, uint32_t nfold,
+template <typename T, int OP, typename P>
+__device__ __forceinline__ void fold_vector_remainder(const FoldLaunch& L, const P& ptrs, const SegmentView& sv, uint32_t nfold,
                                                       uint64_t vbase, uint64_t left, uint32_t tid) {
     if (tid >= left) return;
     const uint32_t nr = L.nranks;
@@ -399,19 +466,19 @@ __device__ __forceinline__ void fold_vector_remainder(const FoldLaunch& L, const
     const uint64_t in_off = sv.in_begin * sizeof(T) + (vbase + tid) * kVecBytes;
     const uint64_t out_off = sv.out_begin * sizeof(T) + (vbase + tid) * kVecBytes;
     AccFor<T, OP> a;
-    a.seed(load_vec(static_cast<const char*>(L.in[sv.start]) + in_off));
+    a.seed(load_vec(ptrs.in(sv.start) + in_off));
     for (uint32_t j0 = 1; j0 < nfold; j0 += 8) {  // the loads of up to eight ranks in flight together
         u32x4 x[8];
 #pragma unroll
         for (uint32_t b = 0; b < 8; ++b)
-            if (j0 + b < nfold) x[b] = load_vec(static_cast<const char*>(L.in[rotate_rank(sv.start, sv.dir, j0 + b, nr)]) + in_off);
+            if (j0 + b < nfold) x[b] = load_vec(ptrs.in(rotate_rank(sv.start, sv.dir, j0 + b, nr)) + in_off);
 #pragma unroll
         for (uint32_t b = 0; b < 8; ++b)
             if (j0 + b < nfold) a.fold(x[b], new_wins);
     }
     const u32x4 r = a.finish();
     for (uint32_t m = 0; m < L.nout; ++m)
-        store_vec(static_cast<char*>(L.out[rotate_rank(sv.out_first, 1, m, nr)]) + out_off, r);
+        store_vec(ptrs.out(rotate_rank(sv.out_first, 1, m, nr)) + out_off, r);
 }
 
 // Every lane polls the same word (one request per wavefront) until it reaches `target` or the time
@@ -468,9 +535,10 @@ __device__ __forceinline__ void hook_publish(const EdgeHooks& h, uint64_t ticket
 // K > 0: fold count known at compile time, all K loads of a lane are issued before the first use.
 // K == 0: fold count read from the launch, loads issued in groups of four.
 template <typename T, int OP, int K>
-__device__ __forceinline__ void fold_tile(const FoldLaunch& L) {
+__device__ __forceinline__ void fold_tile(const FoldLaunch& L, const LaneArgs& args) {
     constexpr uint32_t EPV = kVecBytes / sizeof(T);
-    const SegmentView sv = find_segment(L, blockIdx.x);
+    const SegmentView sv = find_segment(L, args, blockIdx.x);
+    const LanePtrs& ptrs = args.ptrs;
     const uint32_t local_tile = sv.local_tile, start = sv.start, out_first = sv.out_first;
     const int dir = sv.dir;
     const uint32_t nr = L.nranks;
@@ -489,7 +557,7 @@ __device__ __forceinline__ void fold_tile(const FoldLaunch& L) {
             if (vbase >= nvec) break;
             const uint64_t left = nvec - vbase;  // vectors from this group's start to the segment's end
             if (left < kThreads) {
-                fold_vector_remainder<T, OP>(L, sv, nfold, vbase, left, tid);
+                fold_vector_remainder<T, OP>(L, ptrs, sv, nfold, vbase, left, tid);
                 break;
             }
             const uint64_t in_off = sv.in_begin * sizeof(T) + vbase * kVecBytes;
@@ -499,7 +567,7 @@ __device__ __forceinline__ void fold_tile(const FoldLaunch& L) {
                 u32x4 x[K];
 #pragma unroll
                 for (int j = 0; j < K; ++j)
-                    x[j] = load_tile_any(static_cast<const char*>(L.in[rotate_rank(start, dir, j, nr)]) + in_off, tid);
+                    x[j] = load_tile_any(ptrs.in(rotate_rank(start, dir, j, nr)) + in_off, tid);
                 acc.seed(x[0]);
 #pragma unroll
                 for (int j = 1; j < K; ++j) acc.fold(x[j], new_wins);
@@ -510,8 +578,7 @@ __device__ __forceinline__ void fold_tile(const FoldLaunch& L) {
 #pragma unroll
                     for (uint32_t q = 0; q < 7; ++q)
                         if (j0 + q < nfold)
-                            x[q] = load_tile_any(
-                                    static_cast<const char*>(L.in[rotate_rank(start, dir, j0 + q, nr)]) + in_off, tid);
+                            x[q] = load_tile_any(ptrs.in(rotate_rank(start, dir, j0 + q, nr)) + in_off, tid);
 #pragma unroll
                     for (uint32_t q = 0; q < 7; ++q) {
                         if (j0 + q < nfold) {
@@ -523,17 +590,18 @@ __device__ __forceinline__ void fold_tile(const FoldLaunch& L) {
             }
             const u32x4 res = acc.finish();
             for (uint32_t m = 0; m < nout; ++m)
-                store_tile_any(static_cast<char*>(L.out[rotate_rank(out_first, 1, m, nr)]) + out_off, tid, res, L.keep != 0);
+                store_tile_any(ptrs.out(rotate_rank(out_first, 1, m, nr)) + out_off, tid, res, L.keep != 0);
         }
     } else {
-        fold_element_tile<T, OP>(L, sv, nfold, local_tile, tid);
+        fold_element_tile<T, OP>(L, ptrs, sv, nfold, local_tile, tid);
     }
 }
 
 template <typename T, int OP, int K>
 __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldLaunch L) {
+    const LaneArgs args = load_lane_args(threadIdx.x);  // issued first: nothing below depends on less
     if (!hook_enter(L.hooks, L.hook_target)) return;
-    fold_tile<T, OP, K>(L);
+    fold_tile<T, OP, K>(L, args);
     if (L.hook_ticket) hook_publish(L.hooks, L.hook_ticket);
 }
 
@@ -564,7 +632,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
     // wavefronts of a workgroup may see the poison rise at different moments and must all reach the barriers).
     const bool live = hook_poison(L.hooks) == 0;
     if (!sv.vector) {
-        if (wave == 0 && live) fold_element_tile<T, OP>(L, sv, nfold, sv.local_tile, tid);
+        if (wave == 0 && live) fold_element_tile<T, OP>(L, ArgPtrs{L}, sv, nfold, sv.local_tile, tid);
         return;
     }
     const uint64_t nvec = sv.count / EPV;
@@ -639,7 +707,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
     }
     // the segment's incomplete last group of vectors belongs to whoever owns its index
     if (mine == whole_groups && nvec % kThreads && live)
-        fold_vector_remainder<T, OP>(L, sv, nfold, mine * kThreads, nvec % kThreads, tid);
+        fold_vector_remainder<T, OP>(L, ArgPtrs{L}, sv, nfold, mine * kThreads, nvec % kThreads, tid);
 
     if (nout == 1) {
         if (have && live)
