@@ -260,11 +260,10 @@ private:
         uint64_t all_elems = 0;
         for (const Run& r : m_runs) all_elems += r.count;
         // short launches keep one wavefront per tile, and small tiles; folds that are vectors throughout keep them
-        // longer (kShortVectorMaxBytes)
+        // longer (short_vector_max_bytes)
         const uint64_t vector_tiles = vector_elems / (kThreads * epv);
         if (vector_elems == all_elems && m_nfold >= 2) {
-            const uint64_t one_out_max = m_elem == 1 ? kShortVectorMaxBytesOneOut / 2 : kShortVectorMaxBytesOneOut;
-            m_short = all_elems * m_elem <= (m_nout == 1 ? one_out_max : kShortVectorMaxBytes);
+            m_short = all_elems * m_elem <= short_vector_max_bytes(m_elem, m_nranks);
             m_waves = !m_short && vector_tiles >= kGroupMinTiles ? kGroupWaves : 1;
         } else {
             m_waves = vector_tiles >= kGroupMinTiles ? kGroupWaves : 1;

@@ -344,26 +344,28 @@ constexpr uint32_t kVecIters = 4;
 // of that per workgroup: a wavefront goes through its groups one after the other, one memory round trip each, and
 // when every wavefront of the launch fits the device at once anyway, four times the wavefronts finish in a quarter of
 // the time (5 ranks x 256 KiB fp32 all_reduce: 10.9 -> 5 us).
-// Launches whose buffers are all vectors keep that form well beyond the point where the device is full, because the
+// Folds whose buffers are all vectors keep that form well beyond the point where the device is full, because the
 // group form (which begins where it ends) only pays on long launches.  Measured on MI355X, microseconds per launch,
-// group form / one wavefront per group of vectors, fp32 (fp16 alike), by KiB per buffer:
-//   all_reduce      5 ranks  1024 6.29 / 5.68   2048 6.97 / 6.37   3072 8.43 / 7.38   4096 8.90 / 9.31    8192 15.6 / 16.4
-//                   7 ranks  1024 7.01 / 6.42   2048 8.61 / 7.90   3072 10.2 / 8.91   4096 11.4 / 12.3    8192 21.0 / 21.4
-//                  12 ranks  1024 9.40 / 8.21   2048 12.9 / 10.1   3072 13.8 / 14.5   4096 19.3 / 22.1    8192 35.5 / 34.8
-//                  16 ranks  1024 8.20 / 7.79   2048 11.9 / 11.5   3072 21.1 / 18.8   4096 22.5 / 25.4    8192 43.1 / 44.8
-//   reduce_scatter  5 ranks  1024 5.62 / 5.01   2048 5.80 / 5.20   4096 6.63 / 6.13   8192 10.1 / 9.48   16384 16.9 / 17.3
-//                   7 ranks  1024 5.83 / 5.32   2048 6.03 / 5.67   4096 7.10 / 7.37   8192 13.2 / 12.5   16384 21.0 / 22.2
-//                  12 ranks  1024 7.43 / 6.41   2048 7.71 / 8.35   4096 10.8 / 10.6   8192 22.4 / 20.1   16384 35.2 / 37.3
-//                  16 ranks  1024 7.40 / 7.16   2048 8.06 / 7.56   4096 12.5 / 12.6   8192 23.5 / 22.4   16384 43.8 / 44.8
-// (with the usual four groups per wavefront the one-wavefront form takes 9 - 25 us at 2048 KiB); from 16 MiB to 256 MiB
-// the group form is 2 - 20 % ahead.  Hence: up to 3 MiB per buffer, and up to 8 MiB where every element has one
-// destination (4 MiB for elements of one byte: int8 reduce_scatter of 5 ranks, odd receive length, 6 MiB 9.2 / 10.5).
-// Buffers off the vector grid gain most: fp16 all_reduce of 8 ranks x 1.5 MiB at 48 bytes off 12.2 / 8.8, int8 10.1 / 6.1.  Launches with element tiles (buffers at differing offsets from a 4-byte boundary) keep the 1 MiB limit
-// and take the group form for their vector bodies from kGroupMinTiles on.
+// group form / one wavefront per group of vectors, fp32, by KiB per buffer:
+//   all_reduce      5 ranks  2048 6.00 / 5.39   4096 8.74 / 7.63   8192 15.5 / 15.4   12288 21.6 / 21.0   16384 27.6 / 28.0   32768 61.3 / 66.4
+//                   7 ranks  2048 7.72 / 5.76   4096 11.0 / 9.61   8192 22.7 / 20.3   12288 29.2 / 29.5   16384 37.6 / 38.1   32768 77.6 / 81.2
+//                  12 ranks  2048 13.2 / 8.85   4096 18.9 / 16.1   8192 34.0 / 31.8   12288 53.5 / 54.8   16384 71.0 / 74.7   32768 135 / 145
+//                  16 ranks  2048 12.0 / 10.2   4096 22.0 / 20.1   8192 43.3 / 44.1   12288 69.7 / 71.8   16384 100 / 104     32768 174 / 192
+//     8 ranks, 4 bytes off   2048 8.95 / 6.54   4096 14.1 / 11.4   8192 23.0 / 20.5   12288 31.7 / 31.8   16384 43.5 / 41.4   32768 95.7 / 92.9
+//   reduce_scatter  5 ranks  2048 5.43 / 4.60   4096 6.56 / 5.53   8192 9.77 / 8.59   12288 13.2 / 13.2   16384 16.9 / 17.5   32768 31.4 / 34.0
+//                   7 ranks  2048 5.99 / 4.69   4096 6.65 / 5.98   8192 12.3 / 11.6   12288 16.7 / 16.9   16384 21.0 / 22.3   32768 42.4 / 41.8
+//                  16 ranks  2048 8.56 / 7.33   4096 12.0 / 10.9   8192 23.2 / 22.0   12288 33.6 / 33.7   16384 45.4 / 46.0   32768 89.0 / 91.8
+// (with the usual four groups per wavefront the one-wavefront form takes 9 - 25 us at 2048 KiB; from 16 MiB to 256 MiB
+// the group form is 2 - 20 % ahead).  fp16 and int64 cross at the same sizes.  One-byte elements, whose arithmetic
+// takes longer, cross earlier: int8 all_reduce of 5 / 7 / 16 ranks x 2 MiB 5.97 / 5.65, 11.4 / 7.69, 12.3 / 16.9, x 4 MiB
+// 9.44 / 9.89, 11.7 / 12.7, 22.5 / 22.5.  Hence: up to 8 MiB per buffer, for one-byte elements up to 2 MiB (1 MiB from
+// twelve ranks on).  Launches with element tiles (buffers at differing offsets from a 4-byte boundary) and copies
+// keep the 1 MiB limit and take the group form for their vector bodies from kGroupMinTiles on.
 constexpr uint32_t kShortElemsPerLane = 4;
 constexpr uint64_t kShortTilesMaxBytes = uint64_t(1) << 20;
-constexpr uint64_t kShortVectorMaxBytes = uint64_t(3) << 20;
-constexpr uint64_t kShortVectorMaxBytesOneOut = uint64_t(8) << 20;
+constexpr uint64_t short_vector_max_bytes(uint32_t elem_size, uint32_t nranks) {
+    return elem_size > 1 ? uint64_t(8) << 20 : nranks >= 12 ? uint64_t(1) << 20 : uint64_t(2) << 20;
+}
 constexpr uint32_t vec_iters(const FoldLaunch& L) { return L.short_tiles ? 1u : kVecIters; }
 constexpr uint32_t elems_per_lane(const FoldLaunch& L) { return L.short_tiles ? kShortElemsPerLane : kElemsPerLane; }
 

@@ -179,11 +179,12 @@ def test_either_store_policy_gives_the_same_results(keep, monkeypatch):
 @pytest.mark.parametrize("dtype", [orc.INT8, orc.FLOAT16, orc.FLOAT32, orc.INT64])
 def test_general_folds_of_a_few_mib_keep_one_wavefront_per_group_of_vectors(dtype):
     """Folds through the general kernel whose buffers are vectors throughout keep one wavefront per group of 64
-    vectors up to 3 MiB per buffer (8 MiB where every element has one destination; 4 MiB for one-byte elements):
-    rank counts without a flat kernel, and eight ranks at a common offset from a 16-byte boundary."""
+    vectors up to 8 MiB per buffer (one-byte elements: 2 MiB, and 1 MiB from twelve ranks on): rank counts without a
+    flat kernel, and eight ranks at a common offset from a 16-byte boundary."""
     size = orc.dtype_size(dtype)
     rng = np.random.default_rng(377 + dtype)
-    for nranks, offset, kib in ((5, 0, 2900), (7, 0, 1500), (8, max(size, 4), 2100)):
+    for nranks, offset, kib in ((5, 0, 7900), (7, 0, 1500), (8, max(size, 4), 4100)):
+        kib = min(kib, 1900) if size == 1 else kib
         length = kib * 1024 // size + 5
         ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
         d_in = [to_device(x, offset) for x in ins]
@@ -195,7 +196,7 @@ def test_general_folds_of_a_few_mib_keep_one_wavefront_per_group_of_vectors(dtyp
             got = run_all_reduce(ins, dtype, op, order, mr.Schedule.FUSED, offsets=[offset] * nranks)
             for r in range(nranks):
                 assert_same(got[r], want[r], f"all_reduce dtype={dtype} N={nranks} offset={offset} op={op} rank={r}")
-    for nranks, kib in ((6, 3900 if size == 1 else 7900), (12, 3000)):
+    for nranks, kib in ((6, 1900 if size == 1 else 7900), (12, 900 if size == 1 else 3000)):
         recvlen = kib * 1024 // size // nranks // 16 * 16 + 16
         ins = [rand_array(dtype, recvlen * nranks, rng) for _ in range(nranks)]
         d_in = [to_device(x) for x in ins]
@@ -211,8 +212,8 @@ def test_general_folds_of_a_few_mib_keep_one_wavefront_per_group_of_vectors(dtyp
 
 @pytest.mark.parametrize("dtype", REDUCE_TYPES)
 def test_segment_group_form(dtype):
-    """The general fold kernel with long vector bodies (512 groups of 64 vectors and more) runs in its
-    group form: rank counts without a flat kernel (5 and 16: the fold count is read from the launch and
+    """The general fold kernel with long vector bodies (beyond 8 MiB per buffer; 512 groups of 64 vectors and more
+    for copies and for buffers with element tiles) runs in its group form: rank counts without a flat kernel (5 and 16: the fold count is read from the launch and
     the inputs pass through LDS four at a time), buffers that share an offset from a 16-byte boundary,
     and the ring replay's two-input steps and copies."""
     size = orc.dtype_size(dtype)
@@ -223,8 +224,8 @@ def test_segment_group_form(dtype):
     for nranks, offset, sched, op, order in cases:
         if sched == mr.Schedule.RING and dtype == orc.FLOAT16:
             continue  # the ring replay would round at every hop and is refused for FLOAT16
-        per_chunk = 4300 if sched == mr.Schedule.RING else 0  # ring steps work on one chunk per rank
-        tiles = max(4300, per_chunk * nranks)
+        per_chunk = 8300 if sched == mr.Schedule.RING else 0  # ring steps work on one chunk per rank
+        tiles = max(8300, per_chunk * nranks)
         length = tiles * 1024 // size + 7
         ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
         d_in = [to_device(x, offset) for x in ins]
