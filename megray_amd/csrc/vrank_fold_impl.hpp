@@ -125,6 +125,21 @@ __device__ __forceinline__ void store_tile_any(char* tile_base, uint32_t lane, u
     if ((reinterpret_cast<uintptr_t>(tile_base) & 3u) == 0) store_tile_vec(tile_base, lane, x, keep);
     else store_vec(tile_base + lane * kVecBytes, x);
 }
+// The same for tiles of elements of type T: buffers of 4- and 8-byte elements are element aligned wherever a kernel
+// takes them a vector at a time, so their tiles always sit on 4-byte boundaries.  Leaving the other path out of those
+// kernels matters beyond the test it saves: it is made of flat instructions, which complete out of order with the
+// buffer instructions around them, and a kernel that contains both waits for everything outstanding wherever it
+// waits at all - a wavefront's loads, and its stores to several ranks, then go one at a time.
+template <typename T>
+__device__ __forceinline__ u32x4 load_tile_of(const char* tile_base, uint32_t lane) {
+    if constexpr (sizeof(T) >= 4) return load_tile_vec(tile_base, lane);
+    else return load_tile_any(tile_base, lane);
+}
+template <typename T>
+__device__ __forceinline__ void store_tile_of(char* tile_base, uint32_t lane, u32x4 x, bool keep) {
+    if constexpr (sizeof(T) >= 4) store_tile_vec(tile_base, lane, x, keep);
+    else store_tile_any(tile_base, lane, x, keep);
+}
 
 // One element at byte `offset` (a multiple of the element size, below 1 KiB) of a tile, with the tile stores' cache
 // policy: written through, so that the kernel's end finds nothing to write back (a plain store leaves its line dirty
@@ -466,19 +481,48 @@ __device__ __forceinline__ void fold_vector_remainder(const FoldLaunch& L, const
     const uint64_t in_off = sv.in_begin * sizeof(T) + (vbase + tid) * kVecBytes;
     const uint64_t out_off = sv.out_begin * sizeof(T) + (vbase + tid) * kVecBytes;
     AccFor<T, OP> a;
-    a.seed(load_vec(ptrs.in(sv.start) + in_off));
-    for (uint32_t j0 = 1; j0 < nfold; j0 += 8) {  // the loads of up to eight ranks in flight together
-        u32x4 x[8];
+    // the loads of up to eight ranks in flight together, every batch size and the stores as straight-line code (see fold_tile)
+    const auto batch = [&](auto count, uint32_t j0) {
+        constexpr uint32_t C = decltype(count)::value;
+        u32x4 x[C];
 #pragma unroll
-        for (uint32_t b = 0; b < 8; ++b)
-            if (j0 + b < nfold) x[b] = load_vec(ptrs.in(rotate_rank(sv.start, sv.dir, j0 + b, nr)) + in_off);
+        for (uint32_t q = 0; q < C; ++q) x[q] = load_vec(ptrs.in(rotate_rank(sv.start, sv.dir, j0 + q, nr)) + in_off);
+        if (j0 == 0) a.seed(x[0]);
+        else a.fold(x[0], new_wins);
 #pragma unroll
-        for (uint32_t b = 0; b < 8; ++b)
-            if (j0 + b < nfold) a.fold(x[b], new_wins);
+        for (uint32_t q = 1; q < C; ++q) a.fold(x[q], new_wins);
+    };
+    uint32_t j0 = 0;
+    for (; j0 + 8 <= nfold; j0 += 8) batch(std::integral_constant<uint32_t, 8>{}, j0);
+    switch (nfold - j0) {
+        case 1: batch(std::integral_constant<uint32_t, 1>{}, j0); break;
+        case 2: batch(std::integral_constant<uint32_t, 2>{}, j0); break;
+        case 3: batch(std::integral_constant<uint32_t, 3>{}, j0); break;
+        case 4: batch(std::integral_constant<uint32_t, 4>{}, j0); break;
+        case 5: batch(std::integral_constant<uint32_t, 5>{}, j0); break;
+        case 6: batch(std::integral_constant<uint32_t, 6>{}, j0); break;
+        case 7: batch(std::integral_constant<uint32_t, 7>{}, j0); break;
+        default: break;
     }
     const u32x4 r = a.finish();
-    for (uint32_t m = 0; m < L.nout; ++m)
-        store_vec(ptrs.out(rotate_rank(sv.out_first, 1, m, nr)) + out_off, r);
+    const auto put = [&](auto count, uint32_t m0) {
+        constexpr uint32_t C = decltype(count)::value;
+#pragma unroll
+        for (uint32_t q = 0; q < C; ++q) store_vec(ptrs.out(rotate_rank(sv.out_first, 1, m0 + q, nr)) + out_off, r);
+    };
+    const uint32_t nout = L.nout;
+    uint32_t m0 = 0;
+    for (; m0 + 8 <= nout; m0 += 8) put(std::integral_constant<uint32_t, 8>{}, m0);
+    switch (nout - m0) {
+        case 1: put(std::integral_constant<uint32_t, 1>{}, m0); break;
+        case 2: put(std::integral_constant<uint32_t, 2>{}, m0); break;
+        case 3: put(std::integral_constant<uint32_t, 3>{}, m0); break;
+        case 4: put(std::integral_constant<uint32_t, 4>{}, m0); break;
+        case 5: put(std::integral_constant<uint32_t, 5>{}, m0); break;
+        case 6: put(std::integral_constant<uint32_t, 6>{}, m0); break;
+        case 7: put(std::integral_constant<uint32_t, 7>{}, m0); break;
+        default: break;
+    }
 }
 
 // Every lane polls the same word (one request per wavefront) until it reaches `target` or the time
@@ -567,30 +611,62 @@ __device__ __forceinline__ void fold_tile(const FoldLaunch& L, const LaneArgs& a
                 u32x4 x[K];
 #pragma unroll
                 for (int j = 0; j < K; ++j)
-                    x[j] = load_tile_any(ptrs.in(rotate_rank(start, dir, j, nr)) + in_off, tid);
+                    x[j] = load_tile_of<T>(ptrs.in(rotate_rank(start, dir, j, nr)) + in_off, tid);
                 acc.seed(x[0]);
 #pragma unroll
                 for (int j = 1; j < K; ++j) acc.fold(x[j], new_wins);
             } else {
-                // seven inputs at a time in flight, the seed among the first (eight cost twice the registers)
-                for (uint32_t j0 = 0; j0 < nfold; j0 += 7) {
-                    u32x4 x[7];
+                // seven inputs at a time in flight, the seed among the first (eight cost twice the registers).  Every
+                // batch size is straight-line code of its own: loads guarded one by one leave the compiler with values that
+                // are defined on some paths only, which it copies at every join - after waiting for every load before it.
+                const auto batch = [&](auto count, uint32_t j0) {
+                    constexpr uint32_t C = decltype(count)::value;
+                    u32x4 x[C];
 #pragma unroll
-                    for (uint32_t q = 0; q < 7; ++q)
-                        if (j0 + q < nfold)
-                            x[q] = load_tile_any(ptrs.in(rotate_rank(start, dir, j0 + q, nr)) + in_off, tid);
+                    for (uint32_t q = 0; q < C; ++q)
+                        x[q] = load_tile_of<T>(ptrs.in(rotate_rank(start, dir, j0 + q, nr)) + in_off, tid);
+                    if (j0 == 0) acc.seed(x[0]);
+                    else acc.fold(x[0], new_wins);
 #pragma unroll
-                    for (uint32_t q = 0; q < 7; ++q) {
-                        if (j0 + q < nfold) {
-                            if (j0 + q == 0) acc.seed(x[q]);
-                            else acc.fold(x[q], new_wins);
-                        }
-                    }
+                    for (uint32_t q = 1; q < C; ++q) acc.fold(x[q], new_wins);
+                };
+                uint32_t j0 = 0;
+                for (; j0 + 7 <= nfold; j0 += 7) batch(std::integral_constant<uint32_t, 7>{}, j0);
+                switch (nfold - j0) {
+                    case 1: batch(std::integral_constant<uint32_t, 1>{}, j0); break;
+                    case 2: batch(std::integral_constant<uint32_t, 2>{}, j0); break;
+                    case 3: batch(std::integral_constant<uint32_t, 3>{}, j0); break;
+                    case 4: batch(std::integral_constant<uint32_t, 4>{}, j0); break;
+                    case 5: batch(std::integral_constant<uint32_t, 5>{}, j0); break;
+                    case 6: batch(std::integral_constant<uint32_t, 6>{}, j0); break;
+                    default: break;
                 }
             }
             const u32x4 res = acc.finish();
-            for (uint32_t m = 0; m < nout; ++m)
-                store_tile_any(ptrs.out(rotate_rank(out_first, 1, m, nr)) + out_off, tid, res, L.keep != 0);
+            // the stores likewise, eight at a time and either policy on a path of its own: in a loop the compiler waits
+            // for each store before it issues the next
+            const auto put = [&](auto count, auto kept, uint32_t m0) {
+                constexpr uint32_t C = decltype(count)::value;
+#pragma unroll
+                for (uint32_t q = 0; q < C; ++q)
+                    store_tile_of<T>(ptrs.out(rotate_rank(out_first, 1, m0 + q, nr)) + out_off, tid, res, decltype(kept)::value);
+            };
+            const auto put_all = [&](auto kept) {
+                uint32_t m0 = 0;
+                for (; m0 + 8 <= nout; m0 += 8) put(std::integral_constant<uint32_t, 8>{}, kept, m0);
+                switch (nout - m0) {
+                    case 1: put(std::integral_constant<uint32_t, 1>{}, kept, m0); break;
+                    case 2: put(std::integral_constant<uint32_t, 2>{}, kept, m0); break;
+                    case 3: put(std::integral_constant<uint32_t, 3>{}, kept, m0); break;
+                    case 4: put(std::integral_constant<uint32_t, 4>{}, kept, m0); break;
+                    case 5: put(std::integral_constant<uint32_t, 5>{}, kept, m0); break;
+                    case 6: put(std::integral_constant<uint32_t, 6>{}, kept, m0); break;
+                    case 7: put(std::integral_constant<uint32_t, 7>{}, kept, m0); break;
+                    default: break;
+                }
+            };
+            if (L.keep != 0) put_all(std::true_type{});
+            else put_all(std::false_type{});
         }
     } else {
         fold_element_tile<T, OP>(L, ptrs, sv, nfold, local_tile, tid);
@@ -660,7 +736,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
     AccFor<T, OP> acc;
     if constexpr (K == 1) {
         // a copy: nothing to skew on the load side
-        if (have) acc.seed(load_tile_any(static_cast<const char*>(L.in[sv.start]) + in_base + mine * kGroupBytes, tid));
+        if (have) acc.seed(load_tile_of<T>(static_cast<const char*>(L.in[sv.start]) + in_base + mine * kGroupBytes, tid));
     } else {
         // Long launches keep two loads per wavefront in flight instead of all SK (L.paced, as in the flat group
         // kernel): load q + 2 is issued when load q has arrived.
@@ -670,7 +746,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
             const auto load_input = [&](uint32_t q, uint32_t lane) -> u32x4 {
                 const uint64_t group = first + ((wave + q) % W) * kGroupStride;
                 if (j0 + q < nfold && group < whole_groups)
-                    return load_tile_any(static_cast<const char*>(L.in[rotate_rank(sv.start, sv.dir, j0 + q, nr)]) +
+                    return load_tile_of<T>(static_cast<const char*>(L.in[rotate_rank(sv.start, sv.dir, j0 + q, nr)]) +
                                                  in_base + group * kGroupBytes,
                                          lane);
                 return u32x4{0u, 0u, 0u, 0u};
@@ -711,7 +787,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
 
     if (nout == 1) {
         if (have && live)
-            store_tile_any(static_cast<char*>(L.out[sv.out_first]) + out_base + mine * kGroupBytes, tid, acc.finish(), L.keep != 0);
+            store_tile_of<T>(static_cast<char*>(L.out[sv.out_first]) + out_base + mine * kGroupBytes, tid, acc.finish(), L.keep != 0);
         return;
     }
     if (have) result[wave][tid] = acc.finish();
@@ -720,7 +796,7 @@ __global__ void __launch_bounds__(kThreads * kGroupWaves) fold_segment_group_ker
     for (uint32_t m = 0; m < nout; ++m) {
         const uint32_t k = (wave + m) % W;
         if (folded[k] && live)
-            store_tile_any(static_cast<char*>(L.out[rotate_rank(sv.out_first, 1, m, nr)]) + out_base +
+            store_tile_of<T>(static_cast<char*>(L.out[rotate_rank(sv.out_first, 1, m, nr)]) + out_base +
                                    (first + uint64_t(k) * kGroupStride) * kGroupBytes,
                            tid, result[k][tid], L.keep != 0);
         if (L.paced && (m + 1) % kGroupStoresInFlight == 0 && m + 1 < nout) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -810,7 +886,7 @@ __device__ __forceinline__ TreeAccFor<T, OP> tree_node(const TreeLaunch& L, uint
     if constexpr (SPAN == 1) {
         TreeAccFor<T, OP> a;
         const char* base = static_cast<const char*>(L.in[rotate_rank(L.root, 1, v0, L.nranks)]) + off;
-        if constexpr (TILE) a.seed(load_tile_any(base, tid));
+        if constexpr (TILE) a.seed(load_tile_of<T>(base, tid));
         else a.seed(load_vec(base));
         return a;
     } else {
@@ -838,7 +914,7 @@ __device__ __forceinline__ void tree_tile(const TreeLaunch& L) {
     if ((uint64_t(blockIdx.x) + 1) * kThreads <= nvec) {
         // a whole tile: buffer instructions with the streaming cache policies
         const u32x4 r = tree_node<T, OP, kMaxRanks, true>(L, tile_off, 0, threadIdx.x).finish();
-        store_tile_any(static_cast<char*>(L.out) + tile_off, threadIdx.x, r, L.keep != 0);
+        store_tile_of<T>(static_cast<char*>(L.out) + tile_off, threadIdx.x, r, L.keep != 0);
     } else if (lane < nvec) {
         store_vec(static_cast<char*>(L.out) + lane * kVecBytes, tree_vector<T, OP>(L, lane * kVecBytes));
     }
@@ -1076,7 +1152,7 @@ __device__ __forceinline__ void flat_tile_ragged(const FlatLaunch& L, uint32_t t
             for (uint32_t m = 0; m < nout; ++m) {
                 char* out_tile = static_cast<char*>(L.out[rotate_rank(out_first, 1, m, K)]) + tile_out;
                 if (whole_vector) {
-                    store_tile_any(out_tile, tid, res, keep);
+                    store_tile_of<T>(out_tile, tid, res, keep);
                 } else {
                     T* out = reinterpret_cast<T*>(out_tile) + lane_off;
 #pragma unroll
@@ -1140,7 +1216,7 @@ __device__ __forceinline__ void flat_tile_uncovered(const FlatLaunch& L, uint32_
     for (int m = 0; m < K; ++m) {
         char* out_tile = static_cast<char*>(L.out[m]) + tile_off;
         if (tid < nfull) {
-            store_tile_any(out_tile, tid, merged, keep);
+            store_tile_of<T>(out_tile, tid, merged, keep);
         } else if (tid == nfull) {  // the elements behind the last whole vector
             T* out = reinterpret_cast<T*>(out_tile) + tid * EPV;
 #pragma unroll

@@ -358,13 +358,16 @@ constexpr uint32_t kVecIters = 4;
 // (with the usual four groups per wavefront the one-wavefront form takes 9 - 25 us at 2048 KiB; from 16 MiB to 256 MiB
 // the group form is 2 - 20 % ahead).  fp16 and int64 cross at the same sizes.  One-byte elements, whose arithmetic
 // takes longer, cross earlier: int8 all_reduce of 5 / 7 / 16 ranks x 2 MiB 5.97 / 5.65, 11.4 / 7.69, 12.3 / 16.9, x 4 MiB
-// 9.44 / 9.89, 11.7 / 12.7, 22.5 / 22.5.  Hence: up to 8 MiB per buffer, for one-byte elements up to 2 MiB (1 MiB from
-// twelve ranks on).  Launches with element tiles (buffers at differing offsets from a 4-byte boundary) and copies
+// 9.44 / 9.89, 11.7 / 12.7, 22.5 / 22.5.  On placed buffers the all_reduce of 12 and 16 ranks x 4 MiB reads 19.1 / 21.0 and
+// 22.9 / 25.3 (its stores are kept in the cache at that size), x 8 MiB 35.4 / 32.2 and 43.5 / 43.2.  Hence: up to 8 MiB per
+// buffer (3 MiB for folds of twelve and more ranks with several destinations), for one-byte elements up to 2 MiB (1 MiB
+// from twelve ranks on).  Launches with element tiles (buffers at differing offsets from a 4-byte boundary) and copies
 // keep the 1 MiB limit and take the group form for their vector bodies from kGroupMinTiles on.
 constexpr uint32_t kShortElemsPerLane = 4;
 constexpr uint64_t kShortTilesMaxBytes = uint64_t(1) << 20;
-constexpr uint64_t short_vector_max_bytes(uint32_t elem_size, uint32_t nranks) {
-    return elem_size > 1 ? uint64_t(8) << 20 : nranks >= 12 ? uint64_t(1) << 20 : uint64_t(2) << 20;
+constexpr uint64_t short_vector_max_bytes(uint32_t elem_size, uint32_t nranks, uint32_t nout) {
+    if (elem_size == 1) return nranks >= 12 ? uint64_t(1) << 20 : uint64_t(2) << 20;
+    return nranks >= 12 && nout > 1 ? uint64_t(3) << 20 : uint64_t(8) << 20;
 }
 constexpr uint32_t vec_iters(const FoldLaunch& L) { return L.short_tiles ? 1u : kVecIters; }
 constexpr uint32_t elems_per_lane(const FoldLaunch& L) { return L.short_tiles ? kShortElemsPerLane : kElemsPerLane; }

@@ -179,7 +179,7 @@ def test_either_store_policy_gives_the_same_results(keep, monkeypatch):
 @pytest.mark.parametrize("dtype", [orc.INT8, orc.FLOAT16, orc.FLOAT32, orc.INT64])
 def test_general_folds_of_a_few_mib_keep_one_wavefront_per_group_of_vectors(dtype):
     """Folds through the general kernel whose buffers are vectors throughout keep one wavefront per group of 64
-    vectors up to 8 MiB per buffer (one-byte elements: 2 MiB, and 1 MiB from twelve ranks on): rank counts without a
+    vectors up to 8 MiB per buffer (3 MiB for twelve and more ranks with several destinations; one-byte elements: 2 MiB, and 1 MiB from twelve ranks on): rank counts without a
     flat kernel, and eight ranks at a common offset from a 16-byte boundary."""
     size = orc.dtype_size(dtype)
     rng = np.random.default_rng(377 + dtype)
