@@ -162,8 +162,10 @@ Status resolve(const Plan& plan, DType dtype, ReduceOp op, std::vector<KernelCal
                 break;
             case Step::kTree:
                 call = {tree_kernel_for(step.tree, dtype, op), step.tree.total_tiles, kThreads, &step.tree};
-                if (step.tree.vector && step.tree.elem_size >= 4 && step.tree.total_tiles >= tree_cap_min_tiles(step.tree.nranks))
-                    call.lds = lds_for_waves_per_cu(call.kernel, kTreeCapWavesPerCu);
+                if (step.tree.vector) {
+                    const uint32_t per_cu = tree_waves_per_cu(step.tree.nranks, step.tree.total_tiles, step.tree.keep != 0, step.tree.elem_size);
+                    if (per_cu) call.lds = lds_for_waves_per_cu(call.kernel, per_cu);
+                }
                 break;
             case Step::kPack:
                 if (step.pack.waves == kGroupWaves) {

@@ -875,14 +875,94 @@ __device__ __forceinline__ T tree_element(const Launch& L, uint32_t n, uint32_t 
     return static_cast<T>(a[0]);
 }
 
-// The same tree on the 16-byte vector at byte offset `off` of up to kMaxRanks buffers, walked depth
-// first: the subtree of SPAN virtual ranks from v0 (v0 < count) is its left half combined with its
-// right half, if there is one.  That is the expression the rounds of the element-wise form build,
-// with at most log2(kMaxRanks) + 1 accumulators alive at a time.
+// The same tree on the 16-byte vector at byte offset `off` of up to kMaxRanks buffers.  The subtree of SPAN virtual
+// ranks from v0 is its left half combined with its right half, if there is one: that is the expression the rounds of
+// the element-wise form build.  It is evaluated eight leaves at a time: the loads of a batch are straight-line code for
+// every batch size and all in flight together, the subtree of a batch is fixed at compile time, and the up to four
+// batch values are combined by the same rule.  (The plain recursive walk, tree_walk below, tests the rank count at every
+// node; that leaves the compiler with loads on some paths only, and it waits for each before it issues the next, so
+// that a wavefront has two or three loads in flight.  Long launches of few ranks and 4- or 8-byte elements whose
+// stores stream are served best that way, and keep it: TreeLaunch::batch.)
 // TILE: `off` is the byte offset of a whole tile, loaded with one buffer instruction per rank (lane `tid`
 // takes its vector of it); otherwise `off` is the lane's own vector.
+template <typename T, int OP, uint32_t SPAN, uint32_t C>
+__device__ __forceinline__ TreeAccFor<T, OP> tree_of_batch(const u32x4* x) {  // C of the SPAN leaves exist, 1 <= C <= SPAN
+    if constexpr (SPAN == 1) {
+        TreeAccFor<T, OP> a;
+        a.seed(x[0]);
+        return a;
+    } else {
+        constexpr uint32_t H = SPAN / 2;
+        TreeAccFor<T, OP> left = tree_of_batch<T, OP, H, (C < H ? C : H)>(x);
+        if constexpr (C > H) left.merge(tree_of_batch<T, OP, H, C - H>(x + H));
+        return left;
+    }
+}
+// (the rank pointers come out of a register that holds the descriptor's in[], lane l entry l: see LanePtrs)
+struct TreeRanks {
+    LanePtrs ptrs;
+    uint32_t root, nranks, batch;
+};
+__device__ __forceinline__ TreeRanks load_tree_ranks(const TreeLaunch& L, uint32_t lane) {
+    using Constant = const __attribute__((address_space(4))) char;
+    Constant* base = (Constant*)__builtin_amdgcn_kernarg_segment_ptr();  // the descriptor is the only argument
+    const auto* ptr = reinterpret_cast<const __attribute__((address_space(4))) uint32_t*>(
+            base + offsetof(TreeLaunch, in) + (lane % kMaxRanks) * sizeof(void*));
+    TreeRanks r;
+    r.ptrs.lo = ptr[0];
+    r.ptrs.hi = ptr[1];
+    r.root = L.root;
+    r.nranks = L.nranks;
+    r.batch = L.batch;
+    return r;
+}
+template <typename T, int OP, bool TILE, uint32_t B, uint32_t C>
+__device__ __forceinline__ TreeAccFor<T, OP> tree_batch(const TreeRanks& L, uint64_t off, uint32_t v0, uint32_t tid) {
+    u32x4 x[C];
+#pragma unroll
+    for (uint32_t q = 0; q < C; ++q) {
+        const char* base = L.ptrs.in(rotate_rank(L.root, 1, v0 + q, L.nranks)) + off;
+        if constexpr (TILE) x[q] = load_tile_of<T>(base, tid);
+        else x[q] = load_vec(base);
+    }
+    return tree_of_batch<T, OP, B, C>(x);
+}
+template <typename T, int OP, bool TILE, uint32_t B>
+__device__ __forceinline__ TreeAccFor<T, OP> tree_batch_of(const TreeRanks& L, uint64_t off, uint32_t v0, uint32_t tid) {
+    const uint32_t left = L.nranks - v0;  // leaves from v0 on: a whole batch, or what is left
+    if constexpr (B >= 8) {
+        switch (left) {
+            case 7: return tree_batch<T, OP, TILE, B, 7>(L, off, v0, tid);
+            case 6: return tree_batch<T, OP, TILE, B, 6>(L, off, v0, tid);
+            case 5: return tree_batch<T, OP, TILE, B, 5>(L, off, v0, tid);
+            case 4: return tree_batch<T, OP, TILE, B, 4>(L, off, v0, tid);
+            default: break;
+        }
+    }
+    if constexpr (B >= 4) {
+        switch (left) {
+            case 3: return tree_batch<T, OP, TILE, B, 3>(L, off, v0, tid);
+            case 2: return tree_batch<T, OP, TILE, B, 2>(L, off, v0, tid);
+            default: break;
+        }
+    }
+    if (left == 1) return tree_batch<T, OP, TILE, B, 1>(L, off, v0, tid);
+    return tree_batch<T, OP, TILE, B, B>(L, off, v0, tid);
+}
+// the batch values of SPAN batches from batch b0, combined by the same rule
+template <typename T, int OP, bool TILE, uint32_t B, uint32_t SPAN>
+__device__ __forceinline__ TreeAccFor<T, OP> tree_top(const TreeRanks& L, uint64_t off, uint32_t b0, uint32_t tid) {
+    if constexpr (SPAN == 1) {
+        return tree_batch_of<T, OP, TILE, B>(L, off, b0 * B, tid);
+    } else {
+        TreeAccFor<T, OP> left = tree_top<T, OP, TILE, B, SPAN / 2>(L, off, b0, tid);
+        if ((b0 + SPAN / 2) * B < L.nranks) left.merge(tree_top<T, OP, TILE, B, SPAN / 2>(L, off, b0 + SPAN / 2, tid));
+        return left;
+    }
+}
+// The plain recursive walk, one leaf at a time, rank pointers read from the descriptor as they are needed (see above).
 template <typename T, int OP, uint32_t SPAN, bool TILE>
-__device__ __forceinline__ TreeAccFor<T, OP> tree_node(const TreeLaunch& L, uint64_t off, uint32_t v0, uint32_t tid) {
+__device__ __forceinline__ TreeAccFor<T, OP> tree_walk(const TreeLaunch& L, uint64_t off, uint32_t v0, uint32_t tid) {
     if constexpr (SPAN == 1) {
         TreeAccFor<T, OP> a;
         const char* base = static_cast<const char*>(L.in[rotate_rank(L.root, 1, v0, L.nranks)]) + off;
@@ -890,19 +970,23 @@ __device__ __forceinline__ TreeAccFor<T, OP> tree_node(const TreeLaunch& L, uint
         else a.seed(load_vec(base));
         return a;
     } else {
-        TreeAccFor<T, OP> left = tree_node<T, OP, SPAN / 2, TILE>(L, off, v0, tid);
-        if (v0 + SPAN / 2 < L.nranks) left.merge(tree_node<T, OP, SPAN / 2, TILE>(L, off, v0 + SPAN / 2, tid));
+        TreeAccFor<T, OP> left = tree_walk<T, OP, SPAN / 2, TILE>(L, off, v0, tid);
+        if (v0 + SPAN / 2 < L.nranks) left.merge(tree_walk<T, OP, SPAN / 2, TILE>(L, off, v0 + SPAN / 2, tid));
         return left;
     }
 }
-
-template <typename T, int OP>
-__device__ __forceinline__ u32x4 tree_vector(const TreeLaunch& L, uint64_t off) {
-    return tree_node<T, OP, kMaxRanks, false>(L, off, 0, 0).finish();
+template <typename T, int OP, bool TILE>
+__device__ __forceinline__ TreeAccFor<T, OP> tree_node(const TreeRanks& L, uint64_t off, uint32_t tid) {
+    return tree_top<T, OP, TILE, 8, kMaxRanks / 8>(L, off, 0, tid);
 }
 
 template <typename T, int OP>
-__device__ __forceinline__ void tree_tile(const TreeLaunch& L) {
+__device__ __forceinline__ u32x4 tree_vector(const TreeRanks& L, uint64_t off) {
+    return tree_node<T, OP, false>(L, off, 0).finish();
+}
+
+template <typename T, int OP>
+__device__ __forceinline__ void tree_tile(const TreeLaunch& L, const TreeRanks& ranks) {
     constexpr uint32_t EPV = kVecBytes / sizeof(T);
     const uint64_t lane = uint64_t(blockIdx.x) * kThreads + threadIdx.x;
     if (!L.vector) {
@@ -913,10 +997,11 @@ __device__ __forceinline__ void tree_tile(const TreeLaunch& L) {
     const uint64_t tile_off = uint64_t(blockIdx.x) * kThreads * kVecBytes;
     if ((uint64_t(blockIdx.x) + 1) * kThreads <= nvec) {
         // a whole tile: buffer instructions with the streaming cache policies
-        const u32x4 r = tree_node<T, OP, kMaxRanks, true>(L, tile_off, 0, threadIdx.x).finish();
+        const u32x4 r = L.batch == 1 ? tree_walk<T, OP, kMaxRanks, true>(L, tile_off, 0, threadIdx.x).finish()
+                                     : tree_node<T, OP, true>(ranks, tile_off, threadIdx.x).finish();
         store_tile_of<T>(static_cast<char*>(L.out) + tile_off, threadIdx.x, r, L.keep != 0);
     } else if (lane < nvec) {
-        store_vec(static_cast<char*>(L.out) + lane * kVecBytes, tree_vector<T, OP>(L, lane * kVecBytes));
+        store_vec(static_cast<char*>(L.out) + lane * kVecBytes, tree_vector<T, OP>(ranks, lane * kVecBytes));
     }
     // the elements behind the last whole vector: the first lanes of the last workgroup
     if (blockIdx.x == gridDim.x - 1 && threadIdx.x < L.count % EPV) {
@@ -927,8 +1012,9 @@ __device__ __forceinline__ void tree_tile(const TreeLaunch& L) {
 
 template <typename T, int OP>
 __global__ void __launch_bounds__(kThreads) fold_tree_kernel(const TreeLaunch L) {
+    const TreeRanks ranks = load_tree_ranks(L, threadIdx.x);  // issued first
     if (!hook_enter(L.hooks, L.hook_target)) return;
-    tree_tile<T, OP>(L);
+    tree_tile<T, OP>(L, ranks);
     if (L.hook_ticket) hook_publish(L.hooks, L.hook_ticket);
 }
 

@@ -230,19 +230,38 @@ constexpr uint32_t flat_one_out_waves_per_cu(uint32_t nranks, uint64_t tiles_per
            : nranks == 4 ? (elem_size >= 4 ? 14u : 12u)
                          : 0u;
 }
-// The tree kernel (reduce towards a root for rank counts the flat kernels do not have) walks its tree depth first with
-// a few loads in flight per wavefront, and likes 16 wavefronts per CU for elements of 4 and 8 bytes once its launches are
-// long (fp32 at 256 MiB per buffer: 5 / 7 / 12 / 16 ranks 80 / 81 / 79 / 78 -> 85 / 87 / 84 / 82 % of the HBM peak, int64 and
-// fp64 79 -> 84 - 85).  How long depends on the number of ranks; all that fit against 16 per CU, fp32, by MiB per buffer:
-//   5 - 7 ranks   16 MiB 83 - 84 against 77 - 80   32 MiB 82 - 84 against 79 - 82   64 MiB 84 - 84.5 against 82 - 86   128 MiB 84 - 86 against 87 - 89
-//   9 - 11 ranks  16 MiB 81.9 - 82.7 against 81.1 - 83.5   32 MiB 80.8 - 81.3 against 82.9 - 83.5   64 MiB 81.7 - 83.4 against 85.7 - 86.5
-//   12 - 32 ranks  8 MiB 77.5 - 83.8 against 80.6 - 85.0   16 MiB 82.2 - 83.1 against 83.3 - 86.8   32 MiB 80.6 - 81.4 against 84.0 - 85.6
-// (14 and 18 per CU are behind 16 throughout).  Elements of 1 and 2 bytes spend longer on their conversions and lose 10
-// points to any cap.
-constexpr uint32_t tree_cap_min_tiles(uint32_t nranks) {  // tiles of 1 KiB per buffer
-    return nranks >= 12 ? 16384u : nranks >= 9 ? 32768u : 65536u;
+// The tree kernel (reduce towards a root for rank counts the flat kernels do not have) has eight loads of 1 KiB in
+// flight per wavefront, and like the one-output flat folds it wants fewer wavefronts per CU than fit once its launches
+// are long, fewer still where its stores stream past the cache (from 128 MiB written on, kKeepMaxBytes) and the more
+// ranks it folds.  Measured on MI355X, % of the HBM peak, fp32, all that fit / 9 / 10 / 12 / 14 / 16 / 20 wavefronts per CU, by
+// MiB per buffer:
+//    5 ranks   16 MiB 86.2 / 72.5 / 76.0 / 79.8 / 82.6 / 83.5 / 87.1   64 MiB 83.8 / 77.3 / 81.0 / 85.6 / 87.3 / 87.4 / 86.1
+//             128 MiB 86.2 / 79.2 / 82.9 / 87.6 / 89.6 / 90.6 / 88.3   256 MiB 79.0 / 76.3 / 80.2 / 84.8 / 85.5 / 83.4 / 80.6
+//    7 ranks   16 MiB 85.2 / 79.8 / 81.2 / 82.9 / 83.8 / 86.2 / 87.5   64 MiB 82.5 / 83.4 / 85.1 / 87.0 / 87.0 / 87.3 / 86.0
+//             128 MiB 83.1 / 83.8 / 85.5 / 88.2 / 88.6 / 88.2 / 87.2   256 MiB 77.1 / 82.7 / 83.9 / 83.9 / 81.0 / 81.6 / 79.5
+//   12 ranks   16 MiB 84.7 / 78.1 / 80.5 / 82.6 / 83.5 / 86.2 / 85.0   64 MiB 82.0 / 82.2 / 84.1 / 86.1 / 86.1 / 86.4 / 84.9
+//             128 MiB 81.8 / 82.5 / 84.9 / 87.4 / 87.2 / 86.7 / 85.2   256 MiB 76.9 / 80.3 / 82.6 / 84.5 / 82.1 / 81.6 / 80.1
+//   16 ranks   16 MiB 83.9 / 82.1 / 83.6 / 85.4 / 85.6 / 86.6 / 84.6   64 MiB 80.9 / 84.3 / 85.8 / 86.4 / 85.8 / 85.4 / 83.3
+//             128 MiB 78.9 / 83.2 / 85.0 / 85.6 / 84.8 / 83.6 / 80.9   256 MiB 76.0 / 83.5 / 84.7 / 82.0 / 80.9 / 80.1 / 78.1
+//   32 ranks   16 MiB 81.9 / 84.5 / 86.1 / 86.3 / 86.1 / 87.6 / 82.7   64 MiB 80.3 / 85.1 / 86.1 / 85.4 / 84.5 / 84.5 / 81.8
+//             128 MiB 80.2 / 84.4 / 85.6 / 85.1 / 84.1 / 83.7 / 81.8   256 MiB 75.7 / 81.8 / 81.9 / 80.8 / 80.1 / 79.8 / 77.6
+// (1 GiB reads like 256 MiB, 8 MiB is best left alone; fp16: 7 ranks x 64 / 256 MiB 82.8 / 77.9 with all that fit, 87.2 at 16 and
+// 84.8 at 12; 16 ranks 80.5 / 76.3, 84.8 and 82.2 at 12 and 10.)
+// Where the stores stream (256 MiB and 1 GiB per buffer) the plain recursive walk at 16 wavefronts per CU (two or three
+// loads per wavefront in flight) is level with the batches at their best occupancy or 1 - 4 points ahead for up to nine
+// ranks of 4- and 8-byte elements (same session: 5 ranks fp32 85.9 / 87.5 against 85.5 / 85.5 at 14 / 12, 7 ranks 85.7 / 85.7
+// against 83.9 / 81.3 at 12 / 10, 9 ranks 84.7 / 84.2 against 83.6 / 81.2), behind from twelve ranks on (82.6 / 81.8 against
+// 84.2 / 81.3 at 12 / 10, 16 ranks 82.3 / 81.1 against 83.6 / 82.3 at 10) and for fp16 and uint8, which it serves at full
+// occupancy only (5 ranks 81.0 / 81.2 against 84.9 / 85.6 at 14, 7 ranks 79.9 / 79.4 against 84.8 / 81.8 at 12, 16 ranks
+// 78.4 / 77.9 against 82.6 / 80.8 at 10).
+constexpr uint32_t tree_batch(uint32_t nranks, uint32_t elem_size, bool keep) {  // TreeLaunch::batch
+    return !keep && elem_size >= 4 && nranks <= 9 ? 1u : 8u;
 }
-constexpr uint32_t kTreeCapWavesPerCu = 16;
+constexpr uint32_t tree_waves_per_cu(uint32_t nranks, uint64_t tiles_per_buffer, bool keep, uint32_t elem_size) {  // 0: all that fit
+    if (!keep) return tree_batch(nranks, elem_size, keep) == 1 ? 16u : nranks <= 6 ? 14u : nranks <= 12 ? 12u : 10u;
+    if (tiles_per_buffer >= 32768) return nranks <= 8 ? 16u : nranks <= 12 ? 14u : nranks <= 24 ? 12u : 10u;
+    return tiles_per_buffer >= 16384 && nranks >= 12 ? 16u : 0u;
+}
 // The group form of the flat fold behaves the same way once its launches are long: with all of a wavefront's accesses
 // issued at once (launches that do not pace them, kFlatPaced) fewer workgroups per CU than its LDS allows serve the
 // all_reduce shapes better.  Measured on MI355X, fp32 all_reduce, % of the HBM peak, interleaved in one process, as
@@ -285,7 +304,7 @@ struct TreeLaunch {
     uint32_t vector;       // 1: a lane takes a 16-byte vector (the last workgroup also the odd elements at the end);
                            // 0: a lane takes one element
     uint32_t keep;         // 1: the stores leave their data in the last-level cache
-    uint32_t reserved;
+    uint32_t batch;        // leaves per batch of the tree walk: 8, or 1 (tree_batch)
     EdgeHooks hooks;
     uint64_t hook_target;
     uint64_t hook_ticket;
