@@ -792,7 +792,7 @@ void set_store_policy(Plan& plan) {
             case Step::kFlat: step.flat.exchange = keep ? step.flat.exchange | kFlatKeep : step.flat.exchange & ~kFlatKeep; break;
             case Step::kTree:
                 step.tree.keep = keep ? 1 : 0;
-                step.tree.batch = tree_batch(step.tree.nranks, step.tree.elem_size, keep);
+                step.tree.batch = tree_batch(step.tree.nranks, step.tree.elem_size, keep, step.tree.total_tiles);
                 break;
             case Step::kPack: step.pack.keep = keep ? 1 : 0; break;
         }
@@ -926,7 +926,7 @@ Status plan_reduce(Plan& plan, const void* const* send, void* recv_root, uint32_
         const uint64_t tiles = (lanes + kThreads - 1) / kThreads;
         if (tiles > 0x7fffffffull) return invalid("buffer too large for one tree launch");
         L.total_tiles = uint32_t(tiles);
-        L.batch = tree_batch(nranks, elem_size, true);  // set_store_policy() has the last word
+        L.batch = tree_batch(nranks, elem_size, true, L.total_tiles);  // set_store_policy() has the last word
         plan.steps.push_back(step);
         return MEGRAY_OK;
     }

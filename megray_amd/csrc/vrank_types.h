@@ -254,11 +254,15 @@ constexpr uint32_t flat_one_out_waves_per_cu(uint32_t nranks, uint64_t tiles_per
 // 84.2 / 81.3 at 12 / 10, 16 ranks 82.3 / 81.1 against 83.6 / 82.3 at 10) and for fp16 and uint8, which it serves at full
 // occupancy only (5 ranks 81.0 / 81.2 against 84.9 / 85.6 at 14, 7 ranks 79.9 / 79.4 against 84.8 / 81.8 at 12, 16 ranks
 // 78.4 / 77.9 against 82.6 / 80.8 at 10).
-constexpr uint32_t tree_batch(uint32_t nranks, uint32_t elem_size, bool keep) {  // TreeLaunch::batch
-    return !keep && elem_size >= 4 && nranks <= 9 ? 1u : 8u;
+// It is also ahead between 2 and 8 MiB per buffer from twelve ranks on, whatever the element type (same-process A/B, fp32,
+// microseconds, walk / batches: 12 ranks x 2 MiB 4.10 / 4.15, 4 MiB 8.38 / 9.09, 6 MiB 12.3 / 13.4, 7 MiB 16.5 / 15.7, 8 MiB 17.0 / 16.0; 32 ranks x
+// 1.5 MiB 13.0 / 8.4, 2 MiB 14.1 / 11.3, 4 MiB 20.9 / 24.1, 6 MiB 30.5 / 33.7, 7 MiB 37.6 / 41.0, 8 MiB 41.5 / 42.2).
+constexpr uint32_t tree_batch(uint32_t nranks, uint32_t elem_size, bool keep, uint64_t tiles_per_buffer) {  // TreeLaunch::batch
+    if (!keep) return elem_size >= 4 && nranks <= 9 ? 1u : 8u;
+    return nranks >= 12 && tiles_per_buffer > 2048 && tiles_per_buffer < 8192 ? 1u : 8u;
 }
 constexpr uint32_t tree_waves_per_cu(uint32_t nranks, uint64_t tiles_per_buffer, bool keep, uint32_t elem_size) {  // 0: all that fit
-    if (!keep) return tree_batch(nranks, elem_size, keep) == 1 ? 16u : nranks <= 6 ? 14u : nranks <= 12 ? 12u : 10u;
+    if (!keep) return tree_batch(nranks, elem_size, keep, tiles_per_buffer) == 1 ? 16u : nranks <= 6 ? 14u : nranks <= 12 ? 12u : 10u;
     if (tiles_per_buffer >= 32768) return nranks <= 8 ? 16u : nranks <= 12 ? 14u : nranks <= 24 ? 12u : 10u;
     return tiles_per_buffer >= 16384 && nranks >= 12 ? 16u : 0u;
 }
