@@ -271,6 +271,34 @@ def tree_expectation(ins, dtype, op, root):
         return a[0].astype(np.float16)
 
 
+@pytest.mark.parametrize("dtype", [orc.FLOAT32, orc.FLOAT16, orc.UINT8, orc.INT64])
+def test_tree_reduce_for_every_batch_shape(dtype, monkeypatch):
+    """reduce towards a root in the reference's binomial-tree order (src/ucx/reduce.cpp:56-80) for rank counts without a
+    flat kernel.  The kernel takes the tree eight leaves at a time - whole and partial batches, one to four of them -
+    or walks it leaf by leaf (twelve and more ranks between 2 and 8 MiB per buffer; up to nine ranks of 4- and 8-byte
+    elements where the stores stream, forced here through the store policy): every rank count's tree against the
+    oracle's literal replay, ragged lengths, every root position class."""
+    size = orc.dtype_size(dtype)
+    rng = np.random.default_rng(4100 + dtype)
+    for nranks in (5, 6, 7, 9, 10, 11, 13, 15, 16, 17, 23, 25, 31):
+        for policy, length in (("", 70001), ("never", 33003), ("", (3000 * 1024) // size + 5 if nranks in (13, 25) else 0)):
+            if not length:
+                continue
+            if policy:
+                monkeypatch.setenv("MEGRAY_VRANK_KEEP", policy)
+            else:
+                monkeypatch.delenv("MEGRAY_VRANK_KEEP", raising=False)
+            ins = [rand_array(dtype, length, rng) for _ in range(nranks)]
+            d_in = [to_device(x) for x in ins]
+            for op, root in ((orc.SUM, nranks - 1), (orc.MAX, nranks // 2)):
+                out = empty_device(length * size)
+                mr.reduce_to_root(d_in, out, length, dtype, op, root)
+                torch.cuda.synchronize()
+                assert_same(to_host(out, ins[0].dtype), tree_expectation(ins, dtype, op, root),
+                            f"tree reduce dtype={dtype} N={nranks} len={length} policy={policy!r} op={op} root={root}")
+    monkeypatch.delenv("MEGRAY_VRANK_KEEP", raising=False)
+
+
 @pytest.mark.parametrize("dtype", [orc.FLOAT32, orc.FLOAT16, orc.INT8, orc.INT64])
 def test_large_folds_into_one_output_at_reduced_occupancy(dtype):
     """reduce_scatter, reduce towards a root and the two-phase all_reduce from 8192 tiles per buffer on (four ranks:
